@@ -1,0 +1,62 @@
+"""Builds libflash_moba_hip.so (the C-ABI kernel library) for gfx950 with hipcc.
+
+    python flash-moba_amd/build.py            # build into flash-moba_amd/lib/
+
+hipcc cross-compiles for gfx950 without a GPU.  The library is built in-tree so that it
+travels with the source tree; nothing is installed into site-packages.
+"""
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+LIB = os.path.join(LIBDIR, "libflash_moba_hip.so")
+SOURCES = ["fmoba_host.hip", "mean_pool.hip", "topk_csc.hip", "varlen_sort.hip", "attn_fwd.hip", "attn_bwd.hip"]
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
+    # keep packed-fp32 VALU ops out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", shutil.which("hipcc")):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (looked at $HIPCC, /opt/rocm/bin/hipcc and PATH)")
+
+
+def _compile(src: str, objdir: str) -> str:
+    obj = os.path.join(objdir, src.replace(".hip", ".o"))
+    cmd = [hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+    return obj
+
+
+def build_library(verbose: bool = True, jobs: int = 6) -> str:
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    os.makedirs(LIBDIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(lambda s: _compile(s, objdir), SOURCES))
+    tmp = LIB + ".tmp"
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
+    os.replace(tmp, LIB)
+    if verbose:
+        print("built", LIB, os.path.getsize(LIB), "bytes")
+    return LIB
+
+
+if __name__ == "__main__":
+    build_library()
+    sys.exit(0)

@@ -1,0 +1,192 @@
+// Shared device helpers for the gfx950 FlashMoBA kernels: element types, MFMA wrappers,
+// transposing LDS reads, wave-level utilities and the host-side error plumbing.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/flash_moba_hip.h"
+
+namespace fmoba {
+
+// ------------------------------------------------------------------------------------
+// host-side error handling
+// ------------------------------------------------------------------------------------
+void set_error(const char *fmt, ...);
+#define FMOBA_REQUIRE(cond, ...)          \
+  do {                                    \
+    if (!(cond)) {                        \
+      ::fmoba::set_error(__VA_ARGS__);    \
+      return 1;                           \
+    }                                     \
+  } while (0)
+#define FMOBA_LAUNCH_CHECK(what)                                                     \
+  do {                                                                               \
+    hipError_t e__ = hipGetLastError();                                              \
+    if (e__ != hipSuccess) {                                                         \
+      ::fmoba::set_error("%s: launch failed: %s", what, hipGetErrorString(e__));     \
+      return 2;                                                                      \
+    }                                                                                \
+  } while (0)
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ------------------------------------------------------------------------------------
+// element types
+// ------------------------------------------------------------------------------------
+typedef _Float16 f16_t;
+typedef __bf16 bf16_t;
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <typename T> struct ElemTraits;
+template <> struct ElemTraits<f16_t> {
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ float to_float(f16_t x) { return (float)x; }
+  static __device__ __forceinline__ f16_t from_float(float x) { return (f16_t)x; }
+};
+template <> struct ElemTraits<bf16_t> {
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ float to_float(bf16_t x) { return (float)x; }
+  static __device__ __forceinline__ bf16_t from_float(float x) { return (bf16_t)x; }
+};
+
+// 16 bytes = 8 elements, the unit every kernel moves.
+struct alignas(16) Pack8 {
+  uint32_t w[4];
+};
+
+template <typename T>
+__device__ __forceinline__ float elem_to_float(uint16_t bits) {
+  T x;
+  __builtin_memcpy(&x, &bits, 2);
+  return ElemTraits<T>::to_float(x);
+}
+template <typename T>
+__device__ __forceinline__ uint16_t float_to_elem_bits(float f) {
+  T x = ElemTraits<T>::from_float(f);
+  uint16_t b;
+  __builtin_memcpy(&b, &x, 2);
+  return b;
+}
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return (uint32_t)float_to_elem_bits<T>(lo) | ((uint32_t)float_to_elem_bits<T>(hi) << 16);
+}
+template <typename T>
+__device__ __forceinline__ void unpack8(const Pack8 &p, float (&f)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = elem_to_float<T>((uint16_t)(p.w[i] & 0xffffu));
+    f[2 * i + 1] = elem_to_float<T>((uint16_t)(p.w[i] >> 16));
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// MFMA 32x32x16 (gfx950).  Operand layout, lane l, hh = l / 32:
+//   A (32 x 16): lane holds A[l % 32][hh*8 .. hh*8+7]
+//   B (16 x 32): lane holds B[hh*8 .. hh*8+7][l % 32]
+//   C (32 x 32): lane holds C[8*(i/4) + 4*hh + i%4][l % 32], i = 0..15
+// ------------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ f32x16 mfma32(const Pack8 &a, const Pack8 &b, f32x16 c);
+template <>
+__device__ __forceinline__ f32x16 mfma32<bf16_t>(const Pack8 &a, const Pack8 &b, f32x16 c) {
+  bf16x8 av, bv;
+  __builtin_memcpy(&av, &a, 16);
+  __builtin_memcpy(&bv, &b, 16);
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x16 mfma32<f16_t>(const Pack8 &a, const Pack8 &b, f32x16 c) {
+  f16x8 av, bv;
+  __builtin_memcpy(&av, &a, 16);
+  __builtin_memcpy(&bv, &b, 16);
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c, 0, 0, 0);
+}
+
+// Row of a 32x32 accumulator tile that register i of this lane holds.
+__device__ __forceinline__ int acc_row(int i, int hh) { return 8 * (i >> 2) + 4 * hh + (i & 3); }
+
+// When accumulator registers 8s..8s+7 (s = 0,1) of a 32x32 tile are packed and fed back
+// as the k-operand of the next MFMA, contraction index kappa = hh*8 + v (v = 0..7) of
+// k-step s refers to accumulator row 16*s + 8*(v/4) + 4*hh + v%4.
+__device__ __forceinline__ int ktile_row(int s, int hh, int v) { return 16 * s + 8 * (v >> 2) + 4 * hh + (v & 3); }
+
+// ------------------------------------------------------------------------------------
+// Transposing LDS read (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane i
+// receives element (i % 4) of the 8-byte blocks whose addresses were supplied by lanes
+// i/4, i/4 + 4, i/4 + 8, i/4 + 12 of the same group.
+//
+// tr_frag8 builds the 8-element k-operand of a 32x32x16 MFMA for a matrix X stored
+// row-major in LDS ([k][n], row stride `ld` elements) such that this lane ends up with
+//   X[row(v)][col0 + l % 32],  v = 0..7,
+// where row(v) = rows4_lo + v for v < 4 and rows4_hi + (v - 4) for v >= 4 are the rows
+// THIS lane's half (hh) needs.  Address supplied by lane l (i = l % 16):
+//   &X[rows4_xx + i / 4][col0 + 16 * ((l % 32) / 16) + 4 * (i % 4)].
+// ------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+__device__ __forceinline__ s16x4 ds_read_tr16(const void *lds_generic_ptr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  // generic -> LDS address space: the low 32 bits of a generic LDS pointer are the LDS offset
+  lds_s16x4 *p = (lds_s16x4 *)(uint32_t)(uintptr_t)lds_generic_ptr;
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(p);
+#else
+  (void)lds_generic_ptr;
+  return s16x4{0, 0, 0, 0};
+#endif
+}
+__device__ __forceinline__ Pack8 tr_frag8(const uint16_t *X, int ld, int rows4_lo, int rows4_hi, int col0, int lane) {
+  const int i = lane & 15;
+  const int c = col0 + ((lane & 31) >> 4) * 16 + (i & 3) * 4;
+  const int j = i >> 2;
+  s16x4 lo = ds_read_tr16(X + (rows4_lo + j) * ld + c);
+  s16x4 hi = ds_read_tr16(X + (rows4_hi + j) * ld + c);
+  Pack8 r;
+  __builtin_memcpy(&r.w[0], &lo, 8);
+  __builtin_memcpy(&r.w[2], &hi, 8);
+  return r;
+}
+
+// ------------------------------------------------------------------------------------
+// wave utilities
+// ------------------------------------------------------------------------------------
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+
+// Orders LDS traffic of ONE wave (writes by some lanes, reads by others).
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__device__ __forceinline__ float shfl_xor32_f(float v) { return __shfl_xor(v, 32, 64); }
+__device__ __forceinline__ int shfl_xor32_i(int v) { return __shfl_xor(v, 32, 64); }
+
+// Monotone map float -> uint32 (larger float => larger key); every non-NaN value,
+// including -inf, maps to a key >= 0x007fffff > 0.
+__device__ __forceinline__ uint32_t float_order_key(float f) {
+  uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float order_key_float(uint32_t k) {
+  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __uint_as_float(u);
+}
+
+__device__ __forceinline__ Pack8 ld_global16(const void *p) { return *reinterpret_cast<const Pack8 *>(p); }
+__device__ __forceinline__ Pack8 zero_pack8() {
+  Pack8 r;
+  r.w[0] = r.w[1] = r.w[2] = r.w[3] = 0u;
+  return r;
+}
+
+}  // namespace fmoba

@@ -1,0 +1,511 @@
+// Fused top-k block gating and deterministic CSC build.
+//
+//   topk_gate_kernel : scores S^T = KM * Q^T on MFMA, per-row exact top-k by bisection on
+//                      order-preserving keys held in registers (no score matrix, no sorted
+//                      list and no per-row index list ever reaches HBM); emits one selection
+//                      BIT per (row, chunk) and per-(2048-row segment, chunk) counts.
+//   csc_scan_kernel  : per (sequence, head) scan of the counts -> col_nnz, col_offsets
+//                      (int64) and per-segment start offsets; clears the unused tail of
+//                      the row-list buffer.
+//   csc_fill_kernel  : walks the bit columns in row order and writes each chunk's row list
+//                      ascending, so no sort pass is needed afterwards.
+#include "fmoba_common.h"
+
+namespace fmoba {
+
+constexpr int kGateRows = 128;   // query rows per workgroup (4 waves x 32)
+constexpr int kSegRows = 2048;   // rows per counting segment
+
+struct TopkParams {
+  fmoba_fused_topk_args a;
+  uint32_t *sel;      // [heads][W][total_q] selection bits, word w covers chunks 32w..32w+31
+  int32_t *segcnt;    // [batch][heads][nseg][max_cols]
+  int32_t W, nseg, max_cols;
+};
+
+template <typename T, int HD, int NT>
+__global__ __launch_bounds__(256) void topk_gate_kernel(TopkParams p) {
+  constexpr int KS = HD / 16;
+  constexpr int LD = HD + 16;  // LDS row stride (elements)
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint16_t *sKm = reinterpret_cast<uint16_t *>(smem);
+  int *sHist = reinterpret_cast<int *>(smem + (size_t)NT * 32 * LD * 2);
+
+  const fmoba_fused_topk_args &a = p.a;
+  const int mb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int q0 = a.cu_seqlens_q[b];
+  const int Lq = a.cu_seqlens_q[b + 1] - q0;
+  const int m0 = mb * kGateRows;
+  if (m0 >= Lq) return;
+  const int Lk = a.cu_seqlens_k[b + 1] - a.cu_seqlens_k[b];
+  const int km0 = a.cu_seqlens_km[b];
+  const int Cb = a.cu_seqlens_km[b + 1] - km0;
+  const int off = Lk - Lq;
+  const int B = a.chunk;
+  const int D = a.head_dim;
+  const int hk = h / (a.heads / a.heads_k);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
+
+  // chunks [0, nsc) can be candidates of some row of this block
+  int nsc;
+  if (a.is_causal) {
+    const int rmax = min(m0 + kGateRows - 1, Lq - 1) + off;
+    nsc = rmax < 0 ? 0 : min(Cb, rmax / B);
+  } else {
+    nsc = Cb;
+  }
+  nsc = min(nsc, min(p.max_cols, NT * 32));  // never beyond the LDS tile, whatever max_seqlen_k the caller gave
+  const int n_tiles = (nsc + 31) >> 5;
+
+  // stage the chunk means of this (sequence, kv head) in LDS, zero padded
+  {
+    const uint16_t *kmp = reinterpret_cast<const uint16_t *>(a.km) + (int64_t)hk * a.km_head_stride;
+    const int vecs = HD / 8;
+    for (int v = tid; v < n_tiles * 32 * vecs; v += 256) {
+      const int c = v / vecs, e = (v - c * vecs) * 8;
+      Pack8 x = zero_pack8();
+      if (c < nsc && e < D) x = ld_global16(kmp + (int64_t)(km0 + c) * a.km_row_stride + e);
+      *reinterpret_cast<Pack8 *>(sKm + c * LD + e) = x;
+    }
+    for (int v = tid; v < NT * 32; v += 256) sHist[v] = 0;
+  }
+
+  // this lane's query row and its operand slices (contraction index permuted so that each
+  // half-wave reads one contiguous half of the row)
+  const int r = m0 + wave * 32 + (lane & 31);
+  const bool valid = r < Lq;
+  Pack8 qf[KS];
+  {
+    const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)(q0 + (valid ? r : 0)) * a.q_row_stride + (int64_t)h * a.q_head_stride;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int e = (hh * KS + ks) * 8;
+      qf[ks] = (valid && e < D) ? ld_global16(qp + e) : zero_pack8();
+    }
+  }
+  __syncthreads();
+
+  // scores: lane (query l%32) gets chunk t*32 + acc_row(i, hh) in register i of tile t
+  uint32_t key[NT][16];
+  const int rp = r + off;
+  int nc;  // number of candidate chunks of this row: chunks strictly before its own chunk
+  if (a.is_causal)
+    nc = (valid && rp >= 0) ? min(rp / B, Cb) : 0;
+  else
+    nc = valid ? Cb : 0;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    if (t < n_tiles) {
+      f32x16 acc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const Pack8 af = *reinterpret_cast<const Pack8 *>(sKm + (t * 32 + (lane & 31)) * LD + (hh * KS + ks) * 8);
+        acc = mfma32<T>(af, qf[ks], acc);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int c = t * 32 + acc_row(i, hh);
+        key[t][i] = (c < nc) ? float_order_key(acc[i]) : 0u;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) key[t][i] = 0u;
+    }
+  }
+
+  // K' = number of scored chunks to keep (the own chunk takes one slot in causal mode)
+  const int kp = a.is_causal ? a.topk - 1 : a.topk;
+  const bool need = (nc > kp) && (kp > 0);
+  uint32_t tau = 1u;    // candidates have key >= 1
+  uint32_t iota = 0u;   // among keys equal to tau keep chunks >= iota
+  if (__any(need)) {
+    uint32_t t_acc = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t trial = t_acc | (1u << bit);
+      int cnt = 0;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) cnt += (key[t][i] >= trial) ? 1 : 0;
+        }
+      cnt += shfl_xor32_i(cnt);
+      if (cnt >= kp) t_acc = trial;
+    }
+    if (need) tau = t_acc;
+    // ties at the threshold: keep the (kp - #greater) highest chunk indices
+    int cgt = 0, ceq = 0;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      if (t < n_tiles) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          cgt += (key[t][i] > tau) ? 1 : 0;
+          ceq += (key[t][i] == tau) ? 1 : 0;
+        }
+      }
+    cgt += shfl_xor32_i(cgt);
+    ceq += shfl_xor32_i(ceq);
+    const int needk = kp - cgt;
+    const bool tie = need && (ceq > needk);
+    if (__any(tie)) {
+      uint32_t i_acc = 0u;
+      constexpr int IB = (NT * 32 <= 64) ? 6 : (NT * 32 <= 128 ? 7 : 8);
+      for (int bit = IB - 1; bit >= 0; --bit) {
+        const uint32_t trial = i_acc | (1u << bit);
+        int cnt = 0;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          if (t < n_tiles) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
+              cnt += (key[t][i] == tau && c >= trial) ? 1 : 0;
+            }
+          }
+        cnt += shfl_xor32_i(cnt);
+        if (cnt >= needk) i_acc = trial;
+      }
+      if (tie) iota = i_acc;
+    }
+  }
+
+  // selection words (32 chunks each), own chunk forced in causal mode
+  const bool has_self = a.is_causal && valid && rp >= 0;
+  const int pself = has_self ? rp / B : -1;
+  const int seg = m0 / kSegRows;
+  uint32_t *selp = p.sel + (int64_t)h * p.W * a.total_q + q0 + r;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    if (t < p.W) {
+      uint32_t w = 0u;
+      if (t < n_tiles && kp > 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
+          const uint32_t k = key[t][i];
+          const bool s = (k > tau) || (k == tau && c >= iota);
+          w |= (s && k != 0u) ? (1u << ((8 * (i >> 2) + (i & 3)) + 4 * hh)) : 0u;
+        }
+      }
+      w |= (uint32_t)shfl_xor32_i((int)w);
+      if (has_self && (pself >> 5) == t) w |= 1u << (pself & 31);
+      if (!valid) w = 0u;
+      if (valid && hh == 0) selp[(int64_t)t * a.total_q] = w;
+      // per-chunk counts of this wave's 32 rows
+      int mycnt = 0;
+      const uint32_t wc = (hh == 0) ? w : 0u;
+      if (__any(wc != 0u)) {
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+          const unsigned long long m = __ballot((wc >> j) & 1u);
+          if (lane == j) mycnt = __popcll(m);
+        }
+        if (lane < 32 && mycnt) atomicAdd(&sHist[t * 32 + lane], mycnt);
+      }
+    }
+  }
+  __syncthreads();
+  for (int c = tid; c < p.W * 32 && c < p.max_cols; c += 256) {
+    const int v = sHist[c];
+    if (v) atomicAdd(&p.segcnt[(((int64_t)b * a.heads + h) * p.nseg + seg) * p.max_cols + c], v);
+  }
+}
+
+// grid (heads, batch), block 256
+__global__ __launch_bounds__(256) void csc_scan_kernel(TopkParams p) {
+  const fmoba_fused_topk_args &a = p.a;
+  const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int q0 = a.cu_seqlens_q[b];
+  const int Lq = a.cu_seqlens_q[b + 1] - q0;
+  const int nseg_b = (Lq + kSegRows - 1) / kSegRows;
+  const int64_t bh = (int64_t)b * a.heads + h;
+  int32_t *segc = p.segcnt + bh * p.nseg * p.max_cols;
+  const int64_t base = ((int64_t)q0 * a.heads + (int64_t)Lq * h) * a.topk;
+  __shared__ int sscan[256];
+  __shared__ int64_t stotal;
+  if (tid == 0) stotal = 0;
+  __syncthreads();
+  for (int c0 = 0; c0 < p.max_cols; c0 += 256) {
+    const int c = c0 + tid;
+    int nnz = 0;
+    if (c < p.max_cols) {
+      for (int s = 0; s < nseg_b; ++s) {
+        const int v = segc[(int64_t)s * p.max_cols + c];
+        segc[(int64_t)s * p.max_cols + c] = nnz;
+        nnz += v;
+      }
+    }
+    sscan[tid] = nnz;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+      const int v = (tid >= d) ? sscan[tid - d] : 0;
+      __syncthreads();
+      sscan[tid] += v;
+      __syncthreads();
+    }
+    const int64_t run = stotal;
+    if (c < p.max_cols) {
+      a.col_nnz[bh * p.max_cols + c] = nnz;
+      a.col_offsets[bh * p.max_cols + c] = base + run + (int64_t)(sscan[tid] - nnz);
+    }
+    __syncthreads();
+    if (tid == 255) stotal = run + sscan[255];
+    __syncthreads();
+  }
+  // slots of this (sequence, head) region that no list uses stay 0
+  const int64_t start = base + stotal, end = base + (int64_t)Lq * a.topk;
+  for (int64_t i = start + tid; i < end; i += 256) a.flat_indices[i] = 0;
+}
+
+// grid (nseg * W, heads, batch), block 64: one wave walks 2048 rows of one 32-chunk word column
+__global__ __launch_bounds__(64) void csc_fill_kernel(TopkParams p) {
+  const fmoba_fused_topk_args &a = p.a;
+  const int seg = blockIdx.x / p.W, wc = blockIdx.x - seg * p.W;
+  const int h = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+  const int q0 = a.cu_seqlens_q[b];
+  const int Lq = a.cu_seqlens_q[b + 1] - q0;
+  const int r0 = seg * kSegRows;
+  if (r0 >= Lq) return;
+  const int r1 = min(Lq, r0 + kSegRows);
+  const int64_t bh = (int64_t)b * a.heads + h;
+  int64_t pos = 0;
+  {
+    const int c = wc * 32 + lane;
+    if (lane < 32 && c < p.max_cols)
+      pos = a.col_offsets[bh * p.max_cols + c] + p.segcnt[(bh * p.nseg + seg) * p.max_cols + c];
+  }
+  const uint32_t *words = p.sel + ((int64_t)h * p.W + wc) * a.total_q + q0;
+  const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int rb = r0; rb < r1; rb += 64) {
+    const int r = rb + lane;
+    const uint32_t w = (r < r1) ? words[r] : 0u;
+    if (!__any(w != 0u)) continue;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      const bool bit = (w >> j) & 1u;
+      const unsigned long long m = __ballot(bit);
+      if (m) {
+        const uint32_t lo = __builtin_amdgcn_readlane((uint32_t)pos, j);
+        const uint32_t hi = __builtin_amdgcn_readlane((uint32_t)((uint64_t)pos >> 32), j);
+        const int64_t bj = (int64_t)(((uint64_t)hi << 32) | lo);
+        if (bit) a.flat_indices[bj + __popcll(m & lt)] = r;
+        if (lane == j) pos += __popcll(m);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// ordered per-row lists (indices / values), only produced on request: one wave per
+// (row, head); plain FMA scores, then topk rounds of wave-wide arg-max under the total
+// order (score desc, chunk desc).
+// ------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(64) void topk_raw_kernel(fmoba_fused_topk_args a, int kr) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  float *sScore = reinterpret_cast<float *>(smem);  // [Cpad]
+  const int row_g = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  // locate the sequence of this row
+  int b = 0;
+  while (b + 1 < a.batch && a.cu_seqlens_q[b + 1] <= row_g) ++b;
+  const int q0 = a.cu_seqlens_q[b];
+  const int Lq = a.cu_seqlens_q[b + 1] - q0;
+  const int r = row_g - q0;
+  int32_t *oi = a.raw_indices + ((int64_t)row_g * a.heads + h) * kr;
+  float *ov = a.raw_values + ((int64_t)row_g * a.heads + h) * kr;
+  for (int s = lane; s < kr; s += 64) {
+    oi[s] = -1;
+    ov[s] = -INFINITY;
+  }
+  if (r < 0 || r >= Lq) return;
+  const int Lk = a.cu_seqlens_k[b + 1] - a.cu_seqlens_k[b];
+  const int km0 = a.cu_seqlens_km[b];
+  const int Cb = a.cu_seqlens_km[b + 1] - km0;
+  const int rp = r + Lk - Lq;
+  const int hk = h / (a.heads / a.heads_k);
+  int nc = a.is_causal ? (rp >= 0 ? min(rp / a.chunk, Cb) : 0) : Cb;
+  const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)row_g * a.q_row_stride + (int64_t)h * a.q_head_stride;
+  const uint16_t *kmp = reinterpret_cast<const uint16_t *>(a.km) + (int64_t)hk * a.km_head_stride;
+  for (int c = lane; c < nc; c += 64) {
+    float s = 0.f;
+    const uint16_t *kr_ = kmp + (int64_t)(km0 + c) * a.km_row_stride;
+    for (int d = 0; d < a.head_dim; ++d) s = fmaf(elem_to_float<T>(qp[d]), elem_to_float<T>(kr_[d]), s);
+    sScore[c] = s;
+  }
+  __syncthreads();
+  int slot = 0;
+  if (a.is_causal && rp >= 0) {
+    if (lane == 0) {
+      oi[0] = rp / a.chunk;
+      ov[0] = INFINITY;
+    }
+    slot = 1;
+  }
+  // previous winner (score key, chunk) bounds the next search from above
+  uint32_t pk = 0xffffffffu;
+  int pc = 0x7fffffff;
+  for (; slot < a.topk; ++slot) {
+    uint32_t bk = 0u;
+    int bc = -1;
+    for (int c = lane; c < nc; c += 64) {
+      const float s = sScore[c];
+      if (s == -INFINITY) continue;  // never inserted by a strict '>' against -inf
+      const uint32_t k = float_order_key(s);
+      const bool below_prev = (k < pk) || (k == pk && c < pc);
+      const bool better = (k > bk) || (k == bk && c > bc);
+      if (below_prev && better) {
+        bk = k;
+        bc = c;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const uint32_t ok = (uint32_t)__shfl_xor((int)bk, o, 64);
+      const int oc = __shfl_xor(bc, o, 64);
+      if (ok > bk || (ok == bk && oc > bc)) {
+        bk = ok;
+        bc = oc;
+      }
+    }
+    if (bc < 0) break;
+    if (lane == 0) {
+      oi[slot] = bc;
+      ov[slot] = sScore[bc];
+    }
+    pk = bk;
+    pc = bc;
+  }
+}
+
+__global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+}  // namespace fmoba
+
+extern "C" size_t fmoba_fused_topk_workspace_bytes(int32_t batch, int32_t total_q, int32_t heads, int32_t max_seqlen_q,
+                                                   int32_t max_seqlen_k, int32_t chunk) {
+  using namespace fmoba;
+  if (batch <= 0 || heads <= 0 || chunk <= 0 || total_q < 0) return 0;
+  const int64_t max_cols = ceil_div64(max_seqlen_k, chunk);
+  const int64_t W = ceil_div64(max_cols, 32);
+  const int64_t nseg = ceil_div64(max_seqlen_q > 0 ? max_seqlen_q : 1, kSegRows);
+  return align256((size_t)heads * W * total_q * 4) + align256((size_t)batch * heads * nseg * max_cols * 4) + 256;
+}
+
+namespace fmoba {
+template <typename T, int HD, int NT>
+static int launch_gate(const TopkParams &p, dim3 grid, hipStream_t s) {
+  const size_t smem = (size_t)NT * 32 * (HD + 16) * 2 + (size_t)NT * 32 * 4;
+  auto kern = topk_gate_kernel<T, HD, NT>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+    set_error("fused_topk: cannot reserve %zu bytes of LDS", smem);
+    return 2;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), smem, s, p);
+  return 0;
+}
+template <typename T, int HD>
+static int launch_gate_nt(const TopkParams &p, dim3 grid, hipStream_t s) {
+  if (p.W <= 2) return launch_gate<T, HD, 2>(p, grid, s);
+  if (p.W <= 4) return launch_gate<T, HD, 4>(p, grid, s);
+  return launch_gate<T, HD, 8>(p, grid, s);
+}
+template <typename T>
+static int launch_gate_hd(const TopkParams &p, dim3 grid, hipStream_t s) {
+  if (p.a.head_dim <= 64) return launch_gate_nt<T, 64>(p, grid, s);
+  if (p.a.head_dim <= 128) return launch_gate_nt<T, 128>(p, grid, s);
+  return launch_gate_nt<T, 256>(p, grid, s);
+}
+}  // namespace fmoba
+
+extern "C" int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream) {
+  using namespace fmoba;
+  FMOBA_REQUIRE(a != nullptr, "fused_topk: null args");
+  FMOBA_REQUIRE(a->dtype == FMOBA_DTYPE_F16 || a->dtype == FMOBA_DTYPE_BF16, "FlashMoBA only supports fp16 and bf16 data types");
+  FMOBA_REQUIRE(a->topk >= 1 && a->topk <= 64, "moba_topk must be in [1, 64]");
+  FMOBA_REQUIRE(a->batch > 0, "batch size must be positive");
+  FMOBA_REQUIRE(a->head_dim > 0 && a->head_dim <= 256, "head_size must be <= 256");
+  FMOBA_REQUIRE(a->head_dim % 8 == 0, "head_size must be multiple of 8");
+  FMOBA_REQUIRE(a->heads > 0 && a->heads_k > 0 && a->heads % a->heads_k == 0, "#heads in key/value must divide #heads in query");
+  FMOBA_REQUIRE(a->chunk > 0, "moba_chunk_size must be positive");
+  FMOBA_REQUIRE(a->total_q >= 0 && a->max_seqlen_q >= 0 && a->max_seqlen_k >= 0, "negative size");
+  FMOBA_REQUIRE(a->cu_seqlens_q && a->cu_seqlens_k && a->cu_seqlens_km, "fused_topk: null cu_seqlens pointer");
+  FMOBA_REQUIRE(a->col_offsets && a->col_nnz && (a->flat_indices || (int64_t)a->total_q * a->heads * a->topk == 0),
+                "fused_topk: null output pointer");
+  FMOBA_REQUIRE((a->raw_indices == nullptr) == (a->raw_values == nullptr), "fused_topk: raw_indices and raw_values go together");
+  hipStream_t s = (hipStream_t)stream;
+  const int max_cols = ceil_div(a->max_seqlen_k, a->chunk);
+  const int64_t nslots = (int64_t)a->total_q * a->heads * a->topk;
+  const int kr = (a->topk + 15) / 16 * 16;
+
+  if (max_cols == 0 || a->max_seqlen_k == 0) {
+    // no keys: lists stay empty; the reference fills the row list with -1 here
+    // (csrc/flash_topk/flash_topk_api.cpp:250-255)
+    if (nslots) hipLaunchKernelGGL(fill_i32_kernel, dim3(1024), dim3(256), 0, s, a->flat_indices, nslots, -1);
+    if (a->raw_indices && a->total_q) {
+      hipLaunchKernelGGL(fill_i32_kernel, dim3(1024), dim3(256), 0, s, a->raw_indices, (int64_t)a->total_q * a->heads * kr, -1);
+      hipLaunchKernelGGL(fill_i32_kernel, dim3(1024), dim3(256), 0, s, reinterpret_cast<int32_t *>(a->raw_values),
+                         (int64_t)a->total_q * a->heads * kr, (int32_t)0xff800000);
+    }
+    FMOBA_LAUNCH_CHECK("fused_topk(empty)");
+    return 0;
+  }
+  FMOBA_REQUIRE(max_cols <= 256,
+                "fused_topk: at most 256 key chunks per sequence are supported by this build (got %d = ceil(%d / %d))",
+                max_cols, a->max_seqlen_k, a->chunk);
+  FMOBA_REQUIRE(a->q && a->km, "fused_topk: null q/km pointer");
+  FMOBA_REQUIRE(a->q_row_stride % 8 == 0 && a->q_head_stride % 8 == 0 && a->km_row_stride % 8 == 0 && a->km_head_stride % 8 == 0,
+                "fused_topk: strides must be multiples of 8 elements");
+  FMOBA_REQUIRE(((uintptr_t)a->q % 16) == 0 && ((uintptr_t)a->km % 16) == 0, "fused_topk: q and km must be 16-byte aligned");
+  FMOBA_REQUIRE(a->batch <= 65535 && a->heads <= 65535, "fused_topk: batch/heads too large for the launch grid");
+
+  TopkParams p;
+  p.a = *a;
+  p.max_cols = max_cols;
+  p.W = ceil_div(max_cols, 32);
+  p.nseg = ceil_div(a->max_seqlen_q > 0 ? a->max_seqlen_q : 1, kSegRows);
+  const size_t sel_bytes = align256((size_t)a->heads * p.W * a->total_q * 4);
+  const size_t seg_bytes = align256((size_t)a->batch * a->heads * p.nseg * max_cols * 4);
+  FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= sel_bytes + seg_bytes, "fused_topk: workspace too small (%zu < %zu)",
+                a->workspace_bytes, sel_bytes + seg_bytes);
+  uintptr_t wsp = ((uintptr_t)a->workspace + 255) & ~(uintptr_t)255;
+  FMOBA_REQUIRE(wsp + sel_bytes + seg_bytes <= (uintptr_t)a->workspace + a->workspace_bytes, "fused_topk: workspace too small after alignment");
+  p.sel = reinterpret_cast<uint32_t *>(wsp);
+  p.segcnt = reinterpret_cast<int32_t *>(wsp + sel_bytes);
+
+  if (a->total_q == 0 || a->max_seqlen_q == 0) {
+    // no query rows: every column is empty, offsets are the (constant) region bases
+    const int64_t n = (int64_t)a->batch * a->heads * max_cols;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(256), dim3(256), 0, s, p.segcnt, (int64_t)(seg_bytes / 4), 0);
+    hipLaunchKernelGGL(csc_scan_kernel, dim3(a->heads, a->batch), dim3(256), 0, s, p);
+    (void)n;
+    FMOBA_LAUNCH_CHECK("fused_topk(no rows)");
+    return 0;
+  }
+
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(512), dim3(256), 0, s, p.segcnt, (int64_t)(seg_bytes / 4), 0);
+  dim3 ggrid(ceil_div(a->max_seqlen_q, kGateRows), a->heads, a->batch);
+  int rc = (a->dtype == FMOBA_DTYPE_BF16) ? launch_gate_hd<bf16_t>(p, ggrid, s) : launch_gate_hd<f16_t>(p, ggrid, s);
+  if (rc) return rc;
+  FMOBA_LAUNCH_CHECK("topk_gate_kernel");
+  hipLaunchKernelGGL(csc_scan_kernel, dim3(a->heads, a->batch), dim3(256), 0, s, p);
+  FMOBA_LAUNCH_CHECK("csc_scan_kernel");
+  hipLaunchKernelGGL(csc_fill_kernel, dim3(p.nseg * p.W, a->heads, a->batch), dim3(64), 0, s, p);
+  FMOBA_LAUNCH_CHECK("csc_fill_kernel");
+  if (a->raw_indices) {
+    const size_t smem = (size_t)(max_cols + 64) * 4;
+    dim3 rgrid(a->total_q, a->heads);
+    if (a->dtype == FMOBA_DTYPE_BF16)
+      hipLaunchKernelGGL(topk_raw_kernel<bf16_t>, rgrid, dim3(64), smem, s, *a, kr);
+    else
+      hipLaunchKernelGGL(topk_raw_kernel<f16_t>, rgrid, dim3(64), smem, s, *a, kr);
+    FMOBA_LAUNCH_CHECK("topk_raw_kernel");
+  }
+  return 0;
+}

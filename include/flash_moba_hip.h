@@ -1,0 +1,167 @@
+/*
+ * flash_moba_hip.h -- C ABI of the MI355X (gfx950) FlashMoBA kernels.
+ *
+ * One shared library, libflash_moba_hip.so, exports exactly the entry points declared
+ * here.  Every pointer is a DEVICE pointer owned by the caller unless stated otherwise;
+ * strides are in ELEMENTS; `stream` is a hipStream_t passed as void*.  No entry point
+ * allocates, frees or synchronises: scratch memory comes in through `workspace`
+ * arguments whose size the matching *_workspace_bytes() query returns.  All launches go
+ * to `stream`.  Return value: 0 on success, non-zero on error (then fmoba_last_error()
+ * returns a thread-local, NUL-terminated description).  Arguments are validated on the
+ * host BEFORE anything is launched.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * mit-han-lab/flash-moba checkout).
+ */
+#ifndef FLASH_MOBA_HIP_H_
+#define FLASH_MOBA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FMOBA_DTYPE_F16 0
+#define FMOBA_DTYPE_BF16 1
+
+/* Library/ABI version (major*10000 + minor*100 + patch). */
+int fmoba_version(void);
+/* Last error message of the calling thread ("" if none). */
+const char *fmoba_last_error(void);
+/* 0 if the current HIP device is a gfx950 part the kernels were built for, else non-zero
+ * (replaces the compute-capability check of csrc/flash_topk/flash_topk_api.cpp:147-151). */
+int fmoba_check_device(void);
+
+/* ------------------------------------------------------------------------------------
+ * Per-chunk key mean-pool.
+ * Replaces flash_moba/triton_mean_pool.py:41-109 (mean_pool_kernel) as launched by
+ * flash_topk_mean_pool (:112-157):
+ *   km[cu_km[b] + c, h, :] = cast(sum_fp32(k[cu_k[b] + c*chunk + r, h, :], r < n) / n),
+ *   n = min(chunk, len_b - c*chunk).
+ * Rows of km beyond cu_km[batch] are not touched.
+ * ---------------------------------------------------------------------------------- */
+typedef struct {
+  const void *k;            /* (total_k, heads_k, head_dim) */
+  void *km;                 /* (>= cu_km[batch], heads_k, head_dim) */
+  const int32_t *cu_seqlens_k;  /* (batch + 1) */
+  const int32_t *cu_seqlens_km; /* (batch + 1) */
+  int32_t batch;
+  int32_t max_chunks;       /* ceil(max_seqlen_k / chunk) */
+  int32_t heads_k;
+  int32_t head_dim;         /* multiple of 8 */
+  int32_t chunk;
+  int32_t dtype;            /* FMOBA_DTYPE_* */
+  int64_t k_row_stride, k_head_stride;
+  int64_t km_row_stride, km_head_stride;
+} fmoba_mean_pool_args;
+int fmoba_mean_pool(const fmoba_mean_pool_args *a, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Fused top-k block gating + CSC build.
+ * Replaces moba_fused_topk (csrc/flash_topk/flash_topk_api.cpp:130-258), i.e. the three
+ * kernels of csrc/flash_topk/src/flash_topk_launch_template.h:65-118, AND the segmented
+ * sort the reference runs afterwards (flash_moba/flash_moba_interface.py:570-572): the
+ * row lists written to `flat_indices` are already ascending.
+ *
+ *   col_offsets (batch, heads, max_cols) int64, col_nnz (batch, heads, max_cols) int32,
+ *   flat_indices (total_q*heads*topk) int32  -- all fully written by the call
+ *   (unused slots of flat_indices are 0), max_cols = ceil(max_seqlen_k / chunk).
+ *   raw_indices / raw_values (total_q, heads, round_up(topk,16)) int32 / fp32 are the
+ *   ordered per-row lists (descending score, ties -> higher chunk first, unfilled -1 /
+ *   -inf); pass NULL for both to skip them.
+ * ---------------------------------------------------------------------------------- */
+typedef struct {
+  const void *q;            /* (total_q, heads, head_dim) */
+  const void *km;           /* (total_km, heads_k, head_dim) */
+  const int32_t *cu_seqlens_q, *cu_seqlens_k, *cu_seqlens_km; /* (batch + 1) each */
+  int64_t *col_offsets;
+  int32_t *col_nnz;
+  int32_t *flat_indices;
+  int32_t *raw_indices;     /* optional */
+  float *raw_values;        /* optional */
+  void *workspace;          /* fmoba_fused_topk_workspace_bytes() bytes, 256-byte aligned */
+  size_t workspace_bytes;
+  int32_t batch, total_q, heads, heads_k, head_dim;
+  int32_t max_seqlen_q, max_seqlen_k;
+  int32_t topk, chunk, is_causal, dtype;
+  int64_t q_row_stride, q_head_stride, km_row_stride, km_head_stride;
+} fmoba_fused_topk_args;
+size_t fmoba_fused_topk_workspace_bytes(int32_t batch, int32_t total_q, int32_t heads,
+                                        int32_t max_seqlen_q, int32_t max_seqlen_k, int32_t chunk);
+int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Segmented ascending sort of signed int32 keys with 64-bit segment offsets.
+ * Replaces varlen_sort (csrc/flash_topk/src/varlen_sort.cu:127-162, CUB
+ * DeviceSegmentedSort).  dst[i] = 0 for positions outside every segment.  Segments must
+ * not overlap.  `workspace` holds `total` int32 (used by segments too long for LDS).
+ * ---------------------------------------------------------------------------------- */
+size_t fmoba_varlen_sort_workspace_bytes(int64_t total);
+int fmoba_varlen_sort(const int64_t *seg_starts, const int64_t *seg_ends, int64_t num_segments,
+                      const int32_t *src, int32_t *dst, int64_t total, void *workspace,
+                      size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Sparse attention forward over a CSC pattern.
+ * Replaces moba_varlen_fwd (csrc/flash_moba/flash_moba_api.cpp:375-596).
+ *   out (total_q, heads, head_dim) dtype, softmax_lse (heads, total_q) fp32.
+ * Rows that see no key get out = 0, lse = +inf.  No scratch memory is needed.
+ * ---------------------------------------------------------------------------------- */
+typedef struct {
+  const void *q, *k, *v;
+  void *out;
+  float *softmax_lse;
+  const int64_t *col_offsets;   /* (batch, heads, max_cols) */
+  const int32_t *col_nnz;       /* (batch, heads, max_cols) */
+  const int32_t *row_indices;   /* flat row lists */
+  const int32_t *cu_seqlens_q, *cu_seqlens_k;
+  int32_t batch, total_q, total_k, heads, heads_k, head_dim;
+  int32_t max_seqlen_q, max_seqlen_k, max_cols;
+  int32_t lg_block_m, lg_block_n;
+  int32_t is_causal, dtype;
+  float softmax_scale;
+  int64_t q_row_stride, q_head_stride, k_row_stride, k_head_stride;
+  int64_t v_row_stride, v_head_stride, o_row_stride, o_head_stride;
+} fmoba_attn_fwd_args;
+int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Sparse attention backward.
+ * Replaces moba_varlen_bwd (csrc/flash_moba/flash_moba_api.cpp:610-848).
+ *   dq (total_q, heads, d), dk/dv (total_k, heads, d) -- dk/dv are PER QUERY HEAD; for
+ *   GQA/MQA the caller sums groups of heads/heads_k (flash_moba_api.cpp:842-845).
+ *   softmax_d (heads, total_q + 128*batch) fp32: row (b, r) of head h is stored at
+ *   h*(total_q + 128*batch) + cu_q[b] + 128*b + r (flash_bwd_preprocess_kernel.h:86).
+ *   workspace: fp32 dQ accumulator, fmoba_attn_bwd_workspace_bytes() bytes.
+ * ---------------------------------------------------------------------------------- */
+typedef struct {
+  const void *dout, *q, *k, *v, *out;
+  const float *softmax_lse;
+  void *dq, *dk, *dv;
+  float *softmax_d;
+  const int64_t *col_offsets;
+  const int32_t *col_nnz;
+  const int32_t *row_indices;
+  const int32_t *cu_seqlens_q, *cu_seqlens_k;
+  void *workspace;
+  size_t workspace_bytes;
+  int32_t batch, total_q, total_k, heads, heads_k, head_dim;
+  int32_t max_seqlen_q, max_seqlen_k, max_cols;
+  int32_t lg_block_m, lg_block_n;
+  int32_t is_causal, dtype, deterministic;
+  float softmax_scale;
+  int64_t q_row_stride, q_head_stride, k_row_stride, k_head_stride;
+  int64_t v_row_stride, v_head_stride, o_row_stride, o_head_stride;
+  int64_t do_row_stride, do_head_stride;
+  int64_t dq_row_stride, dq_head_stride, dk_row_stride, dk_head_stride;
+  int64_t dv_row_stride, dv_head_stride;
+} fmoba_attn_bwd_args;
+size_t fmoba_attn_bwd_workspace_bytes(int32_t total_q, int32_t heads, int32_t head_dim);
+int fmoba_attn_bwd(const fmoba_attn_bwd_args *a, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASH_MOBA_HIP_H_ */

@@ -1,0 +1,397 @@
+"""GPU parity tests: every stage of the HIP path (called through the C-ABI binding)
+against the CPU oracle on the same seeded inputs.
+
+Bars: bit-exact for integer artefacts (CSC triple, sorted keys) wherever the oracle's
+score gap between the last kept and first rejected chunk exceeds 1e-3 relative;
+2e-2 abs / 1e-2 rel for bf16/fp16 attention outputs and gradients; 1e-2 abs for the
+mean-pool (the reference's own tolerance, tests/test_triton_mean_pool.py:63-64), tightened
+here to one ulp of the output dtype.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moba_oracle as O
+from gpu_utils import assert_close, csc_structure_ok, selection_sets
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fm():
+    import flash_moba
+    from flash_moba import flash_moba_hip, flash_moba_interface, mean_pool
+
+    class NS:
+        pass
+
+    ns = NS()
+    ns.api = flash_moba
+    ns.hip = flash_moba_hip
+    ns.iface = flash_moba_interface
+    ns.pool = mean_pool
+    return ns
+
+
+# ------------------------------------------------------------------------ mean-pool
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("batch,max_seqlen,heads,d,pool", [
+    (1, 512, 4, 64, 32), (8, 2048, 12, 128, 64), (8, 512, 4, 256, 128), (1, 2048, 12, 64, 512),
+    (8, 2048, 4, 128, 256), (4, 128, 4, 32, 256), (16, 8, 4, 32, 4), (3, 777, 5, 72, 48),
+])
+def test_mean_pool_matches_oracle(fm, batch, max_seqlen, heads, d, pool, dtype):
+    g = torch.Generator().manual_seed(42)
+    seqlens = torch.randint(0, max_seqlen, (batch,), generator=g)
+    cu = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(seqlens, 0)]).to(torch.int32)
+    x = torch.randn((int(seqlens.sum()), heads, d), generator=g).to(dtype)
+    km, cu_km, maxc = fm.pool.flash_topk_mean_pool(x.cuda(), cu.cuda(), max_seqlen, pool)
+    ref, cu_ref = O.mean_pool(x, cu, pool)
+    assert km.shape == ref.shape and km.dtype == dtype
+    assert torch.equal(cu_km.cpu(), cu_ref) and cu_km.dtype == torch.int32
+    assert maxc == (max_seqlen + pool - 1) // pool
+    # fp32 accumulation in a different order: at most one ulp of the 16-bit result
+    ulp = (ref.float().abs() * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)).clamp_min(1e-6)
+    assert ((km.cpu().float() - ref.float()).abs() <= ulp).all()
+    assert torch.allclose(km.cpu().float(), ref.float(), atol=1e-2, rtol=0)
+
+
+def test_mean_pool_all_empty_and_strided(fm):
+    cu = torch.zeros(9, dtype=torch.int32).cuda()
+    km, cu_km, _ = fm.pool.flash_topk_mean_pool(torch.zeros((0, 12, 128), dtype=torch.bfloat16).cuda(), cu, 0, 128)
+    assert km.shape == (0, 12, 128) and cu_km.tolist() == [0] * 9
+    # k taken as a strided view of a packed qkv tensor
+    g = torch.Generator().manual_seed(1)
+    qkv = torch.randn((300, 3, 4, 64), generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0, 100, 300], dtype=torch.int32)
+    k = qkv[:, 1]
+    km, _, _ = fm.pool.flash_topk_mean_pool(qkv.cuda()[:, 1], cu.cuda(), 200, 64)
+    ref, _ = O.mean_pool(k.contiguous(), cu, 64)
+    assert torch.allclose(km.cpu().float(), ref.float(), atol=1e-2)
+
+
+# ------------------------------------------------------------------------ gating + CSC
+def _gate_case(fm, seed, lens_q, lens_k, H, Hk, D, chunk, topk, causal, dtype=torch.bfloat16, integer=False):
+    g = torch.Generator().manual_seed(seed)
+    Tq, Tk = sum(lens_q), sum(lens_k)
+    if integer:
+        q = torch.randint(-2, 3, (Tq, H, D), generator=g).to(dtype)
+        k = torch.randint(-1, 2, (Tk, Hk, D), generator=g).to(dtype)
+    else:
+        q = torch.randn((Tq, H, D), generator=g).to(dtype)
+        k = torch.randn((Tk, Hk, D), generator=g)
+        # per-chunk bias so that scores separate
+        pos = 0
+        for L in lens_k:
+            C = (L + chunk - 1) // chunk
+            if C:
+                k[pos:pos + L] += (0.5 * torch.randn((C, Hk, D), generator=g)).repeat_interleave(chunk, 0)[:L]
+            pos += L
+        k = k.to(dtype)
+    cuq = torch.tensor([0] + list(np.cumsum(lens_q)), dtype=torch.int32)
+    cuk = torch.tensor([0] + list(np.cumsum(lens_k)), dtype=torch.int32)
+    return q, k, cuq, cuk
+
+
+def _check_gating(fm, q, k, cuq, cuk, chunk, topk, causal, integer=False):
+    H = q.shape[1]
+    max_q, max_k = int((cuq[1:] - cuq[:-1]).max()), int((cuk[1:] - cuk[:-1]).max())
+    maxC = (max_k + chunk - 1) // chunk
+    # chunk means from the HIP kernel feed both sides, so that only the gating is compared
+    km_gpu, cu_km, _ = fm.pool.flash_topk_mean_pool(k.cuda(), cuk.cuda(), max_k, chunk)
+    if integer:
+        km_gpu = (km_gpu.float() * chunk).round().to(k.dtype)   # integer-valued chunk sums: scores tie exactly
+    co, cn, flat, values, indices = fm.hip.moba_fused_topk(
+        q.cuda(), km_gpu, cuq.cuda(), cuk.cuda(), cu_km, max_q, max_k, topk, chunk, causal)
+    torch.cuda.synchronize()
+    idx_ref, val_ref, gates = O.fused_topk(q, km_gpu.cpu(), cuq, cuk, cu_km.cpu(), topk, chunk, causal, return_gate=True)
+    co_ref, cn_ref, flat_ref = O.csc_from_topk(idx_ref, cuq, topk, maxC)
+    assert co.dtype == torch.int64 and cn.dtype == torch.int32 and flat.dtype == torch.int32
+    assert co.shape == co_ref.shape and cn.shape == cn_ref.shape and flat.shape == flat_ref.shape
+    csc_structure_ok(co, cn, flat, cuq, H, topk)
+    unamb = O.topk_gap_mask(gates, cuq, topk, 1e-3) if any(g is not None for g in gates) else None
+    n_amb = 0 if unamb is None else int((~unamb).sum())
+    if n_amb == 0 or integer:
+        # no near-tie anywhere (or exact integer arithmetic): everything must be bit-exact
+        assert torch.equal(cn.cpu(), cn_ref)
+        assert torch.equal(co.cpu(), co_ref)
+        assert torch.equal(flat.cpu(), flat_ref)
+    else:
+        # rows away from near-ties must select exactly the oracle's chunk set
+        cuq_np = cuq.numpy()
+        for b in range(len(cuq_np) - 1):
+            Lq = int(cuq_np[b + 1] - cuq_np[b])
+            for h in range(H):
+                got = selection_sets(co, cn, flat, b, h, Lq, maxC)
+                ref = selection_sets(co_ref, cn_ref, flat_ref, b, h, Lq, maxC)
+                ok_rows = unamb[int(cuq_np[b]):int(cuq_np[b + 1]), h].numpy()
+                assert (got[ok_rows] == ref[ok_rows]).all()
+                assert (got.sum(1) == ref.sum(1)).all()       # same number of chunks everywhere
+        assert n_amb < 0.005 * unamb.numel() + 8
+    # ordered per-row lists (auxiliary outputs): same sets as the CSC, descending scores
+    kr = (topk + 15) // 16 * 16
+    assert indices.shape == (q.shape[0], H, kr) and values.shape == indices.shape
+    mism = (indices.cpu() != idx_ref).float().mean().item()
+    assert mism < 0.005 or integer, mism        # the reference's own bar (tests/test_fused_topk.py:251-254)
+    if integer:
+        assert torch.equal(indices.cpu(), idx_ref)
+        assert torch.equal(values.cpu(), val_ref)
+
+
+@pytest.mark.parametrize("topk", [1, 2, 4, 8, 16, 24, 32, 33, 64])
+@pytest.mark.parametrize("chunk", [1, 16, 32])
+@pytest.mark.parametrize("causal", [True, False])
+def test_gating_reference_grid(fm, topk, chunk, causal):
+    # (b, h, s) grid of tests/test_fused_topk.py:119-122 limited to <= 256 chunks per sequence
+    for (b, h, s, d, dt) in [(1, 4, 128, 64, torch.float16), (2, 8, 256, 128, torch.bfloat16), (4, 4, 512, 256, torch.bfloat16)]:
+        if (s + chunk - 1) // chunk > 256:
+            continue
+        q, k, cuq, cuk = _gate_case(fm, 0, [s] * b, [s] * b, h, h, d, chunk, topk, causal, dt)
+        _check_gating(fm, q, k, cuq, cuk, chunk, topk, causal)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("topk,chunk", [(3, 16), (8, 32), (5, 64)])
+def test_gating_exact_ties_prefer_higher_chunk(fm, topk, chunk, causal):
+    q, k, cuq, cuk = _gate_case(fm, 7, [300, 0, 513], [300, 0, 513], 4, 2, 64, chunk, topk, causal, integer=True)
+    _check_gating(fm, q, k, cuq, cuk, chunk, topk, causal, integer=True)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_gating_ragged_varlen_gqa_and_len_q_ne_len_k(fm, causal):
+    q, k, cuq, cuk = _gate_case(fm, 11, [200, 77, 0, 1, 640], [333, 50, 0, 130, 640], 6, 2, 72, 64, 4, causal)
+    _check_gating(fm, q, k, cuq, cuk, 64, 4, causal)
+
+
+def test_gating_headline_shape_small(fm):
+    # the headline configuration's shape parameters (d=128, chunk 64, top-k 32) at 2 x ~3K tokens
+    q, k, cuq, cuk = _gate_case(fm, 5, [3072, 2112], [3072, 2112], 4, 4, 128, 64, 32, True)
+    _check_gating(fm, q, k, cuq, cuk, 64, 32, True)
+
+
+def test_gating_no_keys(fm):
+    q = torch.randn(10, 2, 64).to(torch.bfloat16).cuda()
+    km = torch.zeros(0, 2, 64, dtype=torch.bfloat16).cuda()
+    cuq = torch.tensor([0, 10], dtype=torch.int32).cuda()
+    z = torch.tensor([0, 0], dtype=torch.int32).cuda()
+    co, cn, flat, val, idx = fm.hip.moba_fused_topk(q, km, cuq, z, z, 10, 0, 4, 16, True)
+    assert co.shape == (1, 2, 0) and (flat == -1).all() and (idx == -1).all() and torch.isinf(val).all()
+
+
+def test_gating_rejects_bad_arguments(fm):
+    q = torch.zeros(8, 2, 64, dtype=torch.bfloat16).cuda()
+    cu = torch.tensor([0, 8], dtype=torch.int32).cuda()
+    with pytest.raises(RuntimeError, match="moba_topk must be <= 64"):
+        fm.hip.moba_fused_topk(q, q, cu, cu, cu, 8, 8, 65, 4, True)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        fm.hip.moba_fused_topk(q[..., :60].contiguous(), q[..., :60].contiguous(), cu, cu, cu, 8, 8, 2, 4, True)
+    with pytest.raises(RuntimeError, match="int32"):
+        fm.hip.moba_fused_topk(q, q, cu.long(), cu, cu, 8, 8, 2, 4, True)
+    with pytest.raises(RuntimeError, match="same dtype"):
+        fm.hip.moba_fused_topk(q, q.half(), cu, cu, cu, 8, 8, 2, 4, True)
+
+
+# ------------------------------------------------------------------------ segmented sort
+@pytest.mark.parametrize("segments,seed,maxlen", [(1, 3, 2 ** 18), (17, 11, 2 ** 16), (128, 47, 2 ** 14), (1024, 97, 4096), (4096, 233, 512)])
+def test_varlen_sort_random(fm, segments, seed, maxlen):
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(0, maxlen, (segments,), generator=g)
+    ends = torch.cumsum(lens, 0).to(torch.int64)
+    starts = ends - lens
+    total = int(ends[-1])
+    src = torch.randint(0, 2 ** 31 - 1, (total,), generator=g, dtype=torch.int64).to(torch.int32)
+    out = fm.hip.varlen_sort(starts.cuda(), ends.cuda(), src.cuda())
+    ref = O.varlen_sort(starts, ends, src)
+    assert torch.equal(out.cpu(), ref)
+
+
+def test_varlen_sort_extremes_gaps_and_small_ranges(fm):
+    i32 = torch.iinfo(torch.int32)
+    vals = torch.tensor([i32.max, i32.min] * 32, dtype=torch.int32)
+    starts = torch.tensor([0, 16, 32, 48], dtype=torch.int64)
+    ends = starts + 16
+    out = fm.hip.varlen_sort(starts.cuda(), ends.cuda(), vals.cuda())
+    assert torch.equal(out.cpu(), O.varlen_sort(starts, ends, vals))
+    # gaps between segments stay zero; negative keys; a long segment of row-index-like keys
+    g = torch.Generator().manual_seed(5)
+    src = torch.randint(-50000, 50000, (100000,), generator=g, dtype=torch.int64).to(torch.int32)
+    starts = torch.tensor([5, 1000, 30000, 99990], dtype=torch.int64)
+    ends = torch.tensor([900, 1000, 90000, 100000], dtype=torch.int64)
+    out = fm.hip.varlen_sort(starts.cuda(), ends.cuda(), src.cuda())
+    assert torch.equal(out.cpu(), O.varlen_sort(starts, ends, src))
+    out = fm.hip.varlen_sort(starts[:0].cuda(), ends[:0].cuda(), src.cuda())
+    assert (out == 0).all()
+
+
+def test_varlen_sort_restores_a_shuffled_csc(fm):
+    # the op as the reference pipeline uses it: shuffle each column list, sort it back
+    q, k, cuq, cuk = _gate_case(fm, 3, [700, 300], [700, 300], 4, 4, 64, 32, 6, True)
+    co, cn, flat = fm.api.flash_topk_varlen_func(q.cuda(), k.cuda(), cuq.cuda(), cuk.cuda(), 700, 700, 6, 32, causal=True)
+    f = flat.cpu().clone()
+    g = torch.Generator().manual_seed(0)
+    for s, n in zip(co.flatten().tolist(), cn.flatten().tolist()):
+        if n > 1:
+            f[s:s + n] = f[s:s + n][torch.randperm(n, generator=g)]
+    back = torch.ops.flash_moba._varlen_sort(co, cn, f.cuda())
+    assert torch.equal(back, flat)
+
+
+# ------------------------------------------------------------------------ attention
+def _random_csc(seed, lens_q, lens_k, H, lg_n, topk, causal):
+    """Random block pattern in the spirit of generate_moba_sparse_mask_topk
+    (flash_moba/moba_test_utils.py:61-96) with the gap-free running offsets of
+    generate_moba_params_from_sparse_mask (:169-191)."""
+    rng = np.random.RandomState(seed)
+    nb = len(lens_q)
+    maxC = (max(lens_k) + lg_n - 1) // lg_n
+    co = np.zeros((nb, H, maxC), dtype=np.int64)
+    cn = np.zeros((nb, H, maxC), dtype=np.int32)
+    rows_all = []
+    offset = 0
+    for b in range(nb):
+        Lq, Lk = lens_q[b], lens_k[b]
+        for h in range(H):
+            lists = [[] for _ in range(maxC)]
+            for r in range(Lq):
+                end_col = Lk - (Lq - r - 1) if causal else Lk
+                nblk = max(0, math.ceil(end_col / lg_n))
+                if nblk > 0:
+                    sel = set(rng.permutation(nblk - 1)[: min(topk - 1, nblk - 1)].tolist()) | {nblk - 1}
+                    for c in sel:
+                        lists[c].append(r)
+            for c in range(maxC):
+                co[b, h, c] = offset
+                cn[b, h, c] = len(lists[c])
+                rows_all.extend(lists[c])
+                offset += len(lists[c])
+    ind = np.array(rows_all if rows_all else [0], dtype=np.int32)
+    return torch.from_numpy(co), torch.from_numpy(cn), torch.from_numpy(ind)
+
+
+def _attn_inputs(seed, lens_q, lens_k, H, Hk, D, dtype):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((sum(lens_q), H, D), generator=g).to(dtype)
+    k = torch.randn((sum(lens_k), Hk, D), generator=g).to(dtype)
+    v = torch.randn((sum(lens_k), Hk, D), generator=g).to(dtype)
+    dout = torch.randn((sum(lens_q), H, D), generator=g).to(dtype)
+    cuq = torch.tensor([0] + list(np.cumsum(lens_q)), dtype=torch.int32)
+    cuk = torch.tensor([0] + list(np.cumsum(lens_k)), dtype=torch.int32)
+    return q, k, v, dout, cuq, cuk
+
+
+def _check_attention(fm, q, k, v, dout, cuq, cuk, co, cn, ind, lg_n, causal, scale=None, lg_m=128, check_grads=True):
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    max_q, max_k = int((cuq[1:] - cuq[:-1]).max()), int((cuk[1:] - cuk[:-1]).max())
+    out, lse, _ = fm.api.flash_moba_attn_varlen_func(
+        qg, kg, vg, cuq.cuda(), cuk.cuda(), max_q, max_k, co.cuda(), cn.cuda(), ind.cuda(),
+        lg_m, lg_n, softmax_scale=scale, causal=causal, return_attn_probs=True)
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = O.attn_fwd_bwd(q, k, v, dout, cuq, cuk, co, cn, ind, lg_n, scale, causal)
+    assert out.dtype == q.dtype and out.shape == q.shape
+    assert lse.dtype == torch.float32 and lse.shape == (q.shape[1], q.shape[0])
+    assert_close("out", out, o_ref, 2e-2, 1e-2)
+    fin = torch.isfinite(lse_ref)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    assert (lse.cpu()[~fin] == float("inf")).all()
+    assert_close("lse", lse.cpu()[fin], lse_ref[fin], 2e-2, 1e-2)
+    if check_grads:
+        dq, dk, dv = torch.autograd.grad(out, (qg, kg, vg), dout.cuda())
+        assert dq.dtype == q.dtype and dk.shape == k.shape and dv.shape == v.shape
+        assert_close("dq", dq, dq_ref, 2e-2, 1e-2)
+        assert_close("dk", dk, dk_ref, 2e-2 * max(1, q.shape[1] // k.shape[1]), 1e-2)
+        assert_close("dv", dv, dv_ref, 2e-2 * max(1, q.shape[1] // k.shape[1]), 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("mha", ["mha", "gqa", "mqa"])
+@pytest.mark.parametrize("d", [64, 128, 96, 59])
+@pytest.mark.parametrize("sq,sk", [(113, 203), (128, 217), (256, 512), (512, 256), (1023, 1024)])
+def test_attention_random_pattern(fm, sq, sk, d, mha, causal, dtype):
+    if dtype == torch.float16 and (d != 128 or mha != "mha"):
+        pytest.skip("fp16 is covered at d=128 / mha")
+    H = 6
+    Hk = {"mha": 6, "gqa": 2, "mqa": 1}[mha]
+    # padded batch in the spirit of tests/test_moba_attn.py:103-104: lengths a little below the maximum
+    rng = np.random.RandomState(sq + sk)
+    lens_q = [max(1, sq - int(x)) for x in rng.randint(0, 20, 3)]
+    lens_k = [max(1, sk - int(x)) for x in rng.randint(0, 20, 3)]
+    q, k, v, dout, cuq, cuk = _attn_inputs(0, lens_q, lens_k, H, Hk, d, dtype)
+    co, cn, ind = _random_csc(1, lens_q, lens_k, H, 64, 4, causal)
+    _check_attention(fm, q, k, v, dout, cuq, cuk, co, cn, ind, 64, causal)
+
+
+@pytest.mark.parametrize("chunk,topk", [(64, 4), (128, 3), (64, 32)])
+def test_attention_on_gated_pattern(fm, chunk, topk):
+    lens = [640, 1, 0, 1300]
+    q, k, v, cu, dout = O.make_inputs(lens, 4, 128, chunk, 21, torch.bfloat16, with_dout=True)
+    co, cn, ind = fm.api.flash_topk_varlen_func(q.cuda(), k.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens), topk, chunk, causal=True)
+    _check_attention(fm, q, k, v, dout, cu, cu, co.cpu(), cn.cpu(), ind.cpu(), chunk, True, lg_m=256)
+
+
+def test_attention_dense_special_case_matches_sdpa(fm):
+    # top-k >= number of chunks: plain causal attention
+    L, H, D, chunk = 512, 2, 128, 64
+    q, k, v, cu = O.make_inputs([L], H, D, chunk, 3, torch.bfloat16)
+    out = fm.api.flash_moba_varlen_func(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), L, L, chunk, 16, causal=True)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.float().transpose(0, 1), k.float().transpose(0, 1), v.float().transpose(0, 1), is_causal=True).transpose(0, 1)
+    assert_close("out", out, ref, 2e-2, 1e-2)
+
+
+def test_attention_rows_without_keys_and_no_keys_at_all(fm):
+    # len_q > len_k, causal: leading rows see nothing -> out 0, lse +inf, zero gradients
+    q, k, v, dout, cuq, cuk = _attn_inputs(4, [200], [130], 2, 2, 64, torch.bfloat16)
+    co, cn, ind = fm.api.flash_topk_varlen_func(q.cuda(), k.cuda(), cuq.cuda(), cuk.cuda(), 200, 130, 2, 64, causal=True)
+    _check_attention(fm, q, k, v, dout, cuq, cuk, co.cpu(), cn.cpu(), ind.cpu(), 64, True)
+    z = torch.zeros(2, dtype=torch.int32).cuda()
+    out, lse, _, _ = fm.hip.moba_varlen_fwd(
+        q.cuda(), k[:0].cuda(), v[:0].cuda(), None, torch.zeros((1, 2, 0), dtype=torch.int64).cuda(),
+        torch.zeros((1, 2, 0), dtype=torch.int32).cuda(), torch.zeros((0,), dtype=torch.int32).cuda(), cuq.cuda(), z,
+        None, None, None, 200, 0, 0.0, 0.125, False, True, 0.0, False, 128, 64, None)
+    assert (out == 0).all() and (lse == float("inf")).all()
+
+
+def test_attention_rejects_unsupported_options(fm):
+    q, k, v, dout, cuq, cuk = _attn_inputs(4, [128], [128], 2, 2, 64, torch.bfloat16)
+    co, cn, ind = _random_csc(1, [128], [128], 2, 64, 2, True)
+    args = [t.cuda() for t in (q, k, v, cuq, cuk)] + [128, 128] + [t.cuda() for t in (co, cn, ind)]
+    with pytest.raises(RuntimeError, match="dropout"):
+        fm.api.flash_moba_attn_varlen_func(*args, 128, 64, dropout_p=0.1)
+    with pytest.raises(RuntimeError, match="softcap"):
+        fm.api.flash_moba_attn_varlen_func(*args, 128, 64, softcap=30.0)
+    with pytest.raises(RuntimeError, match="ALiBi"):
+        fm.api.flash_moba_attn_varlen_func(*args, 128, 64, alibi_slopes=torch.ones(2).cuda())
+    with pytest.raises(RuntimeError, match="m_lg_block_dim"):
+        fm.api.flash_moba_attn_varlen_func(*args, 64, 64)
+    with pytest.raises(RuntimeError, match="n_lg_block_dim"):
+        fm.api.flash_moba_attn_varlen_func(*args, 128, 32)
+    with pytest.raises(RuntimeError, match="int64"):
+        fm.api.flash_moba_attn_varlen_func(*args[:7], co.int().cuda(), cn.cuda(), ind.cuda(), 128, 64)
+
+
+# ------------------------------------------------------------------------ end to end
+def test_end_to_end_config1_shape_against_dense_reference(fm):
+    # BASELINE config 1 (lengths [1024, 2048], 8 heads, d=64, chunk 128, top-k 4) evaluated by the HIP
+    # path in bf16 against the CPU reference path in fp32 on the same (bf16-rounded) inputs
+    lens = [1024, 2048]
+    q, k, v, cu = O.make_inputs(lens, 8, 64, 128, 1001, torch.bfloat16)
+    out = fm.api.flash_moba_varlen_func(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), 2048, 2048, 128, 4, causal=True)
+    ref = O.moba_dense_ref(q.float(), k.float(), v.float(), cu, cu, 128, 4, True)
+    # gating uses bf16-rounded chunk means; a near-tie may flip a chunk for a few rows
+    err = (out.float().cpu() - ref).abs()
+    bad_rows = (err > 2e-2 + 1e-2 * ref.abs()).any(-1)
+    assert bad_rows.float().mean().item() < 0.005
+
+
+def test_end_to_end_backward_runs_through_autograd(fm):
+    lens = [512, 384]
+    q, k, v, cu, dout = O.make_inputs(lens, 4, 128, 64, 77, torch.bfloat16, with_dout=True)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = fm.api.flash_moba_varlen_func(qg, kg, vg, cu.cuda(), cu.cuda(), 512, 512, 64, 3, causal=True)
+    out.backward(dout.cuda())
+    co, cn, ind = fm.api.flash_topk_varlen_func(q.cuda(), k.cuda(), cu.cuda(), cu.cuda(), 512, 512, 3, 64, causal=True)
+    _, _, dq_ref, dk_ref, dv_ref = O.attn_fwd_bwd(q, k, v, dout, cu, cu, co.cpu(), cn.cpu(), ind.cpu(), 64, None, True)
+    assert_close("dq", qg.grad, dq_ref, 2e-2, 1e-2)
+    assert_close("dk", kg.grad, dk_ref, 2e-2, 1e-2)
+    assert_close("dv", vg.grad, dv_ref, 2e-2, 1e-2)

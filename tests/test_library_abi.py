@@ -1,0 +1,118 @@
+"""CPU-side checks of the C-ABI library: it loads and exports every symbol the header
+declares; argument structs have the layout the header gives them; the host-side
+validation of the binding raises before anything touches a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from flash_moba import flash_moba_hip as H
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    src = open(os.path.join(ROOT, "include", "flash_moba_hip.h")).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(fmoba_[a-z_0-9]+)\s*\(", src)))
+
+
+def test_header_declares_the_expected_entry_points():
+    fns = header_functions()
+    for need in ("fmoba_mean_pool", "fmoba_fused_topk", "fmoba_varlen_sort", "fmoba_attn_fwd", "fmoba_attn_bwd",
+                 "fmoba_last_error", "fmoba_version", "fmoba_check_device"):
+        assert need in fns
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = H.load_library()
+    for fn in header_functions():
+        assert hasattr(lib, fn), fn
+        assert fn in H.EXPORTS, f"{fn} is declared in the header but not bound"
+    assert lib.fmoba_version() >= 100
+    assert lib.fmoba_last_error() is not None
+
+
+def test_workspace_queries_are_pure_host_functions():
+    lib = H.load_library()
+    # selection bits: heads * ceil(maxC/32) * total_q words; counts: batch*heads*nseg*maxC words
+    b = lib.fmoba_fused_topk_workspace_bytes(8, 65536, 16, 14336, 14336, 64)
+    assert b >= 16 * 7 * 65536 * 4 + 8 * 16 * 7 * 224 * 4
+    assert lib.fmoba_fused_topk_workspace_bytes(0, 0, 0, 0, 0, 0) == 0
+    assert lib.fmoba_varlen_sort_workspace_bytes(1000) == 4000
+    assert lib.fmoba_attn_bwd_workspace_bytes(1024, 4, 128) >= 1024 * 4 * 128 * 4
+
+
+def test_struct_sizes_match_the_header_layout():
+    # pointers and int64 are 8 bytes, int32/float 4; sizes follow from the field lists
+    assert ctypes.sizeof(H.MeanPoolArgs) == 4 * 8 + 6 * 4 + 4 * 8
+    assert ctypes.sizeof(H.FusedTopkArgs) == 11 * 8 + 8 + 11 * 4 + 4 + 4 * 8
+    assert ctypes.sizeof(H.AttnFwdArgs) % 8 == 0
+    assert ctypes.sizeof(H.AttnBwdArgs) % 8 == 0
+
+
+def test_null_args_are_rejected_with_a_message():
+    lib = H.load_library()
+    assert lib.fmoba_mean_pool(None, None) != 0
+    assert b"null" in lib.fmoba_last_error()
+    assert lib.fmoba_fused_topk(None, None) != 0
+    assert lib.fmoba_attn_fwd(None, None) != 0
+    assert lib.fmoba_attn_bwd(None, None) != 0
+
+
+def test_host_validation_needs_no_gpu():
+    q = torch.zeros(4, 2, 8)          # fp32, CPU
+    cu = torch.tensor([0, 4], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="fp16 and bf16"):
+        H.moba_fused_topk(q, q, cu, cu, cu, 4, 4, 2, 2, True)
+    with pytest.raises(RuntimeError, match="on CUDA"):
+        H.moba_fused_topk(q.half(), q.half(), cu, cu, cu, 4, 4, 2, 2, True)
+    with pytest.raises(RuntimeError, match="int64"):
+        H.varlen_sort(cu, cu, cu)
+
+
+def test_public_api_signatures_are_the_reference_ones():
+    import inspect
+
+    import flash_moba
+    from flash_moba import flash_moba_interface as I
+
+    assert list(inspect.signature(flash_moba.flash_moba_varlen_func).parameters) == [
+        "q", "k", "v", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "moba_chunk_size", "moba_topk", "causal"]
+    assert inspect.signature(flash_moba.flash_moba_varlen_func).parameters["causal"].default is True
+    assert list(inspect.signature(flash_moba.flash_topk_varlen_func).parameters) == [
+        "q", "k", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "moba_topk", "moba_chunk_size", "causal"]
+    assert inspect.signature(flash_moba.flash_topk_varlen_func).parameters["causal"].default is False
+    p = inspect.signature(flash_moba.flash_moba_attn_varlen_func).parameters
+    assert list(p) == ["q", "k", "v", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k",
+                       "moba_col_offsets", "moba_col_nnz", "moba_row_indices", "lg_block_m", "lg_block_n", "dropout_p",
+                       "softmax_scale", "causal", "softcap", "alibi_slopes", "deterministic", "return_attn_probs"]
+    assert (p["lg_block_m"].default, p["lg_block_n"].default, p["causal"].default) == (64, 64, False)
+    for op in ("_moba_fused_topk", "_varlen_sort", "_flash_moba_attn_varlen_forward", "_flash_moba_attn_varlen_backward"):
+        assert hasattr(torch.ops.flash_moba, op)
+    assert I.decide_lg_block_m(8, 128, 8192, True) == 512
+    from flash_moba.triton_mean_pool import flash_topk_mean_pool  # import path of the reference
+    assert callable(flash_topk_mean_pool)
+
+
+def test_fake_shape_functions():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    import flash_moba  # noqa: F401  (registers the ops)
+
+    with FakeTensorMode():
+        q = torch.empty(100, 4, 64, dtype=torch.bfloat16, device="cuda")
+        km = torch.empty(10, 4, 64, dtype=torch.bfloat16, device="cuda")
+        cu = torch.empty(3, dtype=torch.int32, device="cuda")
+        co, cn, ind = torch.ops.flash_moba._moba_fused_topk(q, km, cu, cu, cu, 60, 60, 3, 16, True)
+        assert co.shape == (2, 4, 4) and co.dtype == torch.int64
+        assert cn.shape == (2, 4, 4) and cn.dtype == torch.int32
+        assert ind.shape == (100 * 4 * 3,) and ind.dtype == torch.int32
+        out, lse, p, rng = torch.ops.flash_moba._flash_moba_attn_varlen_forward(
+            q, q, q, cu, cu, 60, 60, co, cn, ind, 128, 64, 0.0, 0.125, True)
+        assert out.shape == q.shape and lse.shape == (4, 100) and p.shape == (0,) and rng.shape == (2,)
+        sd = torch.ops.flash_moba._flash_moba_attn_varlen_backward(
+            q, q, q, q, out, lse, None, None, None, cu, cu, 60, 60, co, cn, ind, 128, 64, 0.0, 0.125, True, 0.0, None, False)
+        assert sd.shape == (4, 100 + 128 * 2)
