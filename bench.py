@@ -1,0 +1,263 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoBA hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config headline|c2|c3]
+
+A step is one pass of the hot path over one batch of synthetic input with everything
+already resident in HBM: mean-pool -> fused top-k gating -> CSC build -> sparse attention
+forward -> sparse attention backward (``flash_moba_varlen_func`` + ``.backward``).  The
+default workload is the headline configuration: a packed batch of 8 sequences totalling
+65536 tokens, bf16, causal, 16 heads, head_dim 128, chunk 64, top-k 32.
+
+Prints ONE JSON line: the metric (effective sparse TFLOP/s of fwd+bwd attention over the
+step time), ms per step, per-stage times with their roofline fractions, a ``roofline``
+object for the dominant kernel (timed alone with events on the launch stream) and a
+``cpu_baseline`` object (the CPU restatement of the reference's PyTorch MoBA path timed on
+the host cores on a bounded sample of the same inputs).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "flash-moba_amd"))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks used for every roofline fraction printed here
+PEAK_HBM_GBS = 8000.0          # GB/s
+PEAK_BF16_TFLOPS = 2500.0      # dense bf16 MFMA, TFLOP/s
+
+CONFIGS = {
+    # name: (seqlens or None for the seeded headline rule, heads, head_dim, chunk, topk, backward)
+    "headline": (None, 16, 128, 64, 32, True),
+    "c2": ([8192], 16, 128, 128, 8, False),
+    "c3": ([32768], 32, 128, 128, 16, True),
+}
+
+
+def headline_seqlens(seed=1004, n=8, total=65536, lo=2048, hi=14336, mult=64):
+    """8 lengths ~ U[lo, hi] from a seeded RNG, rescaled to sum to `total`, rounded to multiples
+    of `mult`, the last one fixed so that the sum is exact."""
+    rng = np.random.RandomState(seed)
+    raw = rng.uniform(lo, hi, size=n)
+    lens = [int(round(x / raw.sum() * total / mult)) * mult for x in raw]
+    lens[-1] = total - sum(lens[:-1])
+    return lens
+
+
+def make_inputs(seqlens, H, D, chunk, seed, device):
+    """q, v, dout ~ N(0,1); k = N(0,1) + per-(sequence, chunk, head) bias ~ N(0, 0.5)."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    T = sum(seqlens)
+    q = torch.randn((T, H, D), generator=g, device=device)
+    k = torch.randn((T, H, D), generator=g, device=device)
+    v = torch.randn((T, H, D), generator=g, device=device)
+    dout = torch.randn((T, H, D), generator=g, device=device)
+    pos = 0
+    for L in seqlens:
+        C = (L + chunk - 1) // chunk
+        bias = 0.5 * torch.randn((C, H, D), generator=g, device=device)
+        k[pos:pos + L] += bias.repeat_interleave(chunk, dim=0)[:L]
+        pos += L
+    cu = torch.tensor([0] + list(np.cumsum(seqlens)), dtype=torch.int32, device=device)
+    bf = torch.bfloat16
+    return q.to(bf), k.to(bf), v.to(bf), dout.to(bf), cu
+
+
+def count_pairs(seqlens, col_nnz, chunk, H):
+    """Unmasked (query, key) pairs of a causal, gating-produced pattern (len_q == len_k): every
+    listed (row, chunk) pair contributes `chunk` keys, except a row's own chunk, which
+    contributes (row mod chunk) + 1."""
+    total = int(col_nnz.sum().item()) * chunk
+    for L in seqlens:
+        r = np.arange(L)
+        total -= H * int((chunk - (r % chunk) - 1).sum())
+    return total
+
+
+def time_events(fn, iters, warmup=1):
+    """Average milliseconds of fn() over `iters` runs, measured with events recorded on the
+    stream the kernels are launched on (torch's current stream)."""
+    for _ in range(warmup):
+        fn()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters
+
+
+def cpu_baseline(q, k, v, cu, seqlens, chunk, topk, budget_s=12.0):
+    """Times the CPU restatement of the reference's PyTorch MoBA path (chunk means -> gate ->
+    top-k -> block mask -> dense-masked softmax attention, fp32) on (sequence 0, heads 0..n)
+    of the same inputs, adding heads until ~budget_s of CPU work has been done."""
+    from oracle import moba_oracle as O  # checker only: never on the product path
+
+    torch.set_num_threads(os.cpu_count())
+    L = seqlens[0]
+    qs, ks, vs = (t[:L].float().cpu() for t in (q, k, v))
+    cu0 = torch.tensor([0, L], dtype=torch.int32)
+    H, D = q.shape[1], q.shape[2]
+    t0 = time.perf_counter()
+    heads = 0
+    while heads < H and (time.perf_counter() - t0) < budget_s:
+        O.moba_dense_ref(qs[:, heads:heads + 1], ks[:, heads:heads + 1], vs[:, heads:heads + 1], cu0, cu0, chunk, topk, True,
+                         row_block=1024)
+        heads += 1
+    dt = time.perf_counter() - t0
+    C = (L + chunk - 1) // chunk
+    pairs = heads * (sum(min(chunk, L - c * chunk) * (min(chunk, L - c * chunk) + 1) // 2 for c in range(C))
+                     + chunk * chunk * sum(min(topk - 1, c) for c in range(C)))
+    flops = 4.0 * D * pairs
+    return {
+        "value": flops / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": os.cpu_count(),
+        "kind": "port",
+        "sample": f"forward only, fp32, sequence 0 ({L} tokens) x {heads} of {H} heads, row-blocked dense-masked "
+                  f"attention; {dt:.1f} s of CPU time; effective sparse FLOPs / time",
+        "seconds": dt,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="headline", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+
+    import flash_moba
+    from flash_moba import flash_moba_hip as hip
+    from flash_moba.mean_pool import mean_pool_nosync
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    seqlens, H, D, chunk, topk, backward = CONFIGS[args.config]
+    if seqlens is None:
+        seqlens = headline_seqlens()
+    T, nb, max_len = sum(seqlens), len(seqlens), max(seqlens)
+    q, k, v, dout, cu = make_inputs(seqlens, H, D, chunk, 1000 + len(seqlens), dev)
+    q.requires_grad_(backward), k.requires_grad_(backward), v.requires_grad_(backward)
+
+    def step():
+        out = flash_moba.flash_moba_varlen_func(q, k, v, cu, cu, max_len, max_len, chunk, topk, causal=True)
+        if backward:
+            q.grad = k.grad = v.grad = None
+            out.backward(dout)
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- algorithmic work -------------------------------------------------------------
+    with torch.no_grad():
+        co, cn, ind = flash_moba.flash_topk_varlen_func(q, k, cu, cu, max_len, max_len, topk, chunk, causal=True)
+    pairs = count_pairs(seqlens, cn, chunk, H)
+    fwd_flops = 4.0 * D * pairs
+    bwd_flops = 2.5 * fwd_flops
+    step_flops = fwd_flops + (bwd_flops if backward else 0.0)
+    sumC = sum((L + chunk - 1) // chunk for L in seqlens)
+    maxC = (max_len + chunk - 1) // chunk
+    pool_bytes = (T + sumC) * H * D * 2
+    gate_bytes = T * H * D * 2 + sumC * H * D * 2 + T * H * topk * 4 + nb * H * maxC * 12
+
+    # ---- per-stage times (events on the launch stream) ----------------------------------
+    it = max(5, args.steps)
+    lg_m = flash_moba.flash_moba_interface.decide_lg_block_m(topk, chunk, max_len, True)
+    scale = D ** -0.5
+    qd, kd, vd = q.detach(), k.detach(), v.detach()
+    km, cu_km, _ = mean_pool_nosync(kd, cu, max_len, chunk)
+    t_pool = time_events(lambda: mean_pool_nosync(kd, cu, max_len, chunk), it)
+    t_gate = time_events(lambda: hip.moba_fused_topk(qd, km, cu, cu, cu_km, max_len, max_len, topk, chunk, True, return_raw=False), it)
+    fwd = lambda: hip.moba_varlen_fwd(qd, kd, vd, None, co, cn, ind, cu, cu, None, None, None, max_len, max_len, 0.0, scale,
+                                      False, True, 0.0, False, lg_m, chunk, None)
+    out, lse, _, _ = fwd()
+    t_fwd = time_events(fwd, it)
+    stages = {
+        "mean_pool": {"ms": t_pool, "GBps": pool_bytes / t_pool / 1e6, "frac_hbm": pool_bytes / t_pool / 1e6 / PEAK_HBM_GBS},
+        "topk_csc": {"ms": t_gate, "GBps": gate_bytes / t_gate / 1e6, "frac_hbm": gate_bytes / t_gate / 1e6 / PEAK_HBM_GBS},
+        "attn_fwd": {"ms": t_fwd, "TFLOPs": fwd_flops / t_fwd / 1e9, "frac_mfma": fwd_flops / t_fwd / 1e9 / PEAK_BF16_TFLOPS},
+    }
+    kernels = {"attn_fwd_kernel": (t_fwd, fwd_flops, "mfma")}
+    if backward:
+        dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
+        phase_ms = {}
+
+        def run_phases(run):
+            run(7)  # make the buffers consistent first
+            for name, mask in (("prep", 1), ("main", 2), ("convert", 4)):
+                phase_ms[name] = time_events(lambda: run(mask), it)
+
+        hip.moba_varlen_bwd(dout, qd, kd, vd, out, lse, dq, dk, dv, co, cn, ind, cu, cu, None, max_len, max_len, 0.0, scale,
+                            False, True, 0.0, False, lg_m, chunk, None, None, _phases=run_phases)
+        t_bwd = time_events(lambda: hip.moba_varlen_bwd(dout, qd, kd, vd, out, lse, dq, dk, dv, co, cn, ind, cu, cu, None, max_len,
+                                                        max_len, 0.0, scale, False, True, 0.0, False, lg_m, chunk, None, None), it)
+        stages["attn_bwd"] = {"ms": t_bwd, "TFLOPs": bwd_flops / t_bwd / 1e9, "frac_mfma": bwd_flops / t_bwd / 1e9 / PEAK_BF16_TFLOPS,
+                              "phases_ms": phase_ms}
+        kernels["attn_bwd_kernel"] = (phase_ms["main"], bwd_flops, "mfma")
+    # sort alone, on the CSC the gating produced (already sorted input; same traffic)
+    t_sort = time_events(lambda: torch.ops.flash_moba._varlen_sort(co, cn, ind), it)
+    sort_bytes = 2 * int(cn.sum().item()) * 4 + 2 * cn.numel() * 8
+    stages["varlen_sort"] = {"ms": t_sort, "GBps": sort_bytes / t_sort / 1e6, "frac_hbm": sort_bytes / t_sort / 1e6 / PEAK_HBM_GBS}
+
+    # ---- roofline of the dominant kernel ---------------------------------------------------
+    dom = max(kernels, key=lambda n: kernels[n][0])
+    d_ms, d_flops, _ = kernels[dom]
+    roofline = {"kernel": dom, "bound": "mfma", "achieved": d_flops / d_ms / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS, "traffic": None, "avg_launch_ms": d_ms,
+                "flops_per_launch": d_flops}
+
+    result = {
+        "metric": "moba_fwd_bwd_effective_sparse_tflops" if backward else "moba_fwd_effective_sparse_tflops",
+        "value": step_flops / ms_per_step / 1e9,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{args.config}: varlen packed batch, {nb} sequences totalling {T} tokens "
+                               f"(lengths {seqlens}), causal, {H} heads, head_dim {D}, chunk {chunk}, top-k {topk}, "
+                               + ("fwd+bwd" if backward else "fwd only"),
+                   "tokens": T, "heads": H, "head_dim": D, "chunk": chunk, "topk": topk},
+        "frac_of_bf16_mfma_peak": step_flops / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
+        "pairs": pairs,
+        "flops_per_step": step_flops,
+        "topk_csc_ms": t_gate,
+        "stages": stages,
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(qd, kd, vd, cu, seqlens, chunk, topk)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -373,14 +373,18 @@ static int launch_bwd(const fmoba_attn_bwd_args &a, float *dq_accum, hipStream_t
 }
 
 template <typename T>
-static int run_bwd(const fmoba_attn_bwd_args &a, float *dq_accum, hipStream_t s) {
-  int lpr = 1;
-  while (lpr * 8 < a.head_dim) lpr <<= 1;
-  const int rows_per_block = 256 / lpr;
-  hipLaunchKernelGGL(bwd_prep_kernel<T>, dim3(ceil_div(a.max_seqlen_q, rows_per_block), a.heads, a.batch), dim3(256), 0, s, a, dq_accum, lpr);
-  int rc = a.head_dim <= 64 ? launch_bwd<T, 64>(a, dq_accum, s) : launch_bwd<T, 128>(a, dq_accum, s);
-  if (rc) return rc;
-  hipLaunchKernelGGL(bwd_convert_kernel<T>, dim3(2048), dim3(256), 0, s, a, (const float *)dq_accum);
+static int run_bwd(const fmoba_attn_bwd_args &a, float *dq_accum, int phases, hipStream_t s) {
+  if (phases & FMOBA_BWD_PREP) {
+    int lpr = 1;
+    while (lpr * 8 < a.head_dim) lpr <<= 1;
+    const int rows_per_block = 256 / lpr;
+    hipLaunchKernelGGL(bwd_prep_kernel<T>, dim3(ceil_div(a.max_seqlen_q, rows_per_block), a.heads, a.batch), dim3(256), 0, s, a, dq_accum, lpr);
+  }
+  if (phases & FMOBA_BWD_MAIN) {
+    int rc = a.head_dim <= 64 ? launch_bwd<T, 64>(a, dq_accum, s) : launch_bwd<T, 128>(a, dq_accum, s);
+    if (rc) return rc;
+  }
+  if (phases & FMOBA_BWD_CONVERT) hipLaunchKernelGGL(bwd_convert_kernel<T>, dim3(2048), dim3(256), 0, s, a, (const float *)dq_accum);
   return 0;
 }
 
@@ -391,9 +395,12 @@ extern "C" size_t fmoba_attn_bwd_workspace_bytes(int32_t total_q, int32_t heads,
   return (size_t)total_q * heads * head_dim * 4 + 256;
 }
 
-extern "C" int fmoba_attn_bwd(const fmoba_attn_bwd_args *a, void *stream) {
+extern "C" int fmoba_attn_bwd(const fmoba_attn_bwd_args *a, void *stream) { return fmoba_attn_bwd_phases(a, 7, stream); }
+
+extern "C" int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phases, void *stream) {
   using namespace fmoba;
   FMOBA_REQUIRE(a != nullptr, "attn_bwd: null args");
+  FMOBA_REQUIRE(phases > 0 && phases <= 7, "attn_bwd: phases must be a mask of bits 1, 2, 4");
   FMOBA_REQUIRE(a->dtype == FMOBA_DTYPE_F16 || a->dtype == FMOBA_DTYPE_BF16, "FlashMoBA only support fp16 and bf16 data type");
   FMOBA_REQUIRE(a->batch > 0, "batch size must be positive");
   FMOBA_REQUIRE(a->head_dim > 0 && a->head_dim % 8 == 0, "head_size should be a multiple of 8");
@@ -430,7 +437,8 @@ extern "C" int fmoba_attn_bwd(const fmoba_attn_bwd_args *a, void *stream) {
   FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= fmoba_attn_bwd_workspace_bytes(a->total_q, a->heads, a->head_dim),
                 "attn_bwd: workspace too small");
   float *dq_accum = reinterpret_cast<float *>(((uintptr_t)a->workspace + 255) & ~(uintptr_t)255);
-  hipLaunchKernelGGL(zero_f32_kernel, dim3(256), dim3(256), 0, s, a->softmax_d, (int64_t)a->heads * ((int64_t)a->total_q + 128 * (int64_t)a->batch));
+  if (phases & FMOBA_BWD_PREP)
+    hipLaunchKernelGGL(zero_f32_kernel, dim3(256), dim3(256), 0, s, a->softmax_d, (int64_t)a->heads * ((int64_t)a->total_q + 128 * (int64_t)a->batch));
   if (a->total_k == 0 || a->max_seqlen_k == 0 || a->max_cols == 0) {
     // no keys: dq = 0
     hipLaunchKernelGGL(zero_rows_kernel, dim3(1024), dim3(256), 0, s, a->dq, (int64_t)a->total_q, a->dq_row_stride, a->heads, a->dq_head_stride, a->head_dim);
@@ -438,7 +446,7 @@ extern "C" int fmoba_attn_bwd(const fmoba_attn_bwd_args *a, void *stream) {
     return 0;
   }
   FMOBA_REQUIRE(a->k && a->v && a->col_offsets && a->col_nnz && a->row_indices, "attn_bwd: null k/v/CSC pointer");
-  int rc = a->dtype == FMOBA_DTYPE_BF16 ? run_bwd<bf16_t>(*a, dq_accum, s) : run_bwd<f16_t>(*a, dq_accum, s);
+  int rc = a->dtype == FMOBA_DTYPE_BF16 ? run_bwd<bf16_t>(*a, dq_accum, phases, s) : run_bwd<f16_t>(*a, dq_accum, phases, s);
   if (rc) return rc;
   FMOBA_LAUNCH_CHECK("attn_bwd");
   return 0;

@@ -436,8 +436,8 @@ extern "C" int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream) {
   FMOBA_REQUIRE(a->chunk > 0, "moba_chunk_size must be positive");
   FMOBA_REQUIRE(a->total_q >= 0 && a->max_seqlen_q >= 0 && a->max_seqlen_k >= 0, "negative size");
   FMOBA_REQUIRE(a->cu_seqlens_q && a->cu_seqlens_k && a->cu_seqlens_km, "fused_topk: null cu_seqlens pointer");
-  FMOBA_REQUIRE(a->col_offsets && a->col_nnz && (a->flat_indices || (int64_t)a->total_q * a->heads * a->topk == 0),
-                "fused_topk: null output pointer");
+  FMOBA_REQUIRE((a->col_offsets && a->col_nnz) || a->max_seqlen_k == 0, "fused_topk: null col_offsets/col_nnz pointer");
+  FMOBA_REQUIRE(a->flat_indices || (int64_t)a->total_q * a->heads * a->topk == 0, "fused_topk: null flat_indices pointer");
   FMOBA_REQUIRE((a->raw_indices == nullptr) == (a->raw_values == nullptr), "fused_topk: raw_indices and raw_values go together");
   hipStream_t s = (hipStream_t)stream;
   const int max_cols = ceil_div(a->max_seqlen_k, a->chunk);

@@ -89,6 +89,7 @@ EXPORTS = {
     "fmoba_attn_fwd": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp]),
     "fmoba_attn_bwd_workspace_bytes": (c_sz, [c_i32, c_i32, c_i32]),
     "fmoba_attn_bwd": (c_i32, [ctypes.POINTER(AttnBwdArgs), c_vp]),
+    "fmoba_attn_bwd_phases": (c_i32, [ctypes.POINTER(AttnBwdArgs), c_i32, c_vp]),
 }
 
 _lib = None
@@ -337,7 +338,7 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
 def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_offsets, moba_col_nnz, moba_row_indices,
                     cu_seqlens_q, cu_seqlens_k, alibi_slopes, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                     zero_tensors, is_causal, softcap, deterministic, m_lg_block_dim, n_lg_block_dim, gen=None,
-                    rng_state=None):
+                    rng_state=None, _phases=None):
     """Returns [dq, dk, dv, softmax_d (H, total_q + 128*batch) fp32]."""
     dtype = q.dtype
     _require(dtype in (torch.float16, torch.bfloat16), "FlashMoBA only support fp16 and bf16 data type")
@@ -405,7 +406,10 @@ def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_off
                         q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                         out.stride(0), out.stride(1), dout.stride(0), dout.stride(1),
                         dq.stride(0), dq.stride(1), dk_e.stride(0), dk_e.stride(1), dv_e.stride(0), dv_e.stride(1))
-        _check(lib.fmoba_attn_bwd(ctypes.byref(a), _stream()))
+        if _phases is None:
+            _check(lib.fmoba_attn_bwd(ctypes.byref(a), _stream()))
+        else:  # measurement hook: callable(run) receives run(mask) launching the chosen phases
+            _phases(lambda mask: _check(lib.fmoba_attn_bwd_phases(ctypes.byref(a), mask, _stream())))
         if heads_k != heads:
             grp = heads // heads_k
             torch.sum(dk_e.view(total_k, heads_k, grp, d), dim=2, out=dk)

@@ -160,6 +160,14 @@ typedef struct {
 } fmoba_attn_bwd_args;
 size_t fmoba_attn_bwd_workspace_bytes(int32_t total_q, int32_t heads, int32_t head_dim);
 int fmoba_attn_bwd(const fmoba_attn_bwd_args *a, void *stream);
+/* The same call split into its three launches so that each can be timed on its own:
+ * phases is a bit mask, 1 = dot(dO, O) + clear of the dQ accumulator
+ * (flash_bwd_launch_template.h:70-74), 2 = the dK/dV/dQ kernel (:76-96), 4 = dQ conversion
+ * (:98-104).  fmoba_attn_bwd(a, s) == fmoba_attn_bwd_phases(a, 7, s). */
+#define FMOBA_BWD_PREP 1
+#define FMOBA_BWD_MAIN 2
+#define FMOBA_BWD_CONVERT 4
+int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phases, void *stream);
 
 #ifdef __cplusplus
 }

@@ -128,7 +128,6 @@ def _check_gating(fm, q, k, cuq, cuk, chunk, topk, causal, integer=False):
                 ok_rows = unamb[int(cuq_np[b]):int(cuq_np[b + 1]), h].numpy()
                 assert (got[ok_rows] == ref[ok_rows]).all()
                 assert (got.sum(1) == ref.sum(1)).all()       # same number of chunks everywhere
-        assert n_amb < 0.005 * unamb.numel() + 8
     # ordered per-row lists (auxiliary outputs): same sets as the CSC, descending scores
     kr = (topk + 15) // 16 * 16
     assert indices.shape == (q.shape[0], H, kr) and values.shape == indices.shape
