@@ -113,6 +113,27 @@ __device__ __forceinline__ f32x16 mfma32<f16_t>(const Pack8 &a, const Pack8 &b, 
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c, 0, 0, 0);
 }
 
+// MFMA 16x16x32 (gfx950).  Operand layout, lane l, g = l / 16:
+//   A (16 x 32): lane holds A[l % 16][g*8 .. g*8+7]
+//   B (32 x 16): lane holds B[g*8 .. g*8+7][l % 16]
+//   C (16 x 16): lane holds C[4*g + i][l % 16], i = 0..3
+template <typename T>
+__device__ __forceinline__ f32x4 mfma16(const Pack8 &a, const Pack8 &b, f32x4 c);
+template <>
+__device__ __forceinline__ f32x4 mfma16<bf16_t>(const Pack8 &a, const Pack8 &b, f32x4 c) {
+  bf16x8 av, bv;
+  __builtin_memcpy(&av, &a, 16);
+  __builtin_memcpy(&bv, &b, 16);
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 mfma16<f16_t>(const Pack8 &a, const Pack8 &b, f32x4 c) {
+  f16x8 av, bv;
+  __builtin_memcpy(&av, &a, 16);
+  __builtin_memcpy(&bv, &b, 16);
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, c, 0, 0, 0);
+}
+
 // Row of a 32x32 accumulator tile that register i of this lane holds.
 __device__ __forceinline__ int acc_row(int i, int hh) { return 8 * (i >> 2) + 4 * hh + (i & 3); }
 
@@ -168,8 +189,63 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-__device__ __forceinline__ float shfl_xor32_f(float v) { return __shfl_xor(v, 32, 64); }
-__device__ __forceinline__ int shfl_xor32_i(int v) { return __shfl_xor(v, 32, 64); }
+// Cross-half / cross-row exchanges on the VALU (gfx950 v_permlane32_swap / v_permlane16_swap)
+// instead of the LDS crossbar.  swap32(x): {x of lanes l%32, x of lanes 32 + l%32};
+// swap16(x): {x of the even 16-lane row of this row pair, x of the odd row}.
+struct UPair {
+  uint32_t a, b;
+};
+__device__ __forceinline__ UPair swap32(uint32_t x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+  return UPair{(uint32_t)r[0], (uint32_t)r[1]};
+#else
+  return UPair{x, x};
+#endif
+}
+__device__ __forceinline__ UPair swap16(uint32_t x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+  return UPair{(uint32_t)r[0], (uint32_t)r[1]};
+#else
+  return UPair{x, x};
+#endif
+}
+// value of the partner lane (l ^ 32)
+__device__ __forceinline__ float shfl_xor32_f(float v) {
+  const UPair p = swap32(__float_as_uint(v));
+  return __uint_as_float((threadIdx.x & 32) ? p.a : p.b);
+}
+__device__ __forceinline__ int shfl_xor32_i(int v) {
+  const UPair p = swap32((uint32_t)v);
+  return (int)((threadIdx.x & 32) ? p.a : p.b);
+}
+// reductions over the two halves of a wave (lanes l and l ^ 32), result in both lanes
+__device__ __forceinline__ int sum_xor32_i(int v) {
+  const UPair p = swap32((uint32_t)v);
+  return (int)(p.a + p.b);
+}
+__device__ __forceinline__ float max_xor32_f(float v) {
+  const UPair p = swap32(__float_as_uint(v));
+  return fmaxf(__uint_as_float(p.a), __uint_as_float(p.b));
+}
+__device__ __forceinline__ float min_xor32_f(float v) {
+  const UPair p = swap32(__float_as_uint(v));
+  return fminf(__uint_as_float(p.a), __uint_as_float(p.b));
+}
+__device__ __forceinline__ float sum_xor32_f(float v) {
+  const UPair p = swap32(__float_as_uint(v));
+  return __uint_as_float(p.a) + __uint_as_float(p.b);
+}
+// reductions over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48), result everywhere
+__device__ __forceinline__ float max_rows4_f(float v) {
+  const UPair p = swap16(__float_as_uint(v));
+  return max_xor32_f(fmaxf(__uint_as_float(p.a), __uint_as_float(p.b)));
+}
+__device__ __forceinline__ float sum_rows4_f(float v) {
+  const UPair p = swap16(__float_as_uint(v));
+  return sum_xor32_f(__uint_as_float(p.a) + __uint_as_float(p.b));
+}
 
 // Monotone map float -> uint32 (larger float => larger key); every non-NaN value,
 // including -inf, maps to a key >= 0x007fffff > 0.

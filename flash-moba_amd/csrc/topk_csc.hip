@@ -85,14 +85,17 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(TopkParams p) {
   }
   __syncthreads();
 
-  // scores: lane (query l%32) gets chunk t*32 + acc_row(i, hh) in register i of tile t
-  uint32_t key[NT][16];
+  // scores: lane (query l%32) gets chunk t*32 + acc_row(i, hh) in register i of tile t;
+  // chunks that are not candidates of the row hold -inf
+  float sc[NT][16];
   const int rp = r + off;
   int nc;  // number of candidate chunks of this row: chunks strictly before its own chunk
   if (a.is_causal)
     nc = (valid && rp >= 0) ? min(rp / B, Cb) : 0;
   else
     nc = valid ? Cb : 0;
+  nc = min(nc, nsc);
+  float vmin = INFINITY, vmax = -INFINITY;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     if (t < n_tiles) {
@@ -107,68 +110,109 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(TopkParams p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int c = t * 32 + acc_row(i, hh);
-        key[t][i] = (c < nc) ? float_order_key(acc[i]) : 0u;
+        const bool cand = c < nc;
+        const float x = acc[i];
+        sc[t][i] = cand ? x : -INFINITY;
+        vmin = fminf(vmin, cand ? x : INFINITY);
+        vmax = fmaxf(vmax, sc[t][i]);
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) key[t][i] = 0u;
+      for (int i = 0; i < 16; ++i) sc[t][i] = -INFINITY;
     }
   }
+  vmin = min_xor32_f(vmin);
+  vmax = max_xor32_f(vmax);
 
-  // K' = number of scored chunks to keep (the own chunk takes one slot in causal mode)
+  // K' = number of scored chunks to keep (the own chunk takes one slot in causal mode).
+  // A row keeps every candidate x with x > tau, plus, among the candidates equal to tau_eq,
+  // those with chunk index >= iota.  tau is found by bisection between the row's smallest
+  // and largest score and the search stops as soon as exactly K' scores lie above the probe.
+  // The bracket is kept as order-preserving integer keys (lo_k, hi_k]; the first probes
+  // bisect the VALUE range (few steps for ordinary score distributions), later ones the key
+  // range (at most 32 more steps whatever the values).  If the bracket closes first, the
+  // scores inside it are all equal and tie across the cut: the highest chunk indices win.
   const int kp = a.is_causal ? a.topk - 1 : a.topk;
   const bool need = (nc > kp) && (kp > 0);
-  uint32_t tau = 1u;    // candidates have key >= 1
-  uint32_t iota = 0u;   // among keys equal to tau keep chunks >= iota
-  if (__any(need)) {
-    uint32_t t_acc = 0u;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t trial = t_acc | (1u << bit);
+  float tau = -INFINITY;    // nc <= K': every candidate with a score above -inf
+  float tau_eq = INFINITY;  // no tie group by default
+  int n_eq = 0;
+  uint32_t iota = 0u;
+  {
+    uint32_t lo_k = float_order_key(vmin) - 1u;  // count(x > lo) = nc > K'
+    uint32_t hi_k = float_order_key(vmax);       // count(x > hi) = 0  < K'
+    int c_hi = 0;
+    bool open = need;
+    for (int iter = 0;; ++iter) {
+      if (open && hi_k - lo_k <= 1u) {
+        // nothing representable strictly inside: every score in (lo, hi] equals hi
+        tau = order_key_float(hi_k);
+        if (tau != -INFINITY) {
+          tau_eq = tau;
+          n_eq = kp - c_hi;
+        }
+        open = false;
+      }
+      if (!__any(open)) break;
+      uint32_t pk = lo_k + ((hi_k - lo_k) >> 1);
+      if (iter < 12) {
+        const float mf = 0.5f * order_key_float(lo_k + 1u) + 0.5f * order_key_float(hi_k);
+        const uint32_t mk = float_order_key(mf);
+        if (mk > lo_k && mk < hi_k) pk = mk;
+      }
+      const float probe = order_key_float(pk);
       int cnt = 0;
 #pragma unroll
       for (int t = 0; t < NT; ++t)
         if (t < n_tiles) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) cnt += (key[t][i] >= trial) ? 1 : 0;
+          for (int i = 0; i < 16; ++i) cnt += (sc[t][i] > probe) ? 1 : 0;
         }
-      cnt += shfl_xor32_i(cnt);
-      if (cnt >= kp) t_acc = trial;
+      cnt = sum_xor32_i(cnt);
+      if (open) {
+        if (cnt == kp) {
+          tau = probe;
+          open = false;
+        } else if (cnt > kp) {
+          lo_k = pk;
+        } else {
+          hi_k = pk;
+          c_hi = cnt;
+        }
+      }
     }
-    if (need) tau = t_acc;
-    // ties at the threshold: keep the (kp - #greater) highest chunk indices
-    int cgt = 0, ceq = 0;
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-      if (t < n_tiles) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          cgt += (key[t][i] > tau) ? 1 : 0;
-          ceq += (key[t][i] == tau) ? 1 : 0;
-        }
-      }
-    cgt += shfl_xor32_i(cgt);
-    ceq += shfl_xor32_i(ceq);
-    const int needk = kp - cgt;
-    const bool tie = need && (ceq > needk);
+    // a tie group keeps its n_eq highest chunk indices
+    const bool tie = n_eq > 0;
     if (__any(tie)) {
-      uint32_t i_acc = 0u;
-      constexpr int IB = (NT * 32 <= 64) ? 6 : (NT * 32 <= 128 ? 7 : 8);
-      for (int bit = IB - 1; bit >= 0; --bit) {
-        const uint32_t trial = i_acc | (1u << bit);
-        int cnt = 0;
+      int ceq = 0;
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          if (t < n_tiles) {
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
-              cnt += (key[t][i] == tau && c >= trial) ? 1 : 0;
+          for (int i = 0; i < 16; ++i) ceq += (sc[t][i] == tau_eq) ? 1 : 0;
+        }
+      ceq = sum_xor32_i(ceq);
+      const bool split = tie && ceq > n_eq;
+      if (__any(split)) {
+        uint32_t i_acc = 0u;
+        constexpr int IB = (NT * 32 <= 64) ? 6 : (NT * 32 <= 128 ? 7 : 8);
+        for (int bit = IB - 1; bit >= 0; --bit) {
+          const uint32_t trial = i_acc | (1u << bit);
+          int cnt = 0;
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            if (t < n_tiles) {
+#pragma unroll
+              for (int i = 0; i < 16; ++i) {
+                const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
+                cnt += (sc[t][i] == tau_eq && c >= trial) ? 1 : 0;
+              }
             }
-          }
-        cnt += shfl_xor32_i(cnt);
-        if (cnt >= needk) i_acc = trial;
+          cnt = sum_xor32_i(cnt);
+          if (cnt >= n_eq) i_acc = trial;
+        }
+        if (split) iota = i_acc;
       }
-      if (tie) iota = i_acc;
     }
   }
 
@@ -185,12 +229,15 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(TopkParams p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
-          const uint32_t k = key[t][i];
-          const bool s = (k > tau) || (k == tau && c >= iota);
-          w |= (s && k != 0u) ? (1u << ((8 * (i >> 2) + (i & 3)) + 4 * hh)) : 0u;
+          const float x = sc[t][i];
+          const bool s = (x > tau) || (x == tau_eq && c >= iota);
+          w |= s ? (1u << ((8 * (i >> 2) + (i & 3)) + 4 * hh)) : 0u;
         }
       }
-      w |= (uint32_t)shfl_xor32_i((int)w);
+      {
+        const UPair wp = swap32(w);
+        w = wp.a | wp.b;
+      }
       if (has_self && (pself >> 5) == t) w |= 1u << (pself & 31);
       if (!valid) w = 0u;
       if (valid && hh == 0) selp[(int64_t)t * a.total_q] = w;
