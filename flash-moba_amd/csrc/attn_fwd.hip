@@ -218,17 +218,22 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(fmoba_attn_fwd_args a, in
     Pack8 qf[KS4];
 #pragma unroll
     for (int ks = 0; ks < KS4; ++ks) qf[ks] = *reinterpret_cast<const Pack8 *>(sQ + rid * LDQ + (g * KS4 + ks) * 8);
-    // S^T: register i of key tile kt holds key key0 + 16*kt + 4*g + i for this lane's row
+    // S^T: register i of key tile kt holds key key0 + 16*kt + 4*g + i for this lane's row.
+    // All K fragments are fetched from LDS before the first MFMA so that the LDS round trips
+    // overlap instead of preceding each MFMA.
+    Pack8 kf[KS4][4];
+#pragma unroll
+    for (int ks = 0; ks < KS4; ++ks)
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+        kf[ks][kt] = *reinterpret_cast<const Pack8 *>(sK + (kt * 16 + l16) * LDQ + (g * KS4 + ks) * 8);
     f32x4 s[4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS4; ++ks) {
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
-        const Pack8 af = *reinterpret_cast<const Pack8 *>(sK + (kt * 16 + l16) * LDQ + (g * KS4 + ks) * 8);
-        s[kt] = mfma16<T>(af, qf[ks], s[kt]);
-      }
+      for (int kt = 0; kt < 4; ++kt) s[kt] = mfma16<T>(kf[ks][kt], qf[ks], s[kt]);
     }
     const int rowpos = m0 + rid + off;
     float mloc = -INFINITY;
@@ -281,14 +286,14 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(fmoba_attn_fwd_args a, in
 #pragma unroll
     for (int d2 = 0; d2 < NDT / 2; ++d2) {
       const int dt = (wave - 2) * (NDT / 2) + d2;
+      Pack8 vf[4];
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) vf[ks] = tr_frag8(sV, LDQ, 16 * ks + 8 * hh, 16 * ks + 8 * hh + 4, dt * 32, lane);
       f32x16 o;
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[i] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const Pack8 vf = tr_frag8(sV, LDQ, 16 * ks + 8 * hh, 16 * ks + 8 * hh + 4, dt * 32, lane);
-        o = mfma32<T>(vf, pf[ks], o);
-      }
+      for (int ks = 0; ks < 4; ++ks) o = mfma32<T>(vf[ks], pf[ks], o);
       if (rid >= 0) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {

@@ -44,3 +44,39 @@ def assert_close(name, got, ref, atol, rtol):
     tol = atol + rtol * ref.abs()
     bad = err > tol
     assert not bad.any(), f"{name}: {int(bad.sum())} / {bad.numel()} elements out of tolerance, max err {err.max().item():.4e}"
+
+
+def dense_ref_one_head(q, k, v, dout, km, chunk, topk, row_block=2048):
+    """fp32 dense-masked MoBA of ONE (sequence, head) evaluated with plain torch ops on the
+    tensors' device (test reference for sizes the CPU oracle cannot finish in seconds).
+    q, k, v, dout: (L, D); km: (C, D) chunk means in the storage dtype.  Returns out, dq, dk, dv
+    (fp32) and the boolean (L, C) selection."""
+    L, D = q.shape
+    C = km.shape[0]
+    dev = q.device
+    qf = q.float().requires_grad_(True)
+    kf = k.float().requires_grad_(True)
+    vf = v.float().requires_grad_(True)
+    gate = q.float() @ km.float().T
+    r = torch.arange(L, device=dev)
+    c = torch.arange(C, device=dev)
+    cand = ((c[None] + 1) * chunk - 1) < r[:, None]
+    gate = gate.masked_fill(~cand, float("-inf"))
+    own = c[None] == (r // chunk)[:, None]
+    gate = gate.masked_fill(own, float("inf"))
+    sv, si = torch.sort(gate, dim=-1, descending=False, stable=True)
+    kk = min(topk, C)
+    tv, ti = sv[:, C - kk:], si[:, C - kk:]
+    sel = torch.zeros((L, C), dtype=torch.bool, device=dev)
+    sel.scatter_(1, ti, tv > float("-inf"))
+    outs = []
+    scale = D ** -0.5
+    for r0 in range(0, L, row_block):
+        r1 = min(L, r0 + row_block)
+        m = sel[r0:r1].repeat_interleave(chunk, dim=1)[:, :L] & (torch.arange(L, device=dev)[None] <= r[r0:r1, None])
+        s = (qf[r0:r1] @ kf.T) * scale
+        s = s.masked_fill(~m, float("-inf"))
+        outs.append(torch.softmax(s, -1) @ vf)
+    out = torch.cat(outs)
+    dq, dk, dv = torch.autograd.grad(out, (qf, kf, vf), dout.float())
+    return out.detach(), dq, dk, dv, sel, gate
