@@ -97,13 +97,14 @@ def time_events(fn, iters, warmup=1):
 
 def cpu_baseline(q, k, v, cu, seqlens, chunk, topk, budget_s=12.0):
     """Times the CPU restatement of the reference's PyTorch MoBA path (chunk means -> gate ->
-    top-k -> block mask -> dense-masked softmax attention, fp32) on (sequence 0, heads 0..n)
-    of the same inputs, adding heads until ~budget_s of CPU work has been done."""
+    top-k -> block mask -> dense-masked softmax attention, fp32) on (longest sequence,
+    heads 0..n) of the same inputs, adding heads until ~budget_s of CPU work has been done."""
     from oracle import moba_oracle as O  # checker only: never on the product path
 
     torch.set_num_threads(os.cpu_count())
-    L = seqlens[0]
-    qs, ks, vs = (t[:L].float().cpu() for t in (q, k, v))
+    b = max(range(len(seqlens)), key=lambda i: seqlens[i])  # the longest sequence of the batch
+    L, start = seqlens[b], sum(seqlens[:b])
+    qs, ks, vs = (t[start:start + L].float().cpu() for t in (q, k, v))
     cu0 = torch.tensor([0, L], dtype=torch.int32)
     H, D = q.shape[1], q.shape[2]
     t0 = time.perf_counter()
@@ -122,7 +123,7 @@ def cpu_baseline(q, k, v, cu, seqlens, chunk, topk, budget_s=12.0):
         "unit": "TFLOP/s",
         "cores": os.cpu_count(),
         "kind": "port",
-        "sample": f"forward only, fp32, sequence 0 ({L} tokens) x {heads} of {H} heads, row-blocked dense-masked "
+        "sample": f"forward only, fp32, sequence {b} ({L} tokens, the longest) x {heads} of {H} heads, row-blocked dense-masked "
                   f"attention; {dt:.1f} s of CPU time; effective sparse FLOPs / time",
         "seconds": dt,
     }
@@ -208,7 +209,7 @@ def main():
 
         def run_phases(run):
             run(7)  # make the buffers consistent first
-            for name, mask in (("prep", 1), ("main", 2), ("convert", 4)):
+            for name, mask in (("prep", 1), ("dkdv", 2), ("dq", 4)):
                 phase_ms[name] = time_events(lambda: run(mask), it)
 
         hip.moba_varlen_bwd(dout, qd, kd, vd, out, lse, dq, dk, dv, co, cn, ind, cu, cu, None, max_len, max_len, 0.0, scale,
@@ -217,7 +218,9 @@ def main():
                                                         max_len, 0.0, scale, False, True, 0.0, False, lg_m, chunk, None, None), it)
         stages["attn_bwd"] = {"ms": t_bwd, "TFLOPs": bwd_flops / t_bwd / 1e9, "frac_mfma": bwd_flops / t_bwd / 1e9 / PEAK_BF16_TFLOPS,
                               "phases_ms": phase_ms}
-        kernels["attn_bwd_kernel"] = (phase_ms["main"], bwd_flops, "mfma")
+        # the dK/dV kernel runs four of the five backward GEMMs (S, dP, dV, dK), the dQ kernel the fifth
+        kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 8.0 * D * pairs, "mfma")
+        kernels["attn_bwd_dq_kernel"] = (phase_ms["dq"], 2.0 * D * pairs, "mfma")
     # sort alone, on the CSC the gating produced (already sorted input; same traffic)
     t_sort = time_events(lambda: torch.ops.flash_moba._varlen_sort(co, cn, ind), it)
     sort_bytes = 2 * int(cn.sum().item()) * 4 + 2 * cn.numel() * 8

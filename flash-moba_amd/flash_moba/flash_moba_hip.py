@@ -65,7 +65,7 @@ class AttnBwdArgs(ctypes.Structure):
                 ("dq", c_vp), ("dk", c_vp), ("dv", c_vp), ("softmax_d", c_vp),
                 ("col_offsets", c_vp), ("col_nnz", c_vp), ("row_indices", c_vp),
                 ("cu_seqlens_q", c_vp), ("cu_seqlens_k", c_vp),
-                ("workspace", c_vp), ("workspace_bytes", c_sz),
+                ("workspace", c_vp), ("workspace_bytes", c_sz), ("num_row_indices", c_i64),
                 ("batch", c_i32), ("total_q", c_i32), ("total_k", c_i32), ("heads", c_i32), ("heads_k", c_i32),
                 ("head_dim", c_i32), ("max_seqlen_q", c_i32), ("max_seqlen_k", c_i32), ("max_cols", c_i32),
                 ("lg_block_m", c_i32), ("lg_block_n", c_i32), ("is_causal", c_i32), ("dtype", c_i32),
@@ -87,7 +87,7 @@ EXPORTS = {
     "fmoba_varlen_sort_workspace_bytes": (c_sz, [c_i64]),
     "fmoba_varlen_sort": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_sz, c_vp]),
     "fmoba_attn_fwd": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp]),
-    "fmoba_attn_bwd_workspace_bytes": (c_sz, [c_i32, c_i32, c_i32]),
+    "fmoba_attn_bwd_workspace_bytes": (c_sz, [c_i64, c_i32]),
     "fmoba_attn_bwd": (c_i32, [ctypes.POINTER(AttnBwdArgs), c_vp]),
     "fmoba_attn_bwd_phases": (c_i32, [ctypes.POINTER(AttnBwdArgs), c_i32, c_vp]),
 }
@@ -394,12 +394,13 @@ def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_off
         else:
             dk_e, dv_e = dk, dv
         lib = load_library()
-        ws_bytes = lib.fmoba_attn_bwd_workspace_bytes(total_q, heads, d)
+        n_idx = int(moba_row_indices.numel())
+        ws_bytes = lib.fmoba_attn_bwd_workspace_bytes(n_idx, int(n_lg_block_dim))
         ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
         a = AttnBwdArgs(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), softmax_lse.data_ptr(),
                         dq.data_ptr(), dk_e.data_ptr(), dv_e.data_ptr(), softmax_d.data_ptr(),
                         moba_col_offsets.data_ptr(), moba_col_nnz.data_ptr(), moba_row_indices.data_ptr(),
-                        cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ws.data_ptr(), ws_bytes,
+                        cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ws.data_ptr(), ws_bytes, n_idx,
                         batch, total_q, total_k, heads, heads_k, d, int(max_seqlen_q), int(max_seqlen_k), max_cols,
                         int(m_lg_block_dim), int(n_lg_block_dim), int(bool(is_causal)), _dt(q), int(bool(deterministic)),
                         float(softmax_scale),

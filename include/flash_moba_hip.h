@@ -134,7 +134,12 @@ int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream);
  *   GQA/MQA the caller sums groups of heads/heads_k (flash_moba_api.cpp:842-845).
  *   softmax_d (heads, total_q + 128*batch) fp32: row (b, r) of head h is stored at
  *   h*(total_q + 128*batch) + cu_q[b] + 128*b + r (flash_bwd_preprocess_kernel.h:86).
- *   workspace: fp32 dQ accumulator, fmoba_attn_bwd_workspace_bytes() bytes.
+ *   workspace: the dS tiles (16-bit, one row of lg_block_n entries per entry of
+ *   row_indices) that carry the result of the column-stationary dK/dV pass to the
+ *   row-stationary dQ pass; fmoba_attn_bwd_workspace_bytes() bytes, contents undefined on
+ *   entry and on return.  num_row_indices = number of int32 entries of row_indices
+ *   (every col_offsets[i] + col_nnz[i] must be <= it).  No atomics: results are
+ *   bitwise reproducible whatever `deterministic` says.
  * ---------------------------------------------------------------------------------- */
 typedef struct {
   const void *dout, *q, *k, *v, *out;
@@ -147,6 +152,7 @@ typedef struct {
   const int32_t *cu_seqlens_q, *cu_seqlens_k;
   void *workspace;
   size_t workspace_bytes;
+  int64_t num_row_indices;
   int32_t batch, total_q, total_k, heads, heads_k, head_dim;
   int32_t max_seqlen_q, max_seqlen_k, max_cols;
   int32_t lg_block_m, lg_block_n;
@@ -158,15 +164,16 @@ typedef struct {
   int64_t dq_row_stride, dq_head_stride, dk_row_stride, dk_head_stride;
   int64_t dv_row_stride, dv_head_stride;
 } fmoba_attn_bwd_args;
-size_t fmoba_attn_bwd_workspace_bytes(int32_t total_q, int32_t heads, int32_t head_dim);
+size_t fmoba_attn_bwd_workspace_bytes(int64_t num_row_indices, int32_t lg_block_n);
 int fmoba_attn_bwd(const fmoba_attn_bwd_args *a, void *stream);
 /* The same call split into its three launches so that each can be timed on its own:
- * phases is a bit mask, 1 = dot(dO, O) + clear of the dQ accumulator
- * (flash_bwd_launch_template.h:70-74), 2 = the dK/dV/dQ kernel (:76-96), 4 = dQ conversion
- * (:98-104).  fmoba_attn_bwd(a, s) == fmoba_attn_bwd_phases(a, 7, s). */
+ * phases is a bit mask, 1 = dot(dO, O) (flash_bwd_launch_template.h:70-74), 2 = the
+ * column-stationary dK/dV kernel, which also fills the workspace (:76-96), 4 = the
+ * row-stationary dQ kernel, which reads it (stands where the reference converts its fp32
+ * dQ accumulator, :98-104).  fmoba_attn_bwd(a, s) == fmoba_attn_bwd_phases(a, 7, s). */
 #define FMOBA_BWD_PREP 1
-#define FMOBA_BWD_MAIN 2
-#define FMOBA_BWD_CONVERT 4
+#define FMOBA_BWD_DKDV 2
+#define FMOBA_BWD_DQ 4
 int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phases, void *stream);
 
 #ifdef __cplusplus
