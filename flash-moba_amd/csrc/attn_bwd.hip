@@ -23,6 +23,7 @@
 #include "fmoba_common.h"
 
 #include <type_traits>
+#include <utility>
 
 namespace fmoba {
 
@@ -42,10 +43,20 @@ struct BwdSmem {
   static constexpr size_t oDelta = oLse + 2 * 32 * 4;
   static constexpr size_t oList = oDelta + 2 * 32 * 4;             // int[kListCap]
   static constexpr size_t mainBytes = oList + (size_t)kListCap * 4;
-  static constexpr int LDR = HD + 4;  // floats, output transpose buffer [64 keys][LDR]
-  static constexpr size_t redBytes = (size_t)64 * LDR * 4;
+  static constexpr int LDR = HD + 4;  // floats, output transpose buffer [2][64 keys][LDR]
+  static constexpr size_t redBytes = (size_t)2 * 64 * LDR * 4;
   static constexpr size_t bytes = mainBytes > redBytes ? mainBytes : redBytes;
 };
+
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{})
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 __device__ __forceinline__ int lower_bound_i32b(const int32_t *p, int n, int v) {
   int lo = 0, hi = n;
@@ -124,189 +135,92 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   }
   const int32_t *list = a.row_indices + lbase;
 
-  // K and V halves of this wave as MFMA B operands, for the whole list
-  Pack8 kfr[KS], vfr[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    kfr[ks] = *reinterpret_cast<const Pack8 *>(sK + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + ks) * 8);
-    vfr[ks] = *reinterpret_cast<const Pack8 *>(sV + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + ks) * 8);
-  }
-  f32x16 dv[NDT], dk[NDT];
-#pragma unroll
-  for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      dv[dt][i] = 0.f;
-      dk[dt][i] = 0.f;
-    }
-
   const uint16_t *qg = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)q0 * a.q_row_stride + (int64_t)h * a.q_head_stride;
   const uint16_t *dog = reinterpret_cast<const uint16_t *>(a.dout) + (int64_t)q0 * a.do_row_stride + (int64_t)h * a.do_head_stride;
   const float *lseg = a.softmax_lse + (int64_t)h * a.total_q + q0;
   const float *delg = a.softmax_d + (int64_t)h * ((int64_t)a.total_q + 128 * (int64_t)a.batch) + q0 + 128 * b;
 
-  // loader state: two-deep rings (compile-time parity) of the gathered rows of two rounds
-  Pack8 lq0[NV], lq1[NV], ld0[NV], ld1[NV];
-  int lrow0 = -1, lrow1 = -1;
-  float llse0 = INFINITY, llse1 = INFINITY, ldel0 = 0.f, ldel1 = 0.f;
-
-  for (int seg0 = start; seg0 < nnz; seg0 += kListCap) {
-    const int seg_len = min(kListCap, nnz - seg0);
+  auto fill_list = [&](int seg0, int seg_len) {
     __syncthreads();
     for (int i = tid; i < seg_len; i += 256) {
       int r = list[seg0 + i];
       sList[i] = (r >= 0 && r < Lq) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
     }
     __syncthreads();
-    const int ntile = (seg_len + 31) >> 5;
-    const int nround = (ntile + 1) >> 1;
+  };
+  float *red = reinterpret_cast<float *>(smem);  // [2][64 keys][LDR]: dV^T, dK^T on their way out
 
-    auto load_round = [&](auto par, int r) {
-      constexpr int P = decltype(par)::value;
-#pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        const int v = lt + 128 * i;
-        const int row = v / VPR, e = (v - row * VPR) * 8;  // row 0..63 over the two tiles of the round
-        const int j = r * 64 + row;
-        const int rid = j < seg_len ? sList[j] : -1;
-        Pack8 xq = zero_pack8(), xo = zero_pack8();
-        if (rid >= 0 && e < D) {
-          xq = ld_global16(qg + (int64_t)rid * a.q_row_stride + e);
-          xo = ld_global16(dog + (int64_t)rid * a.do_row_stride + e);
-        }
-        if constexpr (P == 0) {
-          lq0[i] = xq;
-          ld0[i] = xo;
-        } else {
-          lq1[i] = xq;
-          ld1[i] = xo;
-        }
-      }
-      if (lt < 64) {
-        const int j = r * 64 + lt;
-        const int rid = j < seg_len ? sList[j] : -1;
-        float xl = INFINITY, xd = 0.f;
-        if (rid >= 0) {
-          xl = lseg[rid];
-          xd = delg[rid];
-        }
-        if constexpr (P == 0) {
-          lrow0 = rid;
-          llse0 = xl;
-          ldel0 = xd;
-        } else {
-          lrow1 = rid;
-          llse1 = xl;
-          ldel1 = xd;
-        }
-      }
-    };
-    auto store_round = [&](auto par) {
-      constexpr int P = decltype(par)::value;
-#pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        const int v = lt + 128 * i;
-        const int row = v / VPR, e = (v - row * VPR) * 8;
-        *reinterpret_cast<Pack8 *>(sQ + row * LDQ + e) = P == 0 ? lq0[i] : lq1[i];
-        *reinterpret_cast<Pack8 *>(sdO + row * LDQ + e) = P == 0 ? ld0[i] : ld1[i];
-      }
-      if (lt < 64) {
-        sRow[lt] = P == 0 ? lrow0 : lrow1;
-        sLse[lt] = P == 0 ? llse0 : llse1;
-        sDelta[lt] = P == 0 ? ldel0 : ldel1;
-      }
-    };
+  // The two roles run separate code with the same barrier sequence, so that the loaders' rings and the
+  // compute waves' accumulators and operands do not add up in the register allocation.
+  if (is_loader) {
+    // loader state: two-deep rings (compile-time parity) of the gathered rows of two rounds
+    Pack8 lq0[NV], lq1[NV], ld0[NV], ld1[NV];
+    int lrow0 = -1, lrow1 = -1;
+    float llse0 = INFINITY, llse1 = INFINITY, ldel0 = 0.f, ldel1 = 0.f;
 
-    auto process_tile = [&](int tile, int ts) {
-      const uint16_t *tQ = sQ + ts * 32 * LDQ, *tdO = sdO + ts * 32 * LDQ;
-      Pack8 qa[KS], doa[KS];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        qa[ks] = *reinterpret_cast<const Pack8 *>(tQ + (lane & 31) * LDQ + (hh * KS + ks) * 8);
-        doa[ks] = *reinterpret_cast<const Pack8 *>(tdO + (lane & 31) * LDQ + (hh * KS + ks) * 8);
-      }
-      f32x16 s, dp;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s[i] = 0.f;
-        dp[i] = 0.f;
-      }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        s = mfma32<T>(qa[ks], kfr[ks], s);
-        dp = mfma32<T>(doa[ks], vfr[ks], dp);
-      }
-      // this lane's key; register i <-> gathered row acc_row(i, hh)
-      const int j = key0 + kh * 32 + (lane & 31);
-      // key j is visible to row r iff r >= row_thr (rows that do not exist are stored as -1)
-      const int row_thr = j >= Lk ? 0x7fffffff : (causal ? max(0, j - off) : 0);
-      // register i holds gathered row acc_row(i, hh) = 8*(i/4) + 4*hh + i%4 of the tile
-      float pr[16], ds[16];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int base = ts * 32 + 8 * g + 4 * hh;
-        const f32x4 l4 = *reinterpret_cast<const f32x4 *>(sLse + base), d4 = *reinterpret_cast<const f32x4 *>(sDelta + base);
-        const int4 r4 = *reinterpret_cast<const int4 *>(sRow + base);
-        const int rr[4] = {r4.x, r4.y, r4.z, r4.w};
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          const int i = 4 * g + jj;
-          const float x = rr[jj] >= row_thr ? fmaf(s[i], scale_log2, -l4[jj] * kLog2e) : -INFINITY;
-          const float p = __builtin_amdgcn_exp2f(x);
-          pr[i] = p;
-          ds[i] = p * (dp[i] - d4[jj]);
+    for (int seg0 = start; seg0 < nnz; seg0 += kListCap) {
+      const int seg_len = min(kListCap, nnz - seg0);
+      fill_list(seg0, seg_len);
+      const int ntile = (seg_len + 31) >> 5;
+      const int nround = (ntile + 1) >> 1;
+      auto load_round = [&](auto par, int r) {
+        constexpr int P = decltype(par)::value;
+  #pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const int v = lt + 128 * i;
+          const int row = v / VPR, e = (v - row * VPR) * 8;  // row 0..63 over the two tiles of the round
+          const int j = r * 64 + row;
+          const int rid = j < seg_len ? sList[j] : -1;
+          Pack8 xq = zero_pack8(), xo = zero_pack8();
+          if (rid >= 0 && e < D) {
+            xq = ld_global16(qg + (int64_t)rid * a.q_row_stride + e);
+            xo = ld_global16(dog + (int64_t)rid * a.do_row_stride + e);
+          }
+          if constexpr (P == 0) {
+            lq0[i] = xq;
+            ld0[i] = xo;
+          } else {
+            lq1[i] = xq;
+            ld1[i] = xo;
+          }
         }
-      }
-      Pack8 pf[2], dsf[2];
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          pf[s2].w[w] = pack2<T>(pr[8 * s2 + 2 * w], pr[8 * s2 + 2 * w + 1]);
-          dsf[s2].w[w] = pack2<T>(ds[8 * s2 + 2 * w], ds[8 * s2 + 2 * w + 1]);
+        if (lt < 64) {
+          const int j = r * 64 + lt;
+          const int rid = j < seg_len ? sList[j] : -1;
+          float xl = INFINITY, xd = 0.f;
+          if (rid >= 0) {
+            xl = lseg[rid];
+            xd = delg[rid];
+          }
+          if constexpr (P == 0) {
+            lrow0 = rid;
+            llse0 = xl;
+            ldel0 = xd;
+          } else {
+            lrow1 = rid;
+            llse1 = xl;
+            ldel1 = xd;
+          }
         }
-      // dS^T of this wave's 32 keys to its LDS tile [key][row], 4 rows per 8-byte store
-#pragma unroll
-      for (int g = 0; g < 4; ++g)
-        *reinterpret_cast<uint2 *>(sdS + (lane & 31) * LDS_ + 8 * g + 4 * hh) =
-            make_uint2(pack2<T>(ds[4 * g], ds[4 * g + 1]), pack2<T>(ds[4 * g + 2], ds[4 * g + 3]));
-      // dV^T[d][key] += dO^T[d][row] P[row][key];  dK^T[d][key] += Q^T[d][row] dS[row][key]
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        Pack8 dot[2], qt[2];
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          dot[s2] = tr_frag8(tdO, LDQ, 16 * s2 + 4 * hh, 16 * s2 + 8 + 4 * hh, dt * 32, lane);
-          qt[s2] = tr_frag8(tQ, LDQ, 16 * s2 + 4 * hh, 16 * s2 + 8 + 4 * hh, dt * 32, lane);
+      };
+      auto store_round = [&](auto par) {
+        constexpr int P = decltype(par)::value;
+  #pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const int v = lt + 128 * i;
+          const int row = v / VPR, e = (v - row * VPR) * 8;
+          *reinterpret_cast<Pack8 *>(sQ + row * LDQ + e) = P == 0 ? lq0[i] : lq1[i];
+          *reinterpret_cast<Pack8 *>(sdO + row * LDQ + e) = P == 0 ? ld0[i] : ld1[i];
         }
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          dv[dt] = mfma32<T>(dot[s2], pf[s2], dv[dt]);
-          dk[dt] = mfma32<T>(qt[s2], dsf[s2], dk[dt]);
+        if (lt < 64) {
+          sRow[lt] = P == 0 ? lrow0 : lrow1;
+          sLse[lt] = P == 0 ? llse0 : llse1;
+          sDelta[lt] = P == 0 ? ldel0 : ldel1;
         }
-      }
-      // dS rows of this tile to the workspace: lane (row, hh) holds 8 consecutive keys per step
-      wave_lds_fence();
-      const int myrow = sRow[ts * 32 + (lane & 31)];
-      {
-        // the transposing read exchanges data between lanes: every lane takes part, only the store is predicated
-        Pack8 x[2];
-#pragma unroll
-        for (int s4 = 0; s4 < 2; ++s4) x[s4] = tr_frag8(sdS, LDS_, 16 * s4 + 8 * hh, 16 * s4 + 8 * hh + 4, 0, lane);
-        if (myrow >= 0) {
-          uint16_t *wp = ds_ws + (lbase + seg0 + tile * 32 + (lane & 31)) * Bn + koff + kh * 32;
-#pragma unroll
-          for (int s4 = 0; s4 < 2; ++s4) *reinterpret_cast<Pack8 *>(wp + 16 * s4 + 8 * hh) = x[s4];
-        }
-      }
-      wave_lds_fence();
-    };
+      };
 
-    typedef std::integral_constant<int, 0> P0;
-    typedef std::integral_constant<int, 1> P1;
-    // The two roles run separate loops with the same barrier sequence, so that the loaders' rings
-    // and the compute waves' operands do not add up in the register allocation.
-    if (is_loader) {
+      typedef std::integral_constant<int, 0> P0;
+      typedef std::integral_constant<int, 1> P1;
       load_round(P0{}, 0);
       if (nround > 1) load_round(P1{}, 1);
       auto loader_round = [&](auto par, int r) {
@@ -319,47 +233,240 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         loader_round(P0{}, r);
         if (r + 1 < nround) loader_round(P1{}, r + 1);
       }
-    } else {
+    }
+    __syncthreads();
+  } else {
+    f32x16 dv[NDT], dk[NDT];
+  #pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+  #pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        dv[dt][i] = 0.f;
+        dk[dt][i] = 0.f;
+      }
+
+    for (int seg0 = start; seg0 < nnz; seg0 += kListCap) {
+      const int seg_len = min(kListCap, nnz - seg0);
+      fill_list(seg0, seg_len);
+      const int ntile = (seg_len + 31) >> 5;
+      const int nround = (ntile + 1) >> 1;
+      // ---- compute-wave stages ---------------------------------------------------------------------
+      // A compute wave is alone on its SIMD, so the MFMA pipe only stays busy if the softmax arithmetic
+      // of one tile runs between the products of the other tile of the round.  Every stage is cut into
+      // four chunks (a quarter of the products + a quarter of the softmax rows); the operands of chunk
+      // g+1 are read from LDS while chunk g computes, and the scheduler is fenced between chunks: left
+      // alone, the compiler sinks every read next to the MFMA that uses it and waits for it there.
+      typedef std::integral_constant<int, 0> C0;
+      typedef std::integral_constant<int, 1> C1;
+      constexpr int KC = KS / 4;       // k-steps of S / dP per chunk
+      constexpr int BC = NDT / 2;      // (d-tile, row-half) operand pairs of dV / dK per chunk
+      lds_cu16 *trQ = tr_lane_base(sQ, LDQ, lane) + 4 * hh * LDQ, *trdO = tr_lane_base(sdO, LDQ, lane) + 4 * hh * LDQ;
+      lds_cu16 *trdS = tr_lane_base(sdS, LDS_, lane) + 8 * hh * LDS_;
+      Pack8 qa[2][KC], doa[2][KC];     // A operands of S and dP (this lane's row, its half of the head dim), double-buffered by chunk
+      Pack8 kb[2][KC], vb[2][KC];      // B operands: this lane's key, same slices of the head dim
+      Pack8 dot[2][BC], qt[2][BC];     // dO^T / Q^T operands of the dV / dK products, double-buffered by chunk
+      f32x4 lse4[2], del4[2];          // softmax inputs of a chunk's four rows
+      int4 row4[2];
+      Pack8 pf[2][2], dsf[2][2];       // P and dS of both tiles of the round as MFMA operands
+      Pack8 dsx[2];                    // dS rows on their way to the workspace
+      int dsrow = -1;
+      f32x16 s[2], dp[2];
+      auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+      auto ld_a = [&](auto tsc, auto gc) {
+        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+        const uint16_t *tQ = sQ + TS * 32 * LDQ, *tdO = sdO + TS * 32 * LDQ;
+  #pragma unroll
+        for (int t = 0; t < KC; ++t) {
+          qa[G & 1][t] = *reinterpret_cast<const Pack8 *>(tQ + (lane & 31) * LDQ + (hh * KS + G * KC + t) * 8);
+          doa[G & 1][t] = *reinterpret_cast<const Pack8 *>(tdO + (lane & 31) * LDQ + (hh * KS + G * KC + t) * 8);
+          kb[G & 1][t] = *reinterpret_cast<const Pack8 *>(sK + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + G * KC + t) * 8);
+          vb[G & 1][t] = *reinterpret_cast<const Pack8 *>(sV + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + G * KC + t) * 8);
+        }
+      };
+      auto mm_a = [&](auto tsc, auto gc) {
+        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+        if constexpr (G == 0) {
+  #pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            s[TS][i] = 0.f;
+            dp[TS][i] = 0.f;
+          }
+        }
+  #pragma unroll
+        for (int t = 0; t < KC; ++t) {
+          s[TS] = mfma32<T>(qa[G & 1][t], kb[G & 1][t], s[TS]);
+          dp[TS] = mfma32<T>(doa[G & 1][t], vb[G & 1][t], dp[TS]);
+        }
+      };
+      auto ld_b = [&](auto tsc, auto gc) {
+        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+  #pragma unroll
+        for (int t = 0; t < BC; ++t) {
+          const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
+          const int lo = (TS * 32 + 16 * s2) * LDQ + dt * 32, hi = lo + 8 * LDQ;
+          dot[G & 1][t] = tr_frag8_at(trdO, lo, hi);
+          qt[G & 1][t] = tr_frag8_at(trQ, lo, hi);
+        }
+      };
+      auto mm_b = [&](auto tsc, auto gc) {
+        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+        // dV^T[d][key] += dO^T[d][row] P[row][key];  dK^T[d][key] += Q^T[d][row] dS[row][key]
+  #pragma unroll
+        for (int t = 0; t < BC; ++t) {
+          const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
+          dv[dt] = mfma32<T>(dot[G & 1][t], pf[TS][s2], dv[dt]);
+          dk[dt] = mfma32<T>(qt[G & 1][t], dsf[TS][s2], dk[dt]);
+        }
+      };
+      // this lane's key; key j is visible to row r iff r >= row_thr (rows that do not exist are stored as -1)
+      const int j = key0 + kh * 32 + (lane & 31);
+      const int row_thr = j >= Lk ? 0x7fffffff : (causal ? max(0, j - off) : 0);
+      auto ld_s = [&](auto tsc, auto gc) {
+        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+        const int base = TS * 32 + 8 * G + 4 * hh;  // accumulator registers 4G..4G+3 hold rows base..base+3
+        lse4[G & 1] = *reinterpret_cast<const f32x4 *>(sLse + base);
+        del4[G & 1] = *reinterpret_cast<const f32x4 *>(sDelta + base);
+        row4[G & 1] = *reinterpret_cast<const int4 *>(sRow + base);
+      };
+      auto smx = [&](auto tsc, auto gc) {
+        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+        const int rr[4] = {row4[G & 1].x, row4[G & 1].y, row4[G & 1].z, row4[G & 1].w};
+        float pr[4], ds[4];
+  #pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const int i = 4 * G + jj;
+          const float x = rr[jj] >= row_thr ? fmaf(s[TS][i], scale_log2, -lse4[G & 1][jj] * kLog2e) : -INFINITY;
+          pr[jj] = __builtin_amdgcn_exp2f(x);
+          ds[jj] = pr[jj] * (dp[TS][i] - del4[G & 1][jj]);
+        }
+        // operand register s2 = G/2 holds rows 16*s2 + 8*(w/2) + 4*hh + ..: words 2*(G%2), 2*(G%2)+1
+        pf[TS][G >> 1].w[2 * (G & 1)] = pack2<T>(pr[0], pr[1]);
+        pf[TS][G >> 1].w[2 * (G & 1) + 1] = pack2<T>(pr[2], pr[3]);
+        dsf[TS][G >> 1].w[2 * (G & 1)] = pack2<T>(ds[0], ds[1]);
+        dsf[TS][G >> 1].w[2 * (G & 1) + 1] = pack2<T>(ds[2], ds[3]);
+      };
+      // dS^T of this wave's 32 keys goes through its LDS tile [key][row] and comes back as rows: lane
+      // (row, hh) gets 8 consecutive keys per read and stores them to the workspace.  The transposing read
+      // exchanges data between lanes: every lane takes part, only the store is predicated.
+      auto ds_write = [&](auto tsc) {
+        constexpr int TS = decltype(tsc)::value;
+  #pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          *reinterpret_cast<uint2 *>(sdS + (lane & 31) * LDS_ + 16 * s2 + 4 * hh) = make_uint2(dsf[TS][s2].w[0], dsf[TS][s2].w[1]);
+          *reinterpret_cast<uint2 *>(sdS + (lane & 31) * LDS_ + 16 * s2 + 8 + 4 * hh) = make_uint2(dsf[TS][s2].w[2], dsf[TS][s2].w[3]);
+        }
+        wave_lds_fence();
+      };
+      auto ds_read = [&](auto tsc) {
+        constexpr int TS = decltype(tsc)::value;
+        dsrow = sRow[TS * 32 + (lane & 31)];
+  #pragma unroll
+        for (int s4 = 0; s4 < 2; ++s4) dsx[s4] = tr_frag8_at(trdS, 16 * s4 * LDS_, (16 * s4 + 4) * LDS_);
+        wave_lds_fence();
+      };
+      auto ds_store = [&](int tile) {
+        if (dsrow >= 0) {
+          uint16_t *wp = ds_ws + (lbase + seg0 + tile * 32 + (lane & 31)) * Bn + koff + kh * 32;
+  #pragma unroll
+          for (int s4 = 0; s4 < 2; ++s4) *reinterpret_cast<Pack8 *>(wp + 16 * s4 + 8 * hh) = dsx[s4];
+        }
+      };
+      // One round = tiles 2r and 2r+1, both already in LDS.  A list with an odd number of tiles ends with a tile
+      // of absent rows (row id -1, zero data): it runs through the same code and adds nothing.
+      auto process_round = [&](int r) {
+        // S, dP of the first tile
+        ld_a(C0{}, C0{});
+        fence();
+        static_for<4>([&](auto gc) {
+          constexpr int G = decltype(gc)::value;
+          if constexpr (G < 3) ld_a(C0{}, std::integral_constant<int, G + 1>{});
+          mm_a(C0{}, gc);
+          fence();
+        });
+        // S, dP of the second tile between the softmax rows of the first
+        ld_a(C1{}, C0{});
+        ld_s(C0{}, C0{});
+        fence();
+        static_for<4>([&](auto gc) {
+          constexpr int G = decltype(gc)::value;
+          if constexpr (G < 3) {
+            ld_a(C1{}, std::integral_constant<int, G + 1>{});
+            ld_s(C0{}, std::integral_constant<int, G + 1>{});
+          }
+          mm_a(C1{}, gc);
+          smx(C0{}, gc);
+          fence();
+        });
+        // dV, dK of the first tile between the softmax rows of the second
+        ds_write(C0{});
+        ld_b(C0{}, C0{});
+        ld_s(C1{}, C0{});
+        ds_read(C0{});
+        fence();
+        static_for<4>([&](auto gc) {
+          constexpr int G = decltype(gc)::value;
+          if constexpr (G < 3) {
+            ld_b(C0{}, std::integral_constant<int, G + 1>{});
+            ld_s(C1{}, std::integral_constant<int, G + 1>{});
+          }
+          if constexpr (G == 0) ds_store(2 * r);
+          mm_b(C0{}, gc);
+          smx(C1{}, gc);
+          fence();
+        });
+        // dV, dK of the second tile
+        ds_write(C1{});
+        ld_b(C1{}, C0{});
+        ds_read(C1{});
+        fence();
+        static_for<4>([&](auto gc) {
+          constexpr int G = decltype(gc)::value;
+          if constexpr (G < 3) ld_b(C1{}, std::integral_constant<int, G + 1>{});
+          if constexpr (G == 0) ds_store(2 * r + 1);
+          mm_b(C1{}, gc);
+          fence();
+        });
+      };
+
       for (int r = 0; r < nround; ++r) {
         __syncthreads();
         __syncthreads();  // tiles 2r, 2r+1 are in LDS
-        process_tile(2 * r, 0);
-        if (2 * r + 1 < ntile) process_tile(2 * r + 1, 1);
+        process_round(r);
       }
     }
+    __syncthreads();  // every wave is done with the tiles: the output buffer may overwrite them
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 v4, k4;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          v4[jj] = dv[dt][4 * g + jj];
+          k4[jj] = dk[dt][4 * g + jj];
+        }
+        float *rp = red + (size_t)(kh * 32 + (lane & 31)) * LDR + dt * 32 + 8 * g + 4 * hh;
+        *reinterpret_cast<f32x4 *>(rp) = v4;
+        *reinterpret_cast<f32x4 *>(rp + 64 * LDR) = k4;
+      }
   }
+  __syncthreads();
 
-  // ---- dK^T / dV^T go through LDS to be written as rows, once ------------------------------------
-  float *red = reinterpret_cast<float *>(smem);
+  // ---- dK^T / dV^T leave as rows, once ----------------------------------------------------------------
   uint16_t *dkg = reinterpret_cast<uint16_t *>(a.dk) + (int64_t)(k0 + key0) * a.dk_row_stride + (int64_t)h * a.dk_head_stride;
   uint16_t *dvg = reinterpret_cast<uint16_t *>(a.dv) + (int64_t)(k0 + key0) * a.dv_row_stride + (int64_t)h * a.dv_head_stride;
+  for (int v = tid; v < 64 * VPR; v += 256) {
+    const int key = v / VPR, e = (v - key * VPR) * 8;
+    if (key0 + key >= Lk || e >= D) continue;
+    const float *s0 = red + (size_t)key * LDR + e, *s1 = s0 + 64 * LDR;
+    Pack8 ov, ok;
 #pragma unroll
-  for (int which = 0; which < 2; ++which) {
-    __syncthreads();
-    if (!is_loader) {
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          f32x4 v4;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) v4[j] = which == 0 ? dv[dt][4 * g + j] : dk[dt][4 * g + j];
-          *reinterpret_cast<f32x4 *>(red + (size_t)(kh * 32 + (lane & 31)) * LDR + dt * 32 + 8 * g + 4 * hh) = v4;
-        }
+    for (int w = 0; w < 4; ++w) {
+      ov.w[w] = pack2<T>(s0[2 * w], s0[2 * w + 1]);
+      ok.w[w] = pack2<T>(s1[2 * w] * a.softmax_scale, s1[2 * w + 1] * a.softmax_scale);
     }
-    __syncthreads();
-    const float mul = which == 0 ? 1.f : a.softmax_scale;
-    uint16_t *og = which == 0 ? dvg : dkg;
-    const int64_t ors = which == 0 ? a.dv_row_stride : a.dk_row_stride;
-    for (int v = tid; v < 64 * VPR; v += 256) {
-      const int key = v / VPR, e = (v - key * VPR) * 8;
-      if (key0 + key >= Lk || e >= D) continue;
-      const float *s0 = red + (size_t)key * LDR + e;
-      Pack8 o;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) o.w[w] = pack2<T>(s0[2 * w] * mul, s0[2 * w + 1] * mul);
-      *reinterpret_cast<Pack8 *>(og + (int64_t)key * ors + e) = o;
-    }
+    *reinterpret_cast<Pack8 *>(dvg + (int64_t)key * a.dv_row_stride + e) = ov;
+    *reinterpret_cast<Pack8 *>(dkg + (int64_t)key * a.dk_row_stride + e) = ok;
   }
 }
 

@@ -77,9 +77,17 @@ __device__ __forceinline__ uint16_t float_to_elem_bits(float f) {
   __builtin_memcpy(&b, &x, 2);
   return b;
 }
+// Two floats to one 32-bit word of two elements (lo in bits 0..15), round to nearest even:
+// the vector conversion compiles to a single packed convert.
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  return (uint32_t)float_to_elem_bits<T>(lo) | ((uint32_t)float_to_elem_bits<T>(hi) << 16);
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef T elem2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {lo, hi};
+  const elem2_t r = __builtin_convertvector(v, elem2_t);
+  uint32_t b;
+  __builtin_memcpy(&b, &r, 4);
+  return b;
 }
 template <typename T>
 __device__ __forceinline__ void unpack8(const Pack8 &p, float (&f)[8]) {
@@ -174,6 +182,33 @@ __device__ __forceinline__ Pack8 tr_frag8(const uint16_t *X, int ld, int rows4_l
   Pack8 r;
   __builtin_memcpy(&r.w[0], &lo, 8);
   __builtin_memcpy(&r.w[2], &hi, 8);
+  return r;
+}
+
+// The same read through an LDS-address-space pointer.  lane_base = tr_lane_base(X, ld, lane) is
+// computed once per lane; every further offset is a compile-time constant that the
+// instruction's 16-bit offset field absorbs, so a whole tile of transposed operands costs one
+// address register (the generic-pointer form above needs one register per read).
+typedef __attribute__((address_space(3))) const uint16_t lds_cu16;
+__device__ __forceinline__ lds_cu16 *to_lds(const void *lds_generic_ptr) {
+  return (lds_cu16 *)(uint32_t)(uintptr_t)lds_generic_ptr;
+}
+__device__ __forceinline__ lds_cu16 *tr_lane_base(const uint16_t *X, int ld, int lane) {
+  const int i = lane & 15;
+  return to_lds(X) + (i >> 2) * ld + ((lane & 31) >> 4) * 16 + (i & 3) * 4;
+}
+// elem_off_lo / elem_off_hi: (rows4_xx * ld + col0) of tr_frag8, in elements
+__device__ __forceinline__ Pack8 tr_frag8_at(lds_cu16 *lane_base, int elem_off_lo, int elem_off_hi) {
+  Pack8 r;
+#if defined(__HIP_DEVICE_COMPILE__)
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(lane_base + elem_off_lo));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(lane_base + elem_off_hi));
+  __builtin_memcpy(&r.w[0], &lo, 8);
+  __builtin_memcpy(&r.w[2], &hi, 8);
+#else
+  (void)lane_base, (void)elem_off_lo, (void)elem_off_hi;
+  r = Pack8{{0, 0, 0, 0}};
+#endif
   return r;
 }
 
