@@ -31,17 +31,20 @@ constexpr int kListCap = 4096;  // rows of a column list held in LDS at a time
 
 template <int HD>
 struct BwdSmem {
-  static constexpr int LDQ = HD + 16;  // elements, K / V / Q / dO tiles
+  // Row stride of the K / V / Q / dO tiles, in elements.  Measured on gfx950 with 16-byte rows-per-lane reads
+  // (lane -> row lane % 32) and the transposing 8-byte reads: HD + 16 runs both at the LDS peak
+  // (8.4 and 4.7 clk per instruction per CU); strides that leave rows 8-byte aligned are 8x slower.
+  static constexpr int LDQ = HD + 16;
   static constexpr int LDS_ = 32 + 8;  // elements, per-wave dS^T tile [32 keys][32 rows]
   static constexpr size_t oK = 0;
   static constexpr size_t oV = oK + (size_t)64 * LDQ * 2;
-  static constexpr size_t oQ = oV + (size_t)64 * LDQ * 2;          // [2 tile slots][32][LDQ]
-  static constexpr size_t odO = oQ + (size_t)2 * 32 * LDQ * 2;
-  static constexpr size_t odS = odO + (size_t)2 * 32 * LDQ * 2;    // [2 waves][32][LDS_]
-  static constexpr size_t oRow = odS + (size_t)2 * 32 * LDS_ * 2;  // int[2][32]
-  static constexpr size_t oLse = oRow + 2 * 32 * 4;
-  static constexpr size_t oDelta = oLse + 2 * 32 * 4;
-  static constexpr size_t oList = oDelta + 2 * 32 * 4;             // int[kListCap]
+  static constexpr size_t oQ = oV + (size_t)64 * LDQ * 2;          // [2 buffers][2 tile slots][32][LDQ]
+  static constexpr size_t odO = oQ + (size_t)4 * 32 * LDQ * 2;
+  static constexpr size_t odS = odO + (size_t)4 * 32 * LDQ * 2;    // [2 waves][32][LDS_]
+  static constexpr size_t oRow = odS + (size_t)2 * 32 * LDS_ * 2;  // int[2 buffers][64]
+  static constexpr size_t oLse = oRow + 4 * 32 * 4;                // LSE * log2(e)
+  static constexpr size_t oDelta = oLse + 4 * 32 * 4;
+  static constexpr size_t oList = oDelta + 4 * 32 * 4;             // int[kListCap]
   static constexpr size_t mainBytes = oList + (size_t)kListCap * 4;
   static constexpr int LDR = HD + 4;  // floats, output transpose buffer [2][64 keys][LDR]
   static constexpr size_t redBytes = (size_t)2 * 64 * LDR * 4;
@@ -209,29 +212,34 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         for (int i = 0; i < NV; ++i) {
           const int v = lt + 128 * i;
           const int row = v / VPR, e = (v - row * VPR) * 8;
-          *reinterpret_cast<Pack8 *>(sQ + row * LDQ + e) = P == 0 ? lq0[i] : lq1[i];
-          *reinterpret_cast<Pack8 *>(sdO + row * LDQ + e) = P == 0 ? ld0[i] : ld1[i];
+          *reinterpret_cast<Pack8 *>(sQ + (P * 64 + row) * LDQ + e) = P == 0 ? lq0[i] : lq1[i];
+          *reinterpret_cast<Pack8 *>(sdO + (P * 64 + row) * LDQ + e) = P == 0 ? ld0[i] : ld1[i];
         }
         if (lt < 64) {
-          sRow[lt] = P == 0 ? lrow0 : lrow1;
-          sLse[lt] = P == 0 ? llse0 : llse1;
-          sDelta[lt] = P == 0 ? ldel0 : ldel1;
+          sRow[P * 64 + lt] = P == 0 ? lrow0 : lrow1;
+          sLse[P * 64 + lt] = (P == 0 ? llse0 : llse1) * kLog2e;
+          sDelta[P * 64 + lt] = P == 0 ? ldel0 : ldel1;
         }
       };
 
       typedef std::integral_constant<int, 0> P0;
       typedef std::integral_constant<int, 1> P1;
+      // Tiles are double buffered in LDS by round parity, and so are the rings: during round r the loaders
+      // put round r+1 into the other buffer and fetch round r+3 into the registers that this frees.
       load_round(P0{}, 0);
       if (nround > 1) load_round(P1{}, 1);
-      auto loader_round = [&](auto par, int r) {
-        __syncthreads();  // the previous round's readers are done with the tile buffers
-        store_round(par);
-        __syncthreads();
-        if (r + 2 < nround) load_round(par, r + 2);
+      store_round(P0{});
+      if (nround > 2) load_round(P0{}, 2);
+      auto loader_round = [&](auto par, int r) {  // par: parity of round r + 1
+        __syncthreads();  // round r is in LDS; the readers of round r-1 are done with the other buffer
+        if (r + 1 < nround) {
+          store_round(par);
+          if (r + 3 < nround) load_round(par, r + 3);
+        }
       };
       for (int r = 0; r < nround; r += 2) {
-        loader_round(P0{}, r);
-        if (r + 1 < nround) loader_round(P1{}, r + 1);
+        loader_round(P1{}, r);
+        if (r + 1 < nround) loader_round(P0{}, r + 1);
       }
     }
     __syncthreads();
@@ -272,8 +280,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       int dsrow = -1;
       f32x16 s[2], dp[2];
       auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
-      auto ld_a = [&](auto tsc, auto gc) {
-        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+      auto ld_a = [&](auto pc, auto tsc, auto gc) {
+        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value, G = decltype(gc)::value;
         const uint16_t *tQ = sQ + TS * 32 * LDQ, *tdO = sdO + TS * 32 * LDQ;
   #pragma unroll
         for (int t = 0; t < KC; ++t) {
@@ -298,8 +306,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           dp[TS] = mfma32<T>(doa[G & 1][t], vb[G & 1][t], dp[TS]);
         }
       };
-      auto ld_b = [&](auto tsc, auto gc) {
-        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+      auto ld_b = [&](auto pc, auto tsc, auto gc) {
+        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value, G = decltype(gc)::value;
   #pragma unroll
         for (int t = 0; t < BC; ++t) {
           const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
@@ -321,8 +329,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       // this lane's key; key j is visible to row r iff r >= row_thr (rows that do not exist are stored as -1)
       const int j = key0 + kh * 32 + (lane & 31);
       const int row_thr = j >= Lk ? 0x7fffffff : (causal ? max(0, j - off) : 0);
-      auto ld_s = [&](auto tsc, auto gc) {
-        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+      auto ld_s = [&](auto pc, auto tsc, auto gc) {
+        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value, G = decltype(gc)::value;
         const int base = TS * 32 + 8 * G + 4 * hh;  // accumulator registers 4G..4G+3 hold rows base..base+3
         lse4[G & 1] = *reinterpret_cast<const f32x4 *>(sLse + base);
         del4[G & 1] = *reinterpret_cast<const f32x4 *>(sDelta + base);
@@ -335,7 +343,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
           const int i = 4 * G + jj;
-          const float x = rr[jj] >= row_thr ? fmaf(s[TS][i], scale_log2, -lse4[G & 1][jj] * kLog2e) : -INFINITY;
+          const float x = rr[jj] >= row_thr ? fmaf(s[TS][i], scale_log2, -lse4[G & 1][jj]) : -INFINITY;
           pr[jj] = __builtin_amdgcn_exp2f(x);
           ds[jj] = pr[jj] * (dp[TS][i] - del4[G & 1][jj]);
         }
@@ -357,8 +365,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         }
         wave_lds_fence();
       };
-      auto ds_read = [&](auto tsc) {
-        constexpr int TS = decltype(tsc)::value;
+      auto ds_read = [&](auto pc, auto tsc) {
+        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value;
         dsrow = sRow[TS * 32 + (lane & 31)];
   #pragma unroll
         for (int s4 = 0; s4 < 2; ++s4) dsx[s4] = tr_frag8_at(trdS, 16 * s4 * LDS_, (16 * s4 + 4) * LDS_);
@@ -373,25 +381,25 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       };
       // One round = tiles 2r and 2r+1, both already in LDS.  A list with an odd number of tiles ends with a tile
       // of absent rows (row id -1, zero data): it runs through the same code and adds nothing.
-      auto process_round = [&](int r) {
+      auto process_round = [&](auto pc, int r) {  // pc: parity of r = the LDS buffer that holds the round
         // S, dP of the first tile
-        ld_a(C0{}, C0{});
+        ld_a(pc, C0{}, C0{});
         fence();
         static_for<4>([&](auto gc) {
           constexpr int G = decltype(gc)::value;
-          if constexpr (G < 3) ld_a(C0{}, std::integral_constant<int, G + 1>{});
+          if constexpr (G < 3) ld_a(pc, C0{}, std::integral_constant<int, G + 1>{});
           mm_a(C0{}, gc);
           fence();
         });
         // S, dP of the second tile between the softmax rows of the first
-        ld_a(C1{}, C0{});
-        ld_s(C0{}, C0{});
+        ld_a(pc, C1{}, C0{});
+        ld_s(pc, C0{}, C0{});
         fence();
         static_for<4>([&](auto gc) {
           constexpr int G = decltype(gc)::value;
           if constexpr (G < 3) {
-            ld_a(C1{}, std::integral_constant<int, G + 1>{});
-            ld_s(C0{}, std::integral_constant<int, G + 1>{});
+            ld_a(pc, C1{}, std::integral_constant<int, G + 1>{});
+            ld_s(pc, C0{}, std::integral_constant<int, G + 1>{});
           }
           mm_a(C1{}, gc);
           smx(C0{}, gc);
@@ -399,39 +407,42 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         });
         // dV, dK of the first tile between the softmax rows of the second
         ds_write(C0{});
-        ld_b(C0{}, C0{});
-        ld_s(C1{}, C0{});
-        ds_read(C0{});
+        ld_b(pc, C0{}, C0{});
+        ld_s(pc, C1{}, C0{});
+        ds_read(pc, C0{});
         fence();
         static_for<4>([&](auto gc) {
           constexpr int G = decltype(gc)::value;
           if constexpr (G < 3) {
-            ld_b(C0{}, std::integral_constant<int, G + 1>{});
-            ld_s(C1{}, std::integral_constant<int, G + 1>{});
+            ld_b(pc, C0{}, std::integral_constant<int, G + 1>{});
+            ld_s(pc, C1{}, std::integral_constant<int, G + 1>{});
           }
-          if constexpr (G == 0) ds_store(2 * r);
           mm_b(C0{}, gc);
           smx(C1{}, gc);
+          if constexpr (G == 1) ds_store(2 * r);
           fence();
         });
         // dV, dK of the second tile
         ds_write(C1{});
-        ld_b(C1{}, C0{});
-        ds_read(C1{});
+        ld_b(pc, C1{}, C0{});
+        ds_read(pc, C1{});
         fence();
         static_for<4>([&](auto gc) {
           constexpr int G = decltype(gc)::value;
-          if constexpr (G < 3) ld_b(C1{}, std::integral_constant<int, G + 1>{});
-          if constexpr (G == 0) ds_store(2 * r + 1);
+          if constexpr (G < 3) ld_b(pc, C1{}, std::integral_constant<int, G + 1>{});
           mm_b(C1{}, gc);
+          if constexpr (G == 1) ds_store(2 * r + 1);
           fence();
         });
       };
 
-      for (int r = 0; r < nround; ++r) {
-        __syncthreads();
-        __syncthreads();  // tiles 2r, 2r+1 are in LDS
-        process_round(r);
+      for (int r = 0; r < nround; r += 2) {
+        __syncthreads();  // round r is in LDS
+        process_round(C0{}, r);
+        if (r + 1 < nround) {
+          __syncthreads();
+          process_round(C1{}, r + 1);
+        }
       }
     }
     __syncthreads();  // every wave is done with the tiles: the output buffer may overwrite them
