@@ -95,6 +95,16 @@ def time_events(fn, iters, warmup=1):
     return s.elapsed_time(e) / iters
 
 
+# HBM-side bytes per launch on the headline workload: rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch, each scaled by
+# what the same counter reads for a plain 1 GiB copy (the summary of those runs is kept under profiles/).
+# Counter runs cannot be made from inside this script, so the figures are the committed measurement.
+MEASURED_TRAFFIC_BYTES = {
+    ("headline", "attn_fwd_kernel"): 1.712e9,
+    ("headline", "attn_bwd_dkdv_kernel"): 18.588e9,
+    ("headline", "attn_bwd_dq_kernel"): 4.774e9,
+}
+
+
 def cpu_baseline(q, k, v, cu, seqlens, chunk, topk, budget_s=12.0):
     """Times the CPU restatement of the reference's PyTorch MoBA path (chunk means -> gate ->
     top-k -> block mask -> dense-masked softmax attention, fp32) on (longest sequence,
@@ -238,7 +248,8 @@ def main():
     dom = max(kernels, key=lambda n: kernels[n][0])
     d_ms, d_flops, _ = kernels[dom]
     roofline = {"kernel": dom, "bound": "mfma", "achieved": d_flops / d_ms / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS, "traffic": None, "avg_launch_ms": d_ms,
+                "frac": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
+                "traffic_unit": "bytes/launch", "avg_launch_ms": d_ms,
                 "flops_per_launch": d_flops}
 
     result = {
