@@ -501,7 +501,8 @@ struct DqSmem {
   static constexpr size_t oCnt = oLo + kDqColBatch * 4;
   static constexpr size_t oStep = oCnt + kDqColBatch * 4;
   static constexpr size_t oOff = oStep + kDqMaxSteps * 4;          // int64[kDqColBatch]
-  static constexpr size_t oMisc = oOff + kDqColBatch * 8;
+  static constexpr size_t oInfo = oOff + kDqColBatch * 8;          // int4[kDqMaxSteps]: key0, rows, list position (lo, hi)
+  static constexpr size_t oMisc = oInfo + kDqMaxSteps * 16;
   static constexpr size_t bytes = oMisc + 64;
 };
 
@@ -534,6 +535,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
   int *sCnt = reinterpret_cast<int *>(smem + SM::oCnt);
   int *sStep = reinterpret_cast<int *>(smem + SM::oStep);
   int64_t *sOff = reinterpret_cast<int64_t *>(smem + SM::oOff);
+  int4 *sInfo = reinterpret_cast<int4 *>(smem + SM::oInfo);
   int *sMisc = reinterpret_cast<int *>(smem + SM::oMisc);
 
   const DqItem wi = dq_decode_item(blockIdx.x, a.heads * a.batch, nsb_max);
@@ -563,8 +565,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
   const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + (int64_t)k0 * a.k_row_stride + (int64_t)hk * a.k_head_stride;
   const int cols_per_batch = min(kDqColBatch, kDqMaxSteps / nsub);
 
-  Pack8 pk0[KVV], pk1[KVV], pd0[DVV], pd1[DVV];
-  int prow0 = 0, prow1 = 0;
+  // loader rings, four steps deep: the dS rows come from HBM (about 2 us under load), a step takes well under 1 us
+  Pack8 pk[4][KVV], pd[4][DVV];
+  int prow[4] = {0, 0, 0, 0};
 
   for (int cb = 0; cb < ncols; cb += cols_per_batch) {
     const int cend = min(ncols, cb + cols_per_batch);
@@ -605,71 +608,74 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
     const int nsteps = sMisc[0];
     if (nsteps == 0) continue;
 
+    // one record per step, so that a loader needs a single LDS read before it can issue its loads
+    for (int st = tid; st < nsteps; st += 512) {
+      const int code = sStep[st];
+      const int cl = code >> 8, kb = code & 255;
+      const int64_t pos0 = sOff[cl];
+      sInfo[st] = make_int4((cb + cl) * Bn + kb * 64, sCnt[cl], (int)(uint32_t)(pos0 & 0xffffffffll), (int)(pos0 >> 32));
+    }
+    __syncthreads();
+
+    // Loads are unconditional (indices clamped into the valid range, the surplus zeroed when it is stored):
+    // without branches around them the compiler counts outstanding loads exactly, so storing one ring
+    // entry does not wait for the loads of the next one.
     auto load_step = [&](auto par, int step) {
       constexpr int P = decltype(par)::value;
-      const int code = sStep[step];
-      const int cl = code >> 8, kb = code & 255;
-      const int key0 = (cb + cl) * Bn + kb * 64;
-      const int n = sCnt[cl];
-      const int64_t pos0 = sOff[cl];
+      const int4 info = sInfo[min(step, nsteps - 1)];  // past the end: a redundant load, never stored
+      const int key0 = info.x, n = info.y;
+      const int64_t pos0 = (int64_t)(uint32_t)info.z | ((int64_t)info.w << 32);
+      const int koff = key0 - (key0 / Bn) * Bn;  // offset of the 64-key block inside its column
 #pragma unroll
       for (int i = 0; i < KVV; ++i) {
         const int v = ltid + i * 256;
-        const int key = v / VPR, e = (v - key * VPR) * 8;
-        Pack8 x = zero_pack8();
-        if (key0 + key < Lk && e < D) x = ld_global16(kp + (int64_t)(key0 + key) * a.k_row_stride + e);
-        if constexpr (P == 0)
-          pk0[i] = x;
-        else
-          pk1[i] = x;
+        const int key = min(key0 + v / VPR, Lk - 1), e = min((v % VPR) * 8, D - 8);
+        const Pack8 x = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
+        pk[P][i] = x;
       }
 #pragma unroll
       for (int i = 0; i < DVV; ++i) {
         const int v = ltid + i * 256;
-        const int row = v >> 3, e = (v & 7) * 8;
-        Pack8 x = zero_pack8();
-        if (row < n) x = ld_global16(ds_ws + (pos0 + row) * Bn + kb * 64 + e);
-        if constexpr (P == 0)
-          pd0[i] = x;
-        else
-          pd1[i] = x;
+        const int row = min(v >> 3, n - 1), e = (v & 7) * 8;
+        const Pack8 x = ld_global16(ds_ws + (pos0 + row) * Bn + koff + e);
+        pd[P][i] = x;
       }
-      if (ltid < n) {
-        const int rr = a.row_indices[pos0 + ltid];  // raw value: arithmetic here would wait for the load
-        if constexpr (P == 0)
-          prow0 = rr;
-        else
-          prow1 = rr;
-      }
+      prow[P] = a.row_indices[pos0 + min(ltid, n - 1)];
     };
     auto store_step = [&](auto par, int step) {
       constexpr int P = decltype(par)::value;
       const int buf = step & 1;
-      const int code = sStep[step];
-      const int n = sCnt[code >> 8];
-      const int key0 = (cb + (code >> 8)) * Bn + (code & 255) * 64;
+      const int4 info = sInfo[step];
+      const int key0 = info.x, n = info.y;
 #pragma unroll
       for (int i = 0; i < KVV; ++i) {
         const int v = ltid + i * 256;
         const int key = v / VPR, e = (v - key * VPR) * 8;
-        *reinterpret_cast<Pack8 *>(sK + ((size_t)buf * 64 + key) * LDQ + e) = P == 0 ? pk0[i] : pk1[i];
+        const bool ok = key0 + key < Lk && e < D;
+        Pack8 x = pk[P][i];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) x.w[w] = ok ? x.w[w] : 0u;
+        *reinterpret_cast<Pack8 *>(sK + ((size_t)buf * 64 + key) * LDQ + e) = x;
       }
 #pragma unroll
       for (int i = 0; i < DVV; ++i) {
         const int v = ltid + i * 256;
         const int row = v >> 3, e = (v & 7) * 8;
-        *reinterpret_cast<Pack8 *>(sD + ((size_t)buf * kDqRows + row) * LDD + e) = P == 0 ? pd0[i] : pd1[i];
+        Pack8 x = pd[P][i];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) x.w[w] = row < n ? x.w[w] : 0u;
+        *reinterpret_cast<Pack8 *>(sD + ((size_t)buf * kDqRows + row) * LDD + e) = x;
       }
       if (ltid < kDqRows) {
         // the dK/dV pass wrote dS only for rows of this sequence that can see a key of the block
-        const int rr = P == 0 ? prow0 : prow1;
+        const int rr = prow[P];
         const bool ok = ltid < n && rr >= m0 && rr < m0 + rows_sb && !(causal && rr + off < key0);
         sRows[buf * kDqRows + ltid] = ok ? rr - m0 : -1;
       }
     };
     auto compute_step = [&](int step) {
       const int buf = step & 1;
-      const int n = sCnt[sStep[step] >> 8];
+      const int n = sInfo[step].y;
       const uint16_t *tK = sK + (size_t)buf * 64 * LDQ;
       const int dt = wave % NDT;
       for (int tile = wave / NDT; tile * 32 < n; tile += 4 / NDT) {
@@ -701,29 +707,39 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
 
     typedef std::integral_constant<int, 0> P0;
     typedef std::integral_constant<int, 1> P1;
-    // LDS is double buffered by step parity: while the compute waves work on step s the loaders
-    // put step s+1 into the other buffer and then fetch step s+3 into the freed registers
+    typedef std::integral_constant<int, 2> P2;
+    typedef std::integral_constant<int, 3> P3;
+    // LDS is double buffered by step parity: while the compute waves work on step s the loaders put
+    // step s+1 into the other buffer and then fetch step s+5 into the ring entry that this frees
+    // The two roles run separate loops with the same barrier sequence.  Every load_step is issued
+    // unconditionally and no control flow joins the loader path: the compiler sizes each wait by the
+    // smallest number of younger loads over all paths that reach it, and a path without loads (or one
+    // skipped load) would make every store wait for the whole ring.
     if (is_loader) {
       load_step(P0{}, 0);
-      if (nsteps > 1) load_step(P1{}, 1);
+      load_step(P1{}, 1);
+      load_step(P2{}, 2);
+      load_step(P3{}, 3);
       store_step(P0{}, 0);
-      if (nsteps > 2) load_step(P0{}, 2);
-    }
-    auto run_step = [&](auto par, int step) {
-      // par is the parity of step + 1 (the ring entry being stored during this step)
-      __syncthreads();
-      if (is_loader) {
-        if (step + 1 < nsteps) {
-          store_step(par, step + 1);
-          if (step + 3 < nsteps) load_step(par, step + 3);
-        }
-      } else {
-        compute_step(step);
+      load_step(P0{}, 4);
+      auto loader_step = [&](auto par, int step) {  // par: ring entry of step + 1, stored during step
+        __syncthreads();
+        if (step + 1 < nsteps) store_step(par, step + 1);
+        load_step(par, step + 5);
+      };
+      // whole groups of four steps (the step count is padded with empty steps: barriers only)
+      for (int step = 0; step < nsteps; step += 4) {
+        loader_step(P1{}, step);
+        loader_step(P2{}, step + 1);
+        loader_step(P3{}, step + 2);
+        loader_step(P0{}, step + 3);
       }
-    };
-    for (int step = 0; step < nsteps; step += 2) {
-      run_step(P1{}, step);
-      if (step + 1 < nsteps) run_step(P0{}, step + 1);
+    } else {
+      const int nsteps_pad = (nsteps + 3) & ~3;
+      for (int step = 0; step < nsteps_pad; ++step) {
+        __syncthreads();
+        if (step < nsteps) compute_step(step);
+      }
     }
   }
   __syncthreads();
