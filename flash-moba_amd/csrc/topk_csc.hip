@@ -261,6 +261,303 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(TopkParams p) {
   }
 }
 
+// ------------------------------------------------------------------------------------
+// The same gate for sequences with more key chunks than one register tile set holds
+// (NT*32).  Chunks are scored in groups of NT*32; after every group the row keeps the
+// K' best (score, chunk) pairs seen so far in LDS, and the next group competes against
+// them.  The total order (score descending, chunk index descending) is strict, so the
+// running winners after the last group are exactly the global top-K'.  Selection words
+// and counts are then assembled in LDS and written out like the small kernel's.
+// ------------------------------------------------------------------------------------
+constexpr int kBigCap = 32;  // running winners per row (K' = scored chunks kept)
+
+template <typename T, int HD, int NT>
+__global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
+  constexpr int KS = HD / 16;
+  constexpr int LD = HD + 16;
+  constexpr int GC = NT * 32;        // chunks per group
+  constexpr int PL = kBigCap / 2;    // previous winners held per lane (two lanes per row)
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint16_t *sKm = reinterpret_cast<uint16_t *>(smem);
+  uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [W][128], reuses the chunk-mean tile after the last group
+  float *sVal = reinterpret_cast<float *>(smem + (size_t)GC * LD * 2);   // [2][128][kBigCap]
+  int *sIdx = reinterpret_cast<int *>(sVal + 2 * kGateRows * kBigCap);   // [2][128][kBigCap]
+  int *sCnt = sIdx + 2 * kGateRows * kBigCap;                            // [2][128]
+  int *sHist = sCnt + 2 * kGateRows;                                     // [max_cols]
+
+  const fmoba_fused_topk_args &a = p.a;
+  const int mb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int q0 = a.cu_seqlens_q[b];
+  const int Lq = a.cu_seqlens_q[b + 1] - q0;
+  const int m0 = mb * kGateRows;
+  if (m0 >= Lq) return;
+  const int Lk = a.cu_seqlens_k[b + 1] - a.cu_seqlens_k[b];
+  const int km0 = a.cu_seqlens_km[b];
+  const int Cb = min(a.cu_seqlens_km[b + 1] - km0, p.max_cols);
+  const int off = Lk - Lq;
+  const int B = a.chunk;
+  const int D = a.head_dim;
+  const int hk = h / (a.heads / a.heads_k);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
+  const int rs = wave * 32 + (lane & 31);  // row slot inside the block
+
+  int nsc;  // chunks [0, nsc) can be candidates of some row of this block
+  if (a.is_causal) {
+    const int rmax = min(m0 + kGateRows - 1, Lq - 1) + off;
+    nsc = rmax < 0 ? 0 : min(Cb, rmax / B);
+  } else {
+    nsc = Cb;
+  }
+  const int ngroups = (nsc + GC - 1) / GC;
+
+  const int r = m0 + rs;
+  const bool valid = r < Lq;
+  Pack8 qf[KS];
+  {
+    const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)(q0 + (valid ? r : 0)) * a.q_row_stride + (int64_t)h * a.q_head_stride;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int e = (hh * KS + ks) * 8;
+      qf[ks] = (valid && e < D) ? ld_global16(qp + e) : zero_pack8();
+    }
+  }
+  const int rp = r + off;
+  int nc;  // candidate chunks of this row: chunks strictly before its own chunk
+  if (a.is_causal)
+    nc = (valid && rp >= 0) ? min(rp / B, Cb) : 0;
+  else
+    nc = valid ? Cb : 0;
+  const int kp = a.is_causal ? a.topk - 1 : a.topk;
+
+  if (tid < 2 * kGateRows) sCnt[tid] = 0;
+  int cur = 0;
+  const uint16_t *kmp = reinterpret_cast<const uint16_t *>(a.km) + (int64_t)hk * a.km_head_stride;
+  for (int g = 0; g < ngroups; ++g) {
+    const int c0 = g * GC;
+    const int gsc = min(GC, nsc - c0);
+    const int n_tiles = (gsc + 31) >> 5;
+    __syncthreads();  // the previous group's tile and lists are no longer read
+    {
+      const int vecs = HD / 8;
+      for (int v = tid; v < n_tiles * 32 * vecs; v += 256) {
+        const int c = v / vecs, e = (v - c * vecs) * 8;
+        Pack8 x = zero_pack8();
+        if (c < gsc && e < D) x = ld_global16(kmp + (int64_t)(km0 + c0 + c) * a.km_row_stride + e);
+        *reinterpret_cast<Pack8 *>(sKm + c * LD + e) = x;
+      }
+    }
+    const int nxt = cur ^ 1;
+    if (hh == 0) sCnt[nxt * kGateRows + rs] = 0;
+    __syncthreads();
+
+    // this group's scores and the winners so far
+    float sc[NT][16];
+    float pv[PL];
+    int pi[PL];
+    const int m_prev = sCnt[cur * kGateRows + rs];
+    float vmin = INFINITY, vmax = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PL; ++j) {
+      const int e = hh * PL + j;
+      const bool ok = e < m_prev;
+      pv[j] = ok ? sVal[(cur * kGateRows + rs) * kBigCap + e] : -INFINITY;
+      pi[j] = ok ? sIdx[(cur * kGateRows + rs) * kBigCap + e] : -1;
+      vmin = fminf(vmin, ok ? pv[j] : INFINITY);
+      vmax = fmaxf(vmax, pv[j]);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (t < n_tiles) {
+        f32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const Pack8 af = *reinterpret_cast<const Pack8 *>(sKm + (t * 32 + (lane & 31)) * LD + (hh * KS + ks) * 8);
+          acc = mfma32<T>(af, qf[ks], acc);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int c = c0 + t * 32 + acc_row(i, hh);
+          const bool cand = c < nc;
+          const float x = acc[i];
+          sc[t][i] = cand ? x : -INFINITY;
+          vmin = fminf(vmin, cand ? x : INFINITY);
+          vmax = fmaxf(vmax, sc[t][i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[t][i] = -INFINITY;
+      }
+    }
+    vmin = min_xor32_f(vmin);
+    vmax = max_xor32_f(vmax);
+    const int ntot = m_prev + max(0, min(nc - c0, GC));  // candidates that compete in this group
+    const bool need = (ntot > kp) && (kp > 0);
+
+    auto count_gt = [&](float probe) {
+      int cnt = 0;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) cnt += (sc[t][i] > probe) ? 1 : 0;
+        }
+#pragma unroll
+      for (int j = 0; j < PL; ++j) cnt += (pv[j] > probe) ? 1 : 0;
+      return sum_xor32_i(cnt);
+    };
+    float tau = -INFINITY, tau_eq = INFINITY;
+    int n_eq = 0;
+    uint32_t iota = 0u;
+    {
+      uint32_t lo_k = float_order_key(vmin) - 1u;
+      uint32_t hi_k = float_order_key(vmax);
+      int c_hi = 0;
+      bool open = need;
+      for (int iter = 0;; ++iter) {
+        if (open && hi_k - lo_k <= 1u) {
+          tau = order_key_float(hi_k);
+          if (tau != -INFINITY) {
+            tau_eq = tau;
+            n_eq = kp - c_hi;
+          }
+          open = false;
+        }
+        if (!__any(open)) break;
+        uint32_t pk = lo_k + ((hi_k - lo_k) >> 1);
+        if (iter < 12) {
+          const float mf = 0.5f * order_key_float(lo_k + 1u) + 0.5f * order_key_float(hi_k);
+          const uint32_t mk = float_order_key(mf);
+          if (mk > lo_k && mk < hi_k) pk = mk;
+        }
+        const float probe = order_key_float(pk);
+        const int cnt = count_gt(probe);
+        if (open) {
+          if (cnt == kp) {
+            tau = probe;
+            open = false;
+          } else if (cnt > kp) {
+            lo_k = pk;
+          } else {
+            hi_k = pk;
+            c_hi = cnt;
+          }
+        }
+      }
+      const bool tie = n_eq > 0;
+      if (__any(tie)) {
+        auto count_eq_ge = [&](uint32_t trial) {
+          int cnt = 0;
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            if (t < n_tiles) {
+#pragma unroll
+              for (int i = 0; i < 16; ++i) {
+                const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
+                cnt += (sc[t][i] == tau_eq && c >= trial) ? 1 : 0;
+              }
+            }
+#pragma unroll
+          for (int j = 0; j < PL; ++j) cnt += (pv[j] == tau_eq && (uint32_t)pi[j] >= trial && pi[j] >= 0) ? 1 : 0;
+          return sum_xor32_i(cnt);
+        };
+        const int ceq = count_eq_ge(0u);
+        const bool split = tie && ceq > n_eq;
+        if (__any(split)) {
+          uint32_t i_acc = 0u;
+          for (int bit = 23; bit >= 0; --bit) {
+            const uint32_t trial = i_acc | (1u << bit);
+            const int cnt = count_eq_ge(trial);
+            if (cnt >= n_eq) i_acc = trial;
+          }
+          if (split) iota = i_acc;
+        }
+      }
+    }
+
+    // winners of this round -> the other list: count per lane, reserve slots once, then store
+    int nwin = 0;
+    if (kp > 0) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
+            const float x = sc[t][i];
+            nwin += ((x > tau) || (x == tau_eq && c >= iota)) ? 1 : 0;
+          }
+        }
+#pragma unroll
+      for (int j = 0; j < PL; ++j) nwin += (pi[j] >= 0 && ((pv[j] > tau) || (pv[j] == tau_eq && (uint32_t)pi[j] >= iota))) ? 1 : 0;
+    }
+    int slot = 0;
+    if (nwin > 0) slot = atomicAdd(&sCnt[nxt * kGateRows + rs], nwin);
+    float *ov = sVal + (size_t)(nxt * kGateRows + rs) * kBigCap;
+    int *oi = sIdx + (size_t)(nxt * kGateRows + rs) * kBigCap;
+    if (nwin > 0) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
+            const float x = sc[t][i];
+            if (((x > tau) || (x == tau_eq && c >= iota)) && slot < kBigCap) {
+              ov[slot] = x;
+              oi[slot] = (int)c;
+              ++slot;
+            }
+          }
+        }
+#pragma unroll
+      for (int j = 0; j < PL; ++j)
+        if (pi[j] >= 0 && ((pv[j] > tau) || (pv[j] == tau_eq && (uint32_t)pi[j] >= iota)) && slot < kBigCap) {
+          ov[slot] = pv[j];
+          oi[slot] = pi[j];
+          ++slot;
+        }
+    }
+    cur = nxt;
+  }
+  __syncthreads();
+
+  // selection words and per-chunk counts of the block, assembled in LDS
+  for (int v = tid; v < p.W * kGateRows; v += 256) sSel[v] = 0u;
+  for (int c = tid; c < p.max_cols; c += 256) sHist[c] = 0;
+  __syncthreads();
+  if (valid) {
+    const int m = min(sCnt[cur * kGateRows + rs], kBigCap);
+#pragma unroll
+    for (int j = 0; j < PL; ++j) {
+      const int e = hh * PL + j;
+      if (e < m) {
+        const int c = sIdx[(cur * kGateRows + rs) * kBigCap + e];
+        atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
+        atomicAdd(&sHist[c], 1);
+      }
+    }
+    if (hh == 0 && a.is_causal && rp >= 0) {
+      const int c = rp / B;  // the own chunk is always selected
+      if (c < p.max_cols) {
+        atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
+        atomicAdd(&sHist[c], 1);
+      }
+    }
+  }
+  __syncthreads();
+  for (int v = tid; v < p.W * kGateRows; v += 256) {
+    const int t = v / kGateRows, slot_r = v - t * kGateRows;
+    if (m0 + slot_r < Lq) p.sel[((int64_t)h * p.W + t) * a.total_q + q0 + m0 + slot_r] = sSel[v];
+  }
+  const int seg = m0 / kSegRows;
+  for (int c = tid; c < p.max_cols; c += 256) {
+    const int v = sHist[c];
+    if (v) atomicAdd(&p.segcnt[(((int64_t)b * a.heads + h) * p.nseg + seg) * p.max_cols + c], v);
+  }
+}
+
 // grid (heads, batch), block 256
 __global__ __launch_bounds__(256) void csc_scan_kernel(TopkParams p) {
   const fmoba_fused_topk_args &a = p.a;
@@ -463,6 +760,28 @@ static int launch_gate_nt(const TopkParams &p, dim3 grid, hipStream_t s) {
   if (p.W <= 4) return launch_gate<T, HD, 4>(p, grid, s);
   return launch_gate<T, HD, 8>(p, grid, s);
 }
+template <typename T, int HD, int NT>
+static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
+  const size_t tile = (size_t)NT * 32 * (HD + 16) * 2;
+  const size_t smem = tile + (size_t)2 * kGateRows * kBigCap * 8 + (size_t)2 * kGateRows * 4 + (size_t)p.max_cols * 4;
+  if ((size_t)p.W * kGateRows * 4 > tile || smem > 160 * 1024) {
+    set_error("fused_topk: %d key chunks per sequence exceed what the LDS of this build holds", p.max_cols);
+    return 1;
+  }
+  auto kern = topk_gate_big_kernel<T, HD, NT>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+    set_error("fused_topk: cannot reserve %zu bytes of LDS", smem);
+    return 2;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), smem, s, p);
+  return 0;
+}
+template <typename T>
+static int launch_gate_big_hd(const TopkParams &p, dim3 grid, hipStream_t s) {
+  if (p.a.head_dim <= 64) return launch_gate_big<T, 64, 8>(p, grid, s);
+  if (p.a.head_dim <= 128) return launch_gate_big<T, 128, 8>(p, grid, s);
+  return launch_gate_big<T, 256, 4>(p, grid, s);
+}
 template <typename T>
 static int launch_gate_hd(const TopkParams &p, dim3 grid, hipStream_t s) {
   if (p.a.head_dim <= 64) return launch_gate_nt<T, 64>(p, grid, s);
@@ -503,9 +822,12 @@ extern "C" int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream) {
     FMOBA_LAUNCH_CHECK("fused_topk(empty)");
     return 0;
   }
-  FMOBA_REQUIRE(max_cols <= 256,
-                "fused_topk: at most 256 key chunks per sequence are supported by this build (got %d = ceil(%d / %d))",
-                max_cols, a->max_seqlen_k, a->chunk);
+  const bool big = max_cols > 256;  // more chunks than the register-resident gate holds: grouped gate
+  if (big) {
+    const int kp = a->is_causal ? a->topk - 1 : a->topk;
+    FMOBA_REQUIRE(kp <= kBigCap, "fused_topk: with more than 256 key chunks per sequence moba_topk is limited to %d (got %d)",
+                  kBigCap + (a->is_causal ? 1 : 0), a->topk);
+  }
   FMOBA_REQUIRE(a->q && a->km, "fused_topk: null q/km pointer");
   FMOBA_REQUIRE(a->q_row_stride % 8 == 0 && a->q_head_stride % 8 == 0 && a->km_row_stride % 8 == 0 && a->km_head_stride % 8 == 0,
                 "fused_topk: strides must be multiples of 8 elements");
@@ -538,7 +860,11 @@ extern "C" int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream) {
 
   hipLaunchKernelGGL(fill_i32_kernel, dim3(512), dim3(256), 0, s, p.segcnt, (int64_t)(seg_bytes / 4), 0);
   dim3 ggrid(ceil_div(a->max_seqlen_q, kGateRows), a->heads, a->batch);
-  int rc = (a->dtype == FMOBA_DTYPE_BF16) ? launch_gate_hd<bf16_t>(p, ggrid, s) : launch_gate_hd<f16_t>(p, ggrid, s);
+  int rc;
+  if (big)
+    rc = (a->dtype == FMOBA_DTYPE_BF16) ? launch_gate_big_hd<bf16_t>(p, ggrid, s) : launch_gate_big_hd<f16_t>(p, ggrid, s);
+  else
+    rc = (a->dtype == FMOBA_DTYPE_BF16) ? launch_gate_hd<bf16_t>(p, ggrid, s) : launch_gate_hd<f16_t>(p, ggrid, s);
   if (rc) return rc;
   FMOBA_LAUNCH_CHECK("topk_gate_kernel");
   hipLaunchKernelGGL(csc_scan_kernel, dim3(a->heads, a->batch), dim3(256), 0, s, p);
