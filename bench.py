@@ -37,6 +37,7 @@ CONFIGS = {
     "headline": (None, 16, 128, 64, 32, True),
     "c2": ([8192], 16, 128, 128, 8, False),
     "c3": ([32768], 32, 128, 128, 16, True),
+    "c5": ([262144], 16, 128, 128, 16, True),
 }
 
 

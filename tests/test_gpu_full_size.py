@@ -146,3 +146,68 @@ def test_config4_headline_fwd_bwd_64k(mods):
     lhs, rhs = f(v + v2), f(v) + f(v2)
     assert bool(((lhs - rhs).abs() <= 4e-2 + 2e-2 * rhs.abs()).all())
     assert torch.equal(f(v).to(torch.bfloat16), out.detach())      # forward is deterministic
+
+
+def _row_reference(q, k, v, dout, km, chunk, topk, r, h, scale):
+    """fp32 gate -> top-k (own chunk forced, ties to the higher chunk) -> masked softmax attention of ONE
+    query row of a single self-attention sequence, with its dQ (flash_moba/moba_test_utils naive path, row-wise)."""
+    L = q.shape[0]
+    own = r // chunk
+    gate = km[:own, h].float() @ q[r, h].float()
+    sel = torch.zeros((L + chunk - 1) // chunk, dtype=torch.bool, device=q.device)
+    sel[own] = True
+    gap_ok = True
+    if own > 0 and topk > 1:
+        kk = min(topk - 1, own)
+        # total order (score desc, chunk desc): stable sort of the reversed list
+        order = torch.argsort(gate.flip(0), descending=True, stable=True)
+        idx = own - 1 - order
+        sel[idx[:kk]] = True
+        if own > kk:
+            a_, b_ = gate[idx[kk - 1]], gate[idx[kk]]
+            gap_ok = bool((a_ - b_).abs() > 1e-3 * torch.maximum(a_.abs(), b_.abs()))
+    mask = sel.repeat_interleave(chunk)[:L] & (torch.arange(L, device=q.device) <= r)
+    kk_, vv_ = k[mask, h].float(), v[mask, h].float()
+    s = (kk_ @ q[r, h].float()) * scale
+    p = torch.softmax(s, 0)
+    o = p @ vv_
+    dp = vv_ @ dout[r, h].float()
+    ds = p * (dp - (dout[r, h].float() * o).sum())
+    dq = scale * (ds @ kk_)
+    return o, dq, gap_ok
+
+
+def test_config5_long_context_262k(mods):
+    api, pool = mods
+    L, H, D, chunk, topk = 262144, 16, 128, 128, 16
+    q, k, v, dout, cu = _inputs([L], H, D, chunk, 1005)
+    co, cn, ind = api.flash_topk_varlen_func(q, k, cu, cu, L, L, topk, chunk, causal=True)
+    assert co.shape == (1, H, 2048) and co.dtype == torch.int64
+    _check_csc(co, cn, ind, [L], H, chunk, topk)
+    # the last list ends where the last head's region ends minus the slots the first topk-1 chunks leave unused
+    assert int(co[0, -1, -1]) + int(cn[0, -1, -1]) == L * H * topk - chunk * (topk * (topk - 1) // 2)
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    out = api.flash_moba_varlen_func(qg, kg, vg, cu, cu, L, L, chunk, topk, causal=True)
+    out.backward(dout)
+    torch.cuda.synchronize()
+    km, cu_km, _ = pool.flash_topk_mean_pool(k, cu, L, chunk)
+    scale = D ** -0.5
+    checked = 0
+    for h in (0, 9):
+        for r in (0, 1, 127, 128, 129, 4999, 65536, 131071, 200000, 262143):
+            o_ref, dq_ref, gap_ok = _row_reference(q, k, v, dout, km, chunk, topk, r, h, scale)
+            if not gap_ok:
+                continue
+            checked += 1
+            assert bool(((out[r, h].float() - o_ref).abs() <= 2e-2 + 1e-2 * o_ref.abs()).all()), (r, h)
+            assert bool(((qg.grad[r, h].float() - dq_ref).abs() <= 2e-2 + 1e-2 * dq_ref.abs()).all()), (r, h)
+    assert checked >= 16
+    # every probability row sums to one: sum_j dV_j = sum_r dO_r, per head and feature
+    lhs, rhs = vg.grad.float().sum(0), dout.float().sum(0)
+    assert bool(((lhs - rhs).abs() <= 2e-2 * rhs.abs().max()).all()), (lhs - rhs).abs().max().item()
+    # S = scale * Q K^T is bilinear: sum_r <q_r, dQ_r> = sum_j <k_j, dK_j>, per head.  Both gradients are rounded to
+    # bf16 (relative 2^-9 per element, independent), so the two sums differ by about 2^-9 * sqrt(sum of squared terms).
+    tq, tk = qg.grad.float() * q.float(), kg.grad.float() * k.float()
+    eq, ek = tq.sum((0, 2)), tk.sum((0, 2))
+    noise = 2.0 ** -9 * torch.sqrt((tq * tq).sum((0, 2)) + (tk * tk).sum((0, 2)))
+    assert bool(((eq - ek).abs() <= 8 * noise + 1e-3 * eq.abs()).all()), (eq, ek, noise)
