@@ -212,8 +212,13 @@ def main():
     km, cu_km, _ = mean_pool_nosync(kd, cu, max_len, chunk)
     t_pool = time_events(lambda: mean_pool_nosync(kd, cu, max_len, chunk), it)
     t_gate = time_events(lambda: hip.moba_fused_topk(qd, km, cu, cu, cu_km, max_len, max_len, topk, chunk, True, return_raw=False), it)
-    fwd = lambda: hip.moba_varlen_fwd(qd, kd, vd, None, co, cn, ind, cu, cu, None, None, None, max_len, max_len, 0.0, scale,
-                                      False, True, 0.0, False, lg_m, chunk, None)
+    visits = topk * (chunk // hip.fwd_key_block(chunk))  # the bound the gated path hands to the forward
+
+    def fwd():
+        hip.set_visits_hint(visits)
+        return hip.moba_varlen_fwd(qd, kd, vd, None, co, cn, ind, cu, cu, None, None, None, max_len, max_len, 0.0, scale,
+                                   False, True, 0.0, False, lg_m, chunk, None)
+
     out, lse, _, _ = fwd()
     t_fwd = time_events(fwd, it)
     stages = {

@@ -1,46 +1,57 @@
-// Sparse (gather-and-densify) flash attention forward over a CSC pattern.
+// Sparse attention forward over a CSC pattern, column-stationary, in two launches.
 //
-// One workgroup owns a SUPERBLOCK of 128 consecutive query rows of one (sequence, head).
-// The superblock's Q rows (bf16), its fp32 output accumulators and its running softmax
-// statistics stay in LDS for the whole kernel; nothing partial is ever written to HBM.
-// For every key chunk the rows of the superblock that selected it are found in the
-// chunk's ascending row list, gathered from LDS into dense 32-row MFMA tiles and
-// processed with S^T = K Q^T (so that one lane owns one query row: the online-softmax
-// reductions are in-register) followed by O^T += V^T P^T, where V^T fragments come from
-// transposing LDS reads and P^T goes from the S^T accumulators straight into the MFMA
-// operand registers.
+//   attn_fwd_col_kernel     : one workgroup per (key block of KB = 64 or 128 keys, head,
+//                             sequence).  K of the block lives in MFMA operand registers, V in
+//                             LDS; the block's ascending row list is walked in gathered 32-row
+//                             tiles: S^T = K Q^T (one lane owns one query row, so the softmax
+//                             reductions over the block's keys stay in registers), P^T goes from
+//                             the accumulators straight into the operand registers of
+//                             O^T = V^T P^T (V^T through transposing LDS reads).  Every visit of
+//                             a (row, key block) pair leaves a PARTIAL result: the block-local
+//                             maximum m, the sum l of exp2(s - m) and the unnormalised output row
+//                             (16-bit), in a slot that the row hands out from a counter.
+//   attn_fwd_combine_kernel : one wave per (row, head) merges the row's partials in ascending
+//                             key-block order (sorted by block id, so the result does not depend
+//                             on which slot a visit happened to get): out, log-sum-exp.
+//
+// Work and traffic are proportional to the number of (row, key block) visits whatever the number of
+// chunks per sequence; a row-stationary formulation degenerates when every 128-row block touches
+// thousands of chunks with one or two rows each.
+// In the first kernel waves 0,1 compute (one tile each per round) and waves 2,3 only move data
+// (global -> registers -> LDS), two rounds ahead.
 #include "fmoba_common.h"
 
 #include <type_traits>
+#include <utility>
 
 namespace fmoba {
 
-constexpr int kSuperRows = 128;
-constexpr int kColBatch = 256;   // columns whose list ranges are resolved per batch
-constexpr int kMaxSteps = 512;   // (column, 64-key block) steps per batch
+constexpr int kFwdListCap = 4096;  // rows of a column list held in LDS at a time
 
-template <int HD>
-struct FwdSmem {
-  static constexpr int LDQ = HD + 16;  // elements, Q / K / V tiles
-  static constexpr int LDO = HD + 4;   // floats, output accumulators
-  static constexpr int LDP = 64 + 8;   // elements, probability tile [32 rows][64 keys]
-  static constexpr size_t oO = 0;
-  static constexpr size_t oQ = oO + (size_t)kSuperRows * LDO * 4;
-  static constexpr size_t oK = oQ + (size_t)kSuperRows * LDQ * 2;
-  static constexpr size_t oV = oK + (size_t)64 * LDQ * 2;
-  static constexpr size_t oP = oV + (size_t)64 * LDQ * 2;          // [2][32][LDP]
-  static constexpr size_t oM = oP + (size_t)2 * 32 * LDP * 2;
-  static constexpr size_t oL = oM + kSuperRows * 4;
-  static constexpr size_t oRows = oL + kSuperRows * 4;             // int[2][kSuperRows]
-  static constexpr size_t oAlpha = oRows + 2 * kSuperRows * 4;     // float[2][32]
-  static constexpr size_t oRid = oAlpha + 2 * 32 * 4;              // int[2][32]
-  static constexpr size_t oLo = oRid + 2 * 32 * 4;                 // int[kColBatch]
-  static constexpr size_t oCnt = oLo + kColBatch * 4;              // int[kColBatch]
-  static constexpr size_t oStep = oCnt + kColBatch * 4;            // int[kMaxSteps]: (column - batch start) << 8 | key block
-  static constexpr size_t oOff = oStep + kMaxSteps * 4;            // int64[kColBatch]: list position of the first entry
-  static constexpr size_t oMisc = oOff + kColBatch * 8;            // int[16]
-  static constexpr size_t bytes = oMisc + 64;
+// NCW compute waves (one 32-row tile each per round) + 2 loader waves
+template <int HD, int KB, int NCW>
+struct FwdColSmem {
+  static constexpr int RR = 32 * NCW;  // rows per round
+  static constexpr int LDQ = HD + 16;  // elements, K / V / Q tiles (conflict-free for the 16-byte row reads and the transposing reads)
+  static constexpr int LDO = HD + 8;   // elements, per-wave output tile [32 rows][LDO]
+  static constexpr size_t oK = 0;
+  static constexpr size_t oV = oK + (size_t)KB * LDQ * 2;
+  static constexpr size_t oQ = oV + (size_t)KB * LDQ * 2;            // [2 buffers][RR rows][LDQ]
+  static constexpr size_t oOut = oQ + (size_t)2 * RR * LDQ * 2;      // [NCW waves][32][LDO]
+  static constexpr size_t oRow = oOut + (size_t)NCW * 32 * LDO * 2;  // int[2][RR]
+  static constexpr size_t oSlot = oRow + 2 * RR * 4;                 // int[2][RR]
+  static constexpr size_t oList = oSlot + 2 * RR * 4;                // int[kFwdListCap]
+  static constexpr size_t bytes = oList + (size_t)kFwdListCap * 4;
 };
+
+template <typename F, int... I>
+__device__ __forceinline__ void fwd_static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void fwd_static_for(F &&f) {
+  fwd_static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 __device__ __forceinline__ int lower_bound_i32(const int32_t *p, int n, int v) {
   int lo = 0, hi = n;
@@ -54,381 +65,378 @@ __device__ __forceinline__ int lower_bound_i32(const int32_t *p, int n, int v) {
   return lo;
 }
 
-// Work items are (sequence, head, superblock).  Hardware deals consecutive workgroup ids
-// round-robin to the 8 XCDs, each with its own L2.  The id is decoded so that all
-// superblocks of one (sequence, head) pair run on ONE XCD (pair p lives on XCD p % 8) and
-// consecutively, so that their K/V re-reads hit that XCD's L2; inside a pair the late
-// superblocks (most key chunks, longest running) are issued first.
-struct WorkItem {
-  int pair, sb;
+struct FwdWs {
+  int32_t *cnt;      // [total_q * heads] visits handed out per (row, head)
+  float4 *hdr;       // [total_q * heads * cap] {m (log2 domain), l, key block id, -}
+  uint16_t *part;    // [total_q * heads * cap][head_dim] unnormalised partial outputs
+  int32_t cap;
 };
-__device__ __forceinline__ WorkItem decode_item(int id, int npairs, int nsb_max) {
-  const int x = id & 7, s = id >> 3;
-  const int pl = s / nsb_max, sbi = s - pl * nsb_max;
-  WorkItem w;
-  w.pair = pl * 8 + x;
-  w.sb = nsb_max - 1 - sbi;
-  if (w.pair >= npairs) w.pair = -1;
-  return w;
-}
 
-// The four waves of a workgroup form a two-stage pipeline over gathered 32-row tiles:
-//   waves 0,1 ("score" stage, 16 rows each): gather Q rows from LDS, S^T = K Q^T on
-//       16x16x32 MFMAs (one lane group of 4 owns one query row), causal/length mask, online
-//       softmax statistics (kept in LDS per superblock row), probabilities -> LDS as bf16;
-//   waves 2,3 ("value" stage, 64 output columns each): O^T += V^T P^T on 32x32x16 MFMAs
-//       (V^T through transposing LDS reads), then read-modify-write of the fp32 output rows.
-// In slot k the score stage works on tile k while the value stage works on tile k-1, so the
-// four SIMDs are busy even when a key chunk has a single tile.  Row statistics are only
-// touched by the score stage and output rows only by the value stage, both in tile order,
-// so results do not depend on timing.
-template <typename T, int HD>
-__global__ __launch_bounds__(512) void attn_fwd_kernel(fmoba_attn_fwd_args a, int nsb_max) {
-  typedef FwdSmem<HD> SM;
-  constexpr int LDQ = SM::LDQ, LDO = SM::LDO, LDP = SM::LDP, NDT = HD / 32, VPR = HD / 8;
-  constexpr int KS4 = HD / 32;         // k-steps of a 16x16x32 MFMA over the head dimension
-  constexpr int KVV = 64 * VPR / 256;  // 16-byte vectors of a K (or V) tile per thread
+template <typename T, int HD, int KB, int NCW>
+__global__ __launch_bounds__((NCW + 2) * 64) void attn_fwd_col_kernel(fmoba_attn_fwd_args a, FwdWs ws) {
+  typedef FwdColSmem<HD, KB, NCW> SM;
+  constexpr int NTHR = (NCW + 2) * 64, RR = SM::RR;
+  constexpr int KS = HD / 16, LDQ = SM::LDQ, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
+  constexpr int KT = KB / 32;                 // 32-key tiles of the block
+  constexpr int NV = RR * VPR / 128;          // 16-byte vectors of a round's gathered Q rows per loader thread
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float *sO = reinterpret_cast<float *>(smem + SM::oO);
-  uint16_t *sQ = reinterpret_cast<uint16_t *>(smem + SM::oQ);
   uint16_t *sK = reinterpret_cast<uint16_t *>(smem + SM::oK);
   uint16_t *sV = reinterpret_cast<uint16_t *>(smem + SM::oV);
-  uint16_t *sP = reinterpret_cast<uint16_t *>(smem + SM::oP);
-  float *sM = reinterpret_cast<float *>(smem + SM::oM);
-  float *sL = reinterpret_cast<float *>(smem + SM::oL);
-  int *sRows = reinterpret_cast<int *>(smem + SM::oRows);
-  float *sAlpha = reinterpret_cast<float *>(smem + SM::oAlpha);
-  int *sRid = reinterpret_cast<int *>(smem + SM::oRid);
-  int *sLo = reinterpret_cast<int *>(smem + SM::oLo);
-  int *sCnt = reinterpret_cast<int *>(smem + SM::oCnt);
-  int *sStep = reinterpret_cast<int *>(smem + SM::oStep);
-  int *sMisc = reinterpret_cast<int *>(smem + SM::oMisc);
-  int64_t *sOff = reinterpret_cast<int64_t *>(smem + SM::oOff);
+  uint16_t *sQ = reinterpret_cast<uint16_t *>(smem + SM::oQ);
+  int *sRow = reinterpret_cast<int *>(smem + SM::oRow);
+  int *sSlot = reinterpret_cast<int *>(smem + SM::oSlot);
+  int *sList = reinterpret_cast<int *>(smem + SM::oList);
 
-  const WorkItem wi = decode_item(blockIdx.x, a.heads * a.batch, nsb_max);
-  if (wi.pair < 0) return;
-  const int b = wi.pair / a.heads, h = wi.pair - b * a.heads, sb = wi.sb;
-  const int q0 = a.cu_seqlens_q[b], Lq = a.cu_seqlens_q[b + 1] - q0;
-  const int m0 = sb * kSuperRows;
-  if (m0 >= Lq) return;
+  const int nb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
-  const int rows_sb = min(kSuperRows, Lq - m0);
+  const int key0 = nb * KB;
+  if (key0 >= Lk) return;
+  const int q0 = a.cu_seqlens_q[b], Lq = a.cu_seqlens_q[b + 1] - q0;
   const int off = Lk - Lq;
   const int D = a.head_dim;
   const int hk = h / (a.heads / a.heads_k);
-  const int Bn = a.lg_block_n;
-  const int nsub = Bn / 64;
-  // waves 0,1: score stage; waves 2,3: value stage; waves 4..7: loaders (global -> registers -> LDS)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
-  const bool is_loader = tid >= 256;
-  const int ltid = tid & 255;
-  const float scale_log2 = a.softmax_scale * 1.4426950408889634f;
+  const bool is_loader = wave >= NCW;
+  const int lt = tid - NCW * 64;
   const bool causal = a.is_causal != 0;
+  const float scale_log2 = a.softmax_scale * 1.4426950408889634f;
 
-  // ---- superblock state -------------------------------------------------------------
+  // ---- K and V of the block ------------------------------------------------------------------
   {
-    const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)(q0 + m0) * a.q_row_stride + (int64_t)h * a.q_head_stride;
-    for (int v = tid; v < kSuperRows * VPR; v += 512) {
-      const int row = v / VPR, e = (v - row * VPR) * 8;
-      Pack8 x = zero_pack8();
-      if (row < rows_sb && e < D) x = ld_global16(qp + (int64_t)row * a.q_row_stride + e);
-      *reinterpret_cast<Pack8 *>(sQ + row * LDQ + e) = x;
-    }
-    for (int v = tid; v < kSuperRows * LDO; v += 512) sO[v] = 0.f;
-    if (tid < kSuperRows) {
-      sM[tid] = -INFINITY;
-      sL[tid] = 0.f;
-    }
-  }
-
-  int ncols = min((Lk + Bn - 1) / Bn, a.max_cols);
-  const int last_rowpos = m0 + rows_sb - 1 + off;  // largest visible key index of the superblock (causal)
-  if (causal) ncols = last_rowpos < 0 ? 0 : min(ncols, last_rowpos / Bn + 1);
-  const int64_t bh = (int64_t)b * a.heads + h;
-  const int64_t *coff = a.col_offsets + bh * a.max_cols;
-  const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + (int64_t)k0 * a.k_row_stride + (int64_t)hk * a.k_head_stride;
-  const uint16_t *vp = reinterpret_cast<const uint16_t *>(a.v) + (int64_t)k0 * a.v_row_stride + (int64_t)hk * a.v_head_stride;
-  const int cols_per_batch = min(kColBatch, kMaxSteps / nsub);
-
-  // Two-deep register rings carry the K tiles (+ row lists) and, separately, the V tiles of
-  // the next two steps from global memory to LDS, so that a load has two pipeline slots to
-  // complete.  Ring entries are picked by compile-time parity (no dynamic register indexing).
-  Pack8 pk0[KVV], pk1[KVV], pv0[KVV], pv1[KVV];
-  int prow0 = 0, prow1 = 0;
-  auto step_key0 = [&](int cb, int step) {
-    const int code = sStep[step];
-    return (cb + (code >> 8)) * Bn + (code & 255) * 64;
-  };
-  auto load_tile = [&](Pack8(&dst)[KVV], const uint16_t *base, int64_t row_stride, int key0) {
-#pragma unroll
-    for (int i = 0; i < KVV; ++i) {
-      const int v = ltid + i * 256;
+    const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + (int64_t)(k0 + key0) * a.k_row_stride + (int64_t)hk * a.k_head_stride;
+    const uint16_t *vp = reinterpret_cast<const uint16_t *>(a.v) + (int64_t)(k0 + key0) * a.v_row_stride + (int64_t)hk * a.v_head_stride;
+    for (int v = tid; v < KB * VPR; v += NTHR) {
       const int key = v / VPR, e = (v - key * VPR) * 8;
-      dst[i] = zero_pack8();
-      if (key0 + key < Lk && e < D) dst[i] = ld_global16(base + (int64_t)(key0 + key) * row_stride + e);
-    }
-  };
-  auto store_tile = [&](const Pack8(&src)[KVV], uint16_t *dst) {
-#pragma unroll
-    for (int i = 0; i < KVV; ++i) {
-      const int v = ltid + i * 256;
-      const int key = v / VPR, e = (v - key * VPR) * 8;
-      *reinterpret_cast<Pack8 *>(dst + key * LDQ + e) = src[i];
-    }
-  };
-  auto load_k = [&](auto par, int cb, int step) {
-    const int cl = sStep[step] >> 8;
-    if constexpr (decltype(par)::value == 0) {
-      load_tile(pk0, kp, a.k_row_stride, step_key0(cb, step));
-      if (ltid < sCnt[cl]) prow0 = a.row_indices[sOff[cl] + ltid];  // raw value: any arithmetic here would wait for the load
-    } else {
-      load_tile(pk1, kp, a.k_row_stride, step_key0(cb, step));
-      if (ltid < sCnt[cl]) prow1 = a.row_indices[sOff[cl] + ltid];
-    }
-  };
-  auto load_v = [&](auto par, int cb, int step) {
-    if constexpr (decltype(par)::value == 0)
-      load_tile(pv0, vp, a.v_row_stride, step_key0(cb, step));
-    else
-      load_tile(pv1, vp, a.v_row_stride, step_key0(cb, step));
-  };
-  auto store_k = [&](auto par, int step, int n) {
-    if constexpr (decltype(par)::value == 0) {
-      store_tile(pk0, sK);
-      if (ltid < n) sRows[(step & 1) * kSuperRows + ltid] = prow0 - m0;
-    } else {
-      store_tile(pk1, sK);
-      if (ltid < n) sRows[(step & 1) * kSuperRows + ltid] = prow1 - m0;
-    }
-  };
-  auto store_v = [&](auto par) {
-    if constexpr (decltype(par)::value == 0)
-      store_tile(pv0, sV);
-    else
-      store_tile(pv1, sV);
-  };
-
-  // ---- score stage: one 16-row half of a tile ----------------------------------------------
-  auto score_stage = [&](int step, int key0, int n, int tile, int buf) {
-    const int l16 = lane & 15, g = lane >> 4;
-    const int slot = 16 * wave + l16;              // row slot inside the 32-row tile
-    const int ridx = tile * 32 + slot;
-    const bool valid = ridx < n;
-    const int rid = valid ? (sRows[(step & 1) * kSuperRows + ridx] & (kSuperRows - 1)) : 0;
-    Pack8 qf[KS4];
-#pragma unroll
-    for (int ks = 0; ks < KS4; ++ks) qf[ks] = *reinterpret_cast<const Pack8 *>(sQ + rid * LDQ + (g * KS4 + ks) * 8);
-    // S^T: register i of key tile kt holds key key0 + 16*kt + 4*g + i for this lane's row.
-    // All K fragments are fetched from LDS before the first MFMA so that the LDS round trips
-    // overlap instead of preceding each MFMA.
-    Pack8 kf[KS4][4];
-#pragma unroll
-    for (int ks = 0; ks < KS4; ++ks)
-#pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
-        kf[ks][kt] = *reinterpret_cast<const Pack8 *>(sK + (kt * 16 + l16) * LDQ + (g * KS4 + ks) * 8);
-    f32x4 s[4];
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < KS4; ++ks) {
-#pragma unroll
-      for (int kt = 0; kt < 4; ++kt) s[kt] = mfma16<T>(kf[ks][kt], qf[ks], s[kt]);
-    }
-    const int rowpos = m0 + rid + off;
-    float mloc = -INFINITY;
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int j = key0 + kt * 16 + 4 * g + i;
-        const bool vis = valid && j < Lk && (!causal || j <= rowpos);
-        const float x = vis ? s[kt][i] * scale_log2 : -INFINITY;
-        s[kt][i] = x;
-        mloc = fmaxf(mloc, x);
+      Pack8 xk = zero_pack8(), xv = zero_pack8();
+      if (key0 + key < Lk && e < D) {
+        xk = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
+        xv = ld_global16(vp + (int64_t)key * a.v_row_stride + e);
       }
-    mloc = max_rows4_f(mloc);
-    const float m_old = sM[rid], l_old = sL[rid];
-    const float m_new = fmaxf(m_old, mloc);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_old - m_use);
-    float rowsum = 0.f;
-    uint16_t *prow_p = sP + ((size_t)buf * 32 + slot) * LDP;
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-      float pr[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        pr[i] = __builtin_amdgcn_exp2f(s[kt][i] - m_use);
-        rowsum += pr[i];
-      }
-      *reinterpret_cast<uint2 *>(prow_p + kt * 16 + 4 * g) = make_uint2(pack2<T>(pr[0], pr[1]), pack2<T>(pr[2], pr[3]));
+      *reinterpret_cast<Pack8 *>(sK + key * LDQ + e) = xk;
+      *reinterpret_cast<Pack8 *>(sV + key * LDQ + e) = xv;
     }
-    rowsum = sum_rows4_f(rowsum);
-    if (g == 0) {
-      if (valid) {
-        sM[rid] = m_new;
-        sL[rid] = l_old * alpha + rowsum;
-      }
-      sAlpha[buf * 32 + slot] = alpha;
-      sRid[buf * 32 + slot] = valid ? rid : -1;
-    }
-  };
-
-  // ---- value stage: 64 output columns of a tile ------------------------------------------------
-  auto value_stage = [&](int buf) {
-    const int slot = lane & 31;
-    const int rid = sRid[buf * 32 + slot];
-    const float alpha = sAlpha[buf * 32 + slot];
-    Pack8 pf[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) pf[ks] = *reinterpret_cast<const Pack8 *>(sP + ((size_t)buf * 32 + slot) * LDP + 16 * ks + 8 * hh);
-#pragma unroll
-    for (int d2 = 0; d2 < NDT / 2; ++d2) {
-      const int dt = (wave - 2) * (NDT / 2) + d2;
-      Pack8 vf[4];
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) vf[ks] = tr_frag8(sV, LDQ, 16 * ks + 8 * hh, 16 * ks + 8 * hh + 4, dt * 32, lane);
-      f32x16 o;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[i] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) o = mfma32<T>(vf[ks], pf[ks], o);
-      if (rid >= 0) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          float *op = sO + rid * LDO + dt * 32 + 8 * g + 4 * hh;
-          f32x4 old = *reinterpret_cast<f32x4 *>(op);
-          f32x4 nw;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) nw[j] = old[j] * alpha + o[4 * g + j];
-          *reinterpret_cast<f32x4 *>(op) = nw;
-        }
-      }
-    }
-  };
-
-  for (int cb = 0; cb < ncols; cb += cols_per_batch) {
-    const int cend = min(ncols, cb + cols_per_batch);
-    __syncthreads();
-    // rows of this superblock inside each column's ascending list
-    for (int c = cb + tid; c < cend; c += 512) {
-      const int nnz = a.col_nnz[bh * a.max_cols + c];
-      int lo = 0, cnt = 0;
-      int64_t base = 0;
-      if (nnz > 0) {
-        base = coff[c];
-        const int32_t *list = a.row_indices + base;
-        lo = lower_bound_i32(list, nnz, m0);
-        const int hi = lo + lower_bound_i32(list + lo, nnz - lo, m0 + kSuperRows);
-        cnt = min(hi - lo, kSuperRows);
-      }
-      sLo[c - cb] = lo;
-      sCnt[c - cb] = cnt;
-      sOff[c - cb] = base + lo;
-    }
-    __syncthreads();
-    // ordered list of the (column, 64-key block) steps that have work
-    if (wave == 0) {
-      int nst = 0;
-      for (int base = 0; base < (cend - cb) * nsub; base += 64) {
-        const int idx = base + lane;
-        const int cl = idx / nsub, kb = idx - cl * nsub;
-        bool act = false;
-        if (cl < cend - cb) {
-          const int key0 = (cb + cl) * Bn + kb * 64;
-          act = sCnt[cl] > 0 && key0 < Lk && !(causal && key0 > last_rowpos);
-        }
-        const unsigned long long m = __ballot(act);
-        if (act) sStep[nst + __popcll(m & ((lane == 0) ? 0ull : (~0ull >> (64 - lane))))] = (cl << 8) | kb;
-        nst += __popcll(m);
-      }
-      if (lane == 0) sMisc[0] = nst;
-    }
-    __syncthreads();
-    const int nsteps = sMisc[0];
-    if (nsteps == 0) continue;
-    typedef std::integral_constant<int, 0> P0;
-    typedef std::integral_constant<int, 1> P1;
-    if (is_loader) {
-      load_k(P0{}, cb, 0);
-      load_v(P0{}, cb, 0);
-      if (nsteps > 1) {
-        load_k(P1{}, cb, 1);
-        load_v(P1{}, cb, 1);
-      }
-    }
-
-    // slot loop: the value stage lags the score stage by one tile
-    int slot_id = 0;
-    bool prev_valid = false, prev_first = false;
-    auto run_step = [&](auto par, int step) {
-      typedef std::integral_constant<int, 1 - decltype(par)::value> Other;
-      const int n = sCnt[sStep[step] >> 8];
-      const int key0 = step_key0(cb, step);
-      const int ntile = (n + 31) >> 5;
-      for (int tile = 0; tile < ntile; ++tile) {
-        __syncthreads();  // every read of the previous slot is done
-        // loader waves: LDS stores of this boundary; after the second barrier they issue the
-        // global loads for two steps ahead while the compute waves run their stages
-        const bool v_other = tile == 0 && prev_valid && prev_first;  // previous step had one tile: its V goes in now
-        if (is_loader) {
-          if (tile == 0) store_k(par, step, n);
-          if (v_other) store_v(Other{});
-          if (tile == 1) store_v(par);                                // V of this step, one slot after its K
-        }
-        __syncthreads();
-        if (is_loader) {
-          if (tile == 0 && step + 2 < nsteps) load_k(par, cb, step + 2);
-          if (v_other && step + 1 < nsteps) load_v(Other{}, cb, step + 1);
-          if (tile == 1 && step + 2 < nsteps) load_v(par, cb, step + 2);
-        } else if (wave < 2) {
-          score_stage(step, key0, n, tile, slot_id & 1);
-        } else if (prev_valid) {
-          value_stage((slot_id - 1) & 1);
-        }
-        prev_valid = true;
-        prev_first = tile == 0;
-        ++slot_id;
-      }
-    };
-    for (int step = 0; step < nsteps; step += 2) {
-      run_step(P0{}, step);
-      if (step + 1 < nsteps) run_step(P1{}, step + 1);
-    }
-    // drain: value stage of the last tile
-    __syncthreads();
-    if (is_loader && prev_valid && prev_first) {
-      if ((nsteps - 1) & 1)
-        store_v(P1{});
-      else
-        store_v(P0{});
-    }
-    __syncthreads();
-    if ((wave == 2 || wave == 3) && prev_valid) value_stage((slot_id - 1) & 1);
   }
   __syncthreads();
 
-  // ---- epilogue: normalise, write out and the log-sum-exp -----------------------------
-  {
-    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + (int64_t)(q0 + m0) * a.o_row_stride + (int64_t)h * a.o_head_stride;
-    for (int v = tid; v < rows_sb * VPR; v += 512) {
-      const int row = v / VPR, e = (v - row * VPR) * 8;
-      if (e >= D) continue;
-      const float l = sL[row];
-      const float inv = (l == 0.f || l != l) ? 1.f : 1.f / l;
-      const float *src = sO + row * LDO + e;
-      Pack8 o;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) o.w[w] = pack2<T>(src[2 * w] * inv, src[2 * w + 1] * inv);
-      *reinterpret_cast<Pack8 *>(op + (int64_t)row * a.o_row_stride + e) = o;
+  // ---- the block's column list --------------------------------------------------------------------
+  const int Bn = a.lg_block_n;
+  const int c = key0 / Bn;
+  const int64_t bh = (int64_t)b * a.heads + h;
+  int nnz = 0;
+  int64_t lbase = 0;
+  int start = 0;
+  if (c < a.max_cols) {
+    nnz = a.col_nnz[bh * a.max_cols + c];
+    lbase = a.col_offsets[bh * a.max_cols + c];
+    if (causal && nnz > 0) start = lower_bound_i32(a.row_indices + lbase, nnz, key0 - off);  // earlier rows see no key of the block
+  }
+  const int32_t *list = a.row_indices + lbase;
+  const uint16_t *qg = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)q0 * a.q_row_stride + (int64_t)h * a.q_head_stride;
+  int32_t *cntg = ws.cnt + (int64_t)q0 * a.heads + h;       // counter of local row r: cntg[r * heads]
+
+  auto fill_list = [&](int seg0, int seg_len) {
+    __syncthreads();
+    for (int i = tid; i < seg_len; i += NTHR) {
+      const int r = list[seg0 + i];
+      sList[i] = (r >= 0 && r < Lq) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
     }
-    if (tid < rows_sb) {
-      const float l = sL[tid], m = sM[tid];
-      const float lse = (l == 0.f || l != l) ? INFINITY : m * 0.6931471805599453f + logf(l);
-      a.softmax_lse[(int64_t)h * a.total_q + q0 + m0 + tid] = lse;
+    __syncthreads();
+  };
+  typedef std::integral_constant<int, 0> C0;
+  typedef std::integral_constant<int, 1> C1;
+
+  // The two roles run separate code with the same barrier sequence (register allocation, exact load counting).
+  if (is_loader) {
+    // two-deep rings of the gathered rows of two rounds; loads are unconditional (indices clamped, the
+    // surplus zeroed when stored) so that the compiler counts outstanding loads exactly
+    Pack8 lq[2][NV];
+    int lrow[2] = {-1, -1}, lslot[2] = {0, 0};
+    for (int seg0 = start; seg0 < nnz; seg0 += kFwdListCap) {
+      const int seg_len = min(kFwdListCap, nnz - seg0);
+      fill_list(seg0, seg_len);
+      const int nround = (seg_len + RR - 1) / RR;
+      auto load_round = [&](auto par, int r) {
+        constexpr int P = decltype(par)::value;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const int v = lt + 128 * i;
+          const int row = v / VPR, e = min((v - row * VPR) * 8, D - 8);
+          const int j = min(r * RR + row, seg_len - 1);
+          const int rid = max(sList[j], 0);
+          lq[P][i] = ld_global16(qg + (int64_t)rid * a.q_row_stride + e);
+        }
+        if (lt < RR) {
+          const int j = r * RR + lt;
+          const int rid = j < seg_len ? sList[j] : -1;
+          lrow[P] = rid;
+          // every visit of a (row, key block) pair takes one slot of the row (the only conditional memory
+          // operation of the loader: a shared dummy counter would serialise the whole grid on one address)
+          if (rid >= 0) lslot[P] = atomicAdd(cntg + (int64_t)rid * a.heads, 1);
+        }
+      };
+      auto store_round = [&](auto par, int r) {
+        constexpr int P = decltype(par)::value;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const int v = lt + 128 * i;
+          const int row = v / VPR, e = (v - row * VPR) * 8;
+          const int j = r * RR + row;
+          const bool ok = e < D && j < seg_len && sList[min(j, seg_len - 1)] >= 0;
+          Pack8 x = lq[P][i];
+#pragma unroll
+          for (int w = 0; w < 4; ++w) x.w[w] = ok ? x.w[w] : 0u;
+          *reinterpret_cast<Pack8 *>(sQ + (P * RR + row) * LDQ + e) = x;
+        }
+        if (lt < RR) {
+          sRow[P * RR + lt] = lrow[P];
+          sSlot[P * RR + lt] = lslot[P];
+        }
+      };
+      load_round(C0{}, 0);
+      load_round(C1{}, 1);  // past the end: rows clamp to the last one, nothing of it is used
+      store_round(C0{}, 0);
+      load_round(C0{}, 2);
+      auto loader_round = [&](auto par, int r) {  // par: parity of round r + 1
+        __syncthreads();  // round r is in LDS; the readers of round r-1 are done with the other buffer
+        if (r + 1 < nround) store_round(par, r + 1);
+        load_round(par, r + 3);
+      };
+      const int nround_pad = (nround + 1) & ~1;
+      for (int r = 0; r < nround_pad; r += 2) {
+        loader_round(C1{}, r);
+        loader_round(C0{}, r + 1);
+      }
+    }
+  } else {
+    // K of this block as the A operand of S^T = K Q^T: lane -> key (lane % 32) of each 32-key tile
+    Pack8 kfr[KT][KS];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        kfr[kt][ks] = *reinterpret_cast<const Pack8 *>(sK + (kt * 32 + (lane & 31)) * LDQ + (hh * KS + ks) * 8);
+    lds_cu16 *trV = tr_lane_base(sV, LDQ, lane) + 4 * hh * LDQ;
+    uint16_t *sOut = reinterpret_cast<uint16_t *>(smem + SM::oOut) + (size_t)wave * 32 * LDO;
+
+    for (int seg0 = start; seg0 < nnz; seg0 += kFwdListCap) {
+      const int seg_len = min(kFwdListCap, nnz - seg0);
+      fill_list(seg0, seg_len);
+      const int ntile = (seg_len + 31) >> 5;
+      const int nround = (seg_len + RR - 1) / RR;
+      const int nround_pad = (nround + 1) & ~1;
+
+      auto process_tile = [&](auto pc, int tile) {
+        constexpr int PB = decltype(pc)::value;
+        const int sidx = PB * RR + wave * 32 + (lane & 31);
+        const int rid = sRow[sidx];
+        // this lane's query row as the B operand
+        Pack8 qb[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qb[ks] = *reinterpret_cast<const Pack8 *>(sQ + (size_t)sidx * LDQ + (hh * KS + ks) * 8);
+        __builtin_amdgcn_sched_barrier(0);
+        f32x16 st[KT];  // S^T: register i of tile kt <-> key kt*32 + acc_row(i, hh), this lane's row
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) st[kt][i] = 0.f;
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) st[kt] = mfma32<T>(kfr[kt][ks], qb[ks], st[kt]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // V^T operands of the first half of the feature tiles: their LDS latency runs under the softmax arithmetic
+        Pack8 vt[NDT][KT][2];
+#pragma unroll
+        for (int dt = 0; dt < NDT / 2; ++dt)
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+              const int lo = (kt * 32 + 16 * s2) * LDQ + dt * 32;
+              vt[dt][kt][s2] = tr_frag8_at(trV, lo, lo + 8 * LDQ);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+        // block-local softmax of the row, log2 domain; keys beyond lim are masked
+        const int lim = rid < 0 ? -1 : min(causal ? rid + off : 0x7fffffff, Lk - 1) - key0;  // last visible key, relative
+        float m = -INFINITY;
+        if (__all(lim >= KB - 1)) {
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              st[kt][i] *= scale_log2;
+              m = fmaxf(m, st[kt][i]);
+            }
+        } else {
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int jrel = kt * 32 + 8 * (i >> 2) + (i & 3) + 4 * hh;
+              st[kt][i] = jrel <= lim ? st[kt][i] * scale_log2 : -INFINITY;
+              m = fmaxf(m, st[kt][i]);
+            }
+        }
+        m = max_xor32_f(m);
+        const float m_use = m == -INFINITY ? 0.f : m;
+        float l = 0.f;
+        Pack8 pf[KT][2];  // P^T as the B operand of O^T = V^T P^T, straight from the accumulators
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+              const float p0 = __builtin_amdgcn_exp2f(st[kt][8 * s2 + 2 * w] - m_use);
+              const float p1 = __builtin_amdgcn_exp2f(st[kt][8 * s2 + 2 * w + 1] - m_use);
+              l += p0 + p1;
+              pf[kt][s2].w[w] = pack2<T>(p0, p1);
+            }
+        l = sum_xor32_f(l);
+        __builtin_amdgcn_sched_barrier(0);
+        // O^T[d][row] = sum_key V^T[d][key] P^T[key][row]; register i of d-tile dt <-> d = dt*32 + acc_row(i, hh)
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+          if (dt == 0) {  // second half of the V^T operands, under the first products
+#pragma unroll
+            for (int d2 = NDT / 2; d2 < NDT; ++d2)
+#pragma unroll
+              for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2) {
+                  const int lo = (kt * 32 + 16 * s2) * LDQ + d2 * 32;
+                  vt[d2][kt][s2] = tr_frag8_at(trV, lo, lo + 8 * LDQ);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          f32x16 o;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[i] = 0.f;
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) o = mfma32<T>(vt[dt][kt][s2], pf[kt][s2], o);
+          // to the wave's row-major output tile, four features (8 bytes) at a time
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            *reinterpret_cast<uint2 *>(sOut + (lane & 31) * LDO + dt * 32 + 8 * g + 4 * hh) =
+                make_uint2(pack2<T>(o[4 * g], o[4 * g + 1]), pack2<T>(o[4 * g + 2], o[4 * g + 3]));
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        // header of the partial
+        const int slot = sSlot[sidx];
+        const bool keep = rid >= 0 && slot < ws.cap;
+        const int64_t pidx = ((int64_t)(q0 + max(rid, 0)) * a.heads + h) * ws.cap + slot;
+        if (keep && hh == 0) ws.hdr[pidx] = make_float4(m, l, __int_as_float(nb), 0.f);
+        wave_lds_fence();
+        // rows leave as 16-byte pieces: lane -> (row 4k + lane / 16, features 8 * (lane % 16))
+        if ((lane & 15) * 8 < D) {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const int row = 4 * k + (lane >> 4);
+            const int r2 = sRow[PB * RR + wave * 32 + row], s2 = sSlot[PB * RR + wave * 32 + row];
+            if (r2 >= 0 && s2 < ws.cap) {
+              const Pack8 x = *reinterpret_cast<const Pack8 *>(sOut + row * LDO + (lane & 15) * 8);
+              *reinterpret_cast<Pack8 *>(ws.part + (((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2) * D + (lane & 15) * 8) = x;
+            }
+          }
+        }
+        wave_lds_fence();
+        (void)tile;
+      };
+
+      for (int r = 0; r < nround_pad; r += 2) {
+        __syncthreads();  // round r is in LDS
+        if (NCW * r + wave < ntile) process_tile(C0{}, NCW * r + wave);
+        __syncthreads();
+        if (NCW * (r + 1) + wave < ntile) process_tile(C1{}, NCW * (r + 1) + wave);
+      }
     }
   }
+}
+
+// one wave per (row, head); block 256 = 4 rows
+template <typename T>
+__global__ __launch_bounds__(256) void attn_fwd_combine_kernel(fmoba_attn_fwd_args a, FwdWs ws) {
+  __shared__ int sOrd[4][64];
+  __shared__ float sWgt[4][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t rh = (int64_t)blockIdx.x * 4 + wv;  // (global row) * heads + head
+  if (rh >= (int64_t)a.total_q * a.heads) return;
+  const int64_t row = rh / a.heads;
+  const int h = (int)(rh - row * a.heads);
+  const int D = a.head_dim;
+  const int n = min(ws.cnt[rh], ws.cap);
+  uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + row * a.o_row_stride + (int64_t)h * a.o_head_stride;
+  float *lsep = a.softmax_lse + (int64_t)h * a.total_q + row;
+  float acc0 = 0.f, acc1 = 0.f, L = 0.f, M = -INFINITY;
+  const float4 *hdr = ws.hdr + rh * ws.cap;
+  const uint16_t *part = ws.part + rh * ws.cap * D;
+  const bool mine = 2 * lane < D;
+  // partials are merged in ascending key-block order (the slot a visit got is arbitrary), 64 at a time
+  for (int base = 0; base < n; base += 64) {
+    const int cntb = min(64, n - base);
+    float mj = -INFINITY, lj = 0.f;
+    int cj = 0x7fffffff;
+    if (lane < cntb) {
+      const float4 x = hdr[base + lane];
+      mj = x.x;
+      lj = x.y;
+      cj = __float_as_int(x.z);
+    }
+    // rank of this lane's partial in the batch; equal ids (malformed pattern) are ordered by slot
+    int rank = 0;
+    for (int i = 0; i < cntb; ++i) {
+      const int ci = __shfl(cj, i, 64);
+      rank += (ci < cj || (ci == cj && i < lane)) ? 1 : 0;
+    }
+    float mb = mj;
+    for (int o = 32; o >= 1; o >>= 1) mb = fmaxf(mb, __shfl_xor(mb, o, 64));
+    const float Mn = fmaxf(M, mb);
+    const float Mu = Mn == -INFINITY ? 0.f : Mn;
+    const float resc = __builtin_amdgcn_exp2f(M - Mu);  // M = -inf: nothing accumulated yet, factor 0 on zeros
+    acc0 *= resc;
+    acc1 *= resc;
+    L *= resc;
+    M = Mn;
+    const float wj = (lane < cntb) ? __builtin_amdgcn_exp2f(mj - Mu) : 0.f;
+    // sum of the weighted l in rank order: every lane adds the same sequence, so L is the same everywhere
+    wave_lds_fence();
+    if (lane < cntb) {
+      sOrd[wv][rank] = lane;
+      sWgt[wv][rank] = wj;
+    }
+    float wl = wj * lj;
+    wave_lds_fence();
+    for (int t = 0; t < cntb; ++t) L += __shfl(wl, sOrd[wv][t], 64);
+    // the rows themselves: independent loads, four in flight
+    if (mine) {
+      int t = 0;
+      for (; t + 4 <= cntb; t += 4) {
+        uint32_t x[4];
+        float w[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          x[u] = *reinterpret_cast<const uint32_t *>(part + (int64_t)(base + sOrd[wv][t + u]) * D + 2 * lane);
+          w[u] = sWgt[wv][t + u];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          acc0 = fmaf(w[u], elem_to_float<T>((uint16_t)(x[u] & 0xffffu)), acc0);
+          acc1 = fmaf(w[u], elem_to_float<T>((uint16_t)(x[u] >> 16)), acc1);
+        }
+      }
+      for (; t < cntb; ++t) {
+        const uint32_t x = *reinterpret_cast<const uint32_t *>(part + (int64_t)(base + sOrd[wv][t]) * D + 2 * lane);
+        const float w = sWgt[wv][t];
+        acc0 = fmaf(w, elem_to_float<T>((uint16_t)(x & 0xffffu)), acc0);
+        acc1 = fmaf(w, elem_to_float<T>((uint16_t)(x >> 16)), acc1);
+      }
+    }
+  }
+  const bool empty = !(L > 0.f);
+  const float inv = empty ? 0.f : 1.f / L;
+  if (mine) *reinterpret_cast<uint32_t *>(op + 2 * lane) = pack2<T>(acc0 * inv, acc1 * inv);
+  if (lane == 0) *lsep = empty ? INFINITY : (M + __builtin_amdgcn_logf(L)) * 0.6931471805599453f;
 }
 
 __global__ void fwd_empty_kernel(void *out, float *lse, int64_t n_out_words, int64_t n_lse) {
@@ -437,29 +445,78 @@ __global__ void fwd_empty_kernel(void *out, float *lse, int64_t n_out_words, int
   for (int64_t i = i0; i < n_lse; i += st) lse[i] = INFINITY;
 }
 
-template <typename T, int HD>
-static int launch_fwd(const fmoba_attn_fwd_args &a, hipStream_t s) {
-  auto kern = attn_fwd_kernel<T, HD>;
-  const size_t smem = FwdSmem<HD>::bytes;
+__global__ void fwd_zero_i32_kernel(int32_t *p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
+// visits per (row, head) of a pattern: grid over list entries is not possible without the segment of each
+// entry, so one workgroup walks one column list
+__global__ __launch_bounds__(256) void csc_row_visits_kernel(fmoba_attn_fwd_args a, int32_t *cnt, int kb) {
+  const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int q0 = a.cu_seqlens_q[b], Lq = a.cu_seqlens_q[b + 1] - q0;
+  const int Lk = a.cu_seqlens_k[b + 1] - a.cu_seqlens_k[b];
+  const int64_t bh = (int64_t)b * a.heads + h;
+  const int nnz = a.col_nnz[bh * a.max_cols + c];
+  const int32_t *list = a.row_indices + a.col_offsets[bh * a.max_cols + c];
+  // key blocks of this column that exist in the sequence
+  const int key_lo = c * a.lg_block_n, key_hi = min(Lk, key_lo + a.lg_block_n);
+  const int nblk = key_hi > key_lo ? (key_hi - key_lo + kb - 1) / kb : 0;
+  if (nblk == 0) return;
+  for (int i = threadIdx.x; i < nnz; i += 256) {
+    const int r = list[i];
+    if (r >= 0 && r < Lq) atomicAdd(&cnt[(int64_t)(q0 + r) * a.heads + h], nblk);
+  }
+}
+__global__ __launch_bounds__(256) void max_i32_kernel(const int32_t *p, int64_t n, int32_t *out) {
+  int m = 0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) m = max(m, p[i]);
+  for (int o = 32; o >= 1; o >>= 1) m = max(m, __shfl_xor(m, o, 64));
+  if ((threadIdx.x & 63) == 0 && m > 0) atomicMax(out, m);
+}
+
+static inline size_t fwd_align256(size_t x) { return (x + 255) & ~(size_t)255; }
+static inline int fwd_key_block(int lg_block_n) { return lg_block_n % 128 == 0 ? 128 : 64; }
+
+template <typename T, int HD, int KB>
+static int launch_fwd_col(const fmoba_attn_fwd_args &a, const FwdWs &ws, hipStream_t s) {
+  // 64-key blocks leave room (registers, LDS) for four compute waves; 128-key blocks for two
+  constexpr int NCW = KB == 64 ? 4 : 2;
+  auto kern = attn_fwd_col_kernel<T, HD, KB, NCW>;
+  const size_t smem = FwdColSmem<HD, KB, NCW>::bytes;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("attn_fwd: cannot reserve %zu bytes of LDS", smem);
     return 2;
   }
-  const int nsb_max = ceil_div(a.max_seqlen_q, kSuperRows);
-  const int64_t pairs_per_xcd = ((int64_t)a.heads * a.batch + 7) / 8;
-  const int64_t items = 8 * pairs_per_xcd * nsb_max;
-  if (items >= ((int64_t)1 << 31)) {
-    set_error("attn_fwd: too many (sequence, head, superblock) work items");
-    return 1;
-  }
-  dim3 grid((unsigned)items);
-  hipLaunchKernelGGL(kern, grid, dim3(512), smem, s, a, nsb_max);
+  dim3 grid(ceil_div(a.max_seqlen_k, KB), a.heads, a.batch);
+  hipLaunchKernelGGL(kern, grid, dim3((NCW + 2) * 64), smem, s, a, ws);
+  return 0;
+}
+template <typename T>
+static int run_fwd(const fmoba_attn_fwd_args &a, const FwdWs &ws, hipStream_t s) {
+  const int kb = fwd_key_block(a.lg_block_n);
+  int rc;
+  if (a.head_dim <= 64)
+    rc = kb == 128 ? launch_fwd_col<T, 64, 128>(a, ws, s) : launch_fwd_col<T, 64, 64>(a, ws, s);
+  else
+    rc = kb == 128 ? launch_fwd_col<T, 128, 128>(a, ws, s) : launch_fwd_col<T, 128, 64>(a, ws, s);
+  if (rc) return rc;
+  const int64_t rows = (int64_t)a.total_q * a.heads;
+  hipLaunchKernelGGL(attn_fwd_combine_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, a, ws);
   return 0;
 }
 
 }  // namespace fmoba
 
-extern "C" int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream) {
+extern "C" int32_t fmoba_attn_fwd_key_block(int32_t lg_block_n) { return fmoba::fwd_key_block(lg_block_n); }
+
+extern "C" size_t fmoba_attn_fwd_workspace_bytes(int32_t total_q, int32_t heads, int32_t head_dim, int32_t max_visits_per_row) {
+  using namespace fmoba;
+  if (total_q <= 0 || heads <= 0 || head_dim <= 0 || max_visits_per_row <= 0) return 256;
+  const size_t rows = (size_t)total_q * heads;
+  return fwd_align256((rows + 1) * 4) + fwd_align256(rows * max_visits_per_row * 16) + fwd_align256(rows * max_visits_per_row * head_dim * 2) + 256;
+}
+
+static int fwd_check_common(const fmoba_attn_fwd_args *a) {
   using namespace fmoba;
   FMOBA_REQUIRE(a != nullptr, "attn_fwd: null args");
   FMOBA_REQUIRE(a->dtype == FMOBA_DTYPE_F16 || a->dtype == FMOBA_DTYPE_BF16, "FlashMoBA only support fp16 and bf16 data type");
@@ -471,10 +528,32 @@ extern "C" int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream) {
   FMOBA_REQUIRE(a->lg_block_m >= 128 && a->lg_block_m <= 1024, "m_lg_block_dim must be at least 128 and at most 1024");
   FMOBA_REQUIRE(a->lg_block_m % 64 == 0, "m_lg_block_dim must be a multiple of 64");
   FMOBA_REQUIRE(a->lg_block_n > 0 && a->lg_block_n % 64 == 0, "n_lg_block_dim must be a multiple of 64");
-  FMOBA_REQUIRE(a->lg_block_n <= 64 * 256, "attn_fwd: n_lg_block_dim above 16384 is not supported");
   FMOBA_REQUIRE(a->total_q >= 0 && a->total_k >= 0 && a->max_seqlen_q >= 0 && a->max_seqlen_k >= 0 && a->max_cols >= 0, "negative size");
   FMOBA_REQUIRE(a->cu_seqlens_q && a->cu_seqlens_k, "attn_fwd: null cu_seqlens pointer");
   FMOBA_REQUIRE(a->batch <= 65535 && a->heads <= 65535, "attn_fwd: batch/heads too large for the launch grid");
+  return 0;
+}
+
+extern "C" int fmoba_csc_max_row_visits(const fmoba_attn_fwd_args *a, int32_t *counts, int32_t *max_out, void *stream) {
+  using namespace fmoba;
+  if (int rc = fwd_check_common(a)) return rc;
+  FMOBA_REQUIRE(counts && max_out, "csc_max_row_visits: null output pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t rows = (int64_t)a->total_q * a->heads;
+  hipLaunchKernelGGL(fwd_zero_i32_kernel, dim3(256), dim3(256), 0, s, counts, rows);
+  hipLaunchKernelGGL(fwd_zero_i32_kernel, dim3(1), dim3(64), 0, s, max_out, (int64_t)1);
+  if (rows > 0 && a->max_cols > 0 && a->total_k > 0) {
+    FMOBA_REQUIRE(a->col_offsets && a->col_nnz && a->row_indices, "csc_max_row_visits: null CSC pointer");
+    hipLaunchKernelGGL(csc_row_visits_kernel, dim3(a->max_cols, a->heads, a->batch), dim3(256), 0, s, *a, counts, fwd_key_block(a->lg_block_n));
+    hipLaunchKernelGGL(max_i32_kernel, dim3(256), dim3(256), 0, s, counts, rows, max_out);
+  }
+  FMOBA_LAUNCH_CHECK("csc_max_row_visits");
+  return 0;
+}
+
+extern "C" int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream) {
+  using namespace fmoba;
+  if (int rc = fwd_check_common(a)) return rc;
   hipStream_t s = (hipStream_t)stream;
   if (a->total_q == 0 || a->max_seqlen_q == 0) return 0;
   FMOBA_REQUIRE(a->q && a->out && a->softmax_lse, "attn_fwd: null q/out/lse pointer");
@@ -493,12 +572,21 @@ extern "C" int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream) {
   for (int64_t x : st) FMOBA_REQUIRE(x % 8 == 0, "attn_fwd: strides must be multiples of 8 elements");
   FMOBA_REQUIRE(((uintptr_t)a->q % 16) == 0 && ((uintptr_t)a->k % 16) == 0 && ((uintptr_t)a->v % 16) == 0 && ((uintptr_t)a->out % 16) == 0,
                 "attn_fwd: q, k, v and out must be 16-byte aligned");
-  int rc;
-  if (a->dtype == FMOBA_DTYPE_BF16)
-    rc = a->head_dim <= 64 ? launch_fwd<bf16_t, 64>(*a, s) : launch_fwd<bf16_t, 128>(*a, s);
-  else
-    rc = a->head_dim <= 64 ? launch_fwd<f16_t, 64>(*a, s) : launch_fwd<f16_t, 128>(*a, s);
+  FMOBA_REQUIRE(a->max_visits_per_row > 0, "attn_fwd: max_visits_per_row must be positive");
+  const size_t need = fmoba_attn_fwd_workspace_bytes(a->total_q, a->heads, a->head_dim, a->max_visits_per_row);
+  FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, "attn_fwd: workspace too small (%zu < %zu)", a->workspace_bytes, need);
+  const size_t rows = (size_t)a->total_q * a->heads;
+  uintptr_t p = ((uintptr_t)a->workspace + 255) & ~(uintptr_t)255;
+  FwdWs ws;
+  ws.cap = a->max_visits_per_row;
+  ws.cnt = reinterpret_cast<int32_t *>(p);
+  p += fwd_align256((rows + 1) * 4);
+  ws.hdr = reinterpret_cast<float4 *>(p);
+  p += fwd_align256(rows * ws.cap * 16);
+  ws.part = reinterpret_cast<uint16_t *>(p);
+  hipLaunchKernelGGL(fwd_zero_i32_kernel, dim3(512), dim3(256), 0, s, ws.cnt, (int64_t)rows + 1);
+  int rc = a->dtype == FMOBA_DTYPE_BF16 ? run_fwd<bf16_t>(*a, ws, s) : run_fwd<f16_t>(*a, ws, s);
   if (rc) return rc;
-  FMOBA_LAUNCH_CHECK("attn_fwd_kernel");
+  FMOBA_LAUNCH_CHECK("attn_fwd");
   return 0;
 }

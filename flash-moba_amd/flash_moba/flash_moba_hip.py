@@ -20,6 +20,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
+import threading
 import os
 from typing import List, Optional
 
@@ -52,10 +53,11 @@ class AttnFwdArgs(ctypes.Structure):
     _fields_ = [("q", c_vp), ("k", c_vp), ("v", c_vp), ("out", c_vp), ("softmax_lse", c_vp),
                 ("col_offsets", c_vp), ("col_nnz", c_vp), ("row_indices", c_vp),
                 ("cu_seqlens_q", c_vp), ("cu_seqlens_k", c_vp),
+                ("workspace", c_vp), ("workspace_bytes", c_sz),
                 ("batch", c_i32), ("total_q", c_i32), ("total_k", c_i32), ("heads", c_i32), ("heads_k", c_i32),
                 ("head_dim", c_i32), ("max_seqlen_q", c_i32), ("max_seqlen_k", c_i32), ("max_cols", c_i32),
                 ("lg_block_m", c_i32), ("lg_block_n", c_i32), ("is_causal", c_i32), ("dtype", c_i32),
-                ("softmax_scale", c_f32),
+                ("max_visits_per_row", c_i32), ("softmax_scale", c_f32),
                 ("q_row_stride", c_i64), ("q_head_stride", c_i64), ("k_row_stride", c_i64), ("k_head_stride", c_i64),
                 ("v_row_stride", c_i64), ("v_head_stride", c_i64), ("o_row_stride", c_i64), ("o_head_stride", c_i64)]
 
@@ -86,6 +88,9 @@ EXPORTS = {
     "fmoba_fused_topk": (c_i32, [ctypes.POINTER(FusedTopkArgs), c_vp]),
     "fmoba_varlen_sort_workspace_bytes": (c_sz, [c_i64]),
     "fmoba_varlen_sort": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_sz, c_vp]),
+    "fmoba_attn_fwd_key_block": (c_i32, [c_i32]),
+    "fmoba_attn_fwd_workspace_bytes": (c_sz, [c_i32, c_i32, c_i32, c_i32]),
+    "fmoba_csc_max_row_visits": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp, c_vp, c_vp]),
     "fmoba_attn_fwd": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp]),
     "fmoba_attn_bwd_workspace_bytes": (c_sz, [c_i64, c_i32]),
     "fmoba_attn_bwd": (c_i32, [ctypes.POINTER(AttnBwdArgs), c_vp]),
@@ -279,6 +284,20 @@ def _reject_unsupported(p_dropout, softcap, alibi_slopes, seqused_k=None, leftpa
     _require(not return_softmax, "return_softmax is only supported when p_dropout > 0.0, which FlashMoBA does not support")
 
 
+# A caller that knows how many (row, key block) visits a query row can have (the gated path: top-k times the
+# key blocks per chunk) leaves the bound here for the next forward call; otherwise it is computed from the
+# pattern, which costs one device-to-host read.
+_hint = threading.local()
+
+
+def set_visits_hint(n):
+    _hint.value = None if n is None else int(n)
+
+
+def fwd_key_block(n_lg_block_dim):
+    return int(load_library().fmoba_attn_fwd_key_block(int(n_lg_block_dim)))
+
+
 def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k,
                     seqused_k, leftpad_k, alibi_slopes, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                     zero_tensors, is_causal, softcap, return_softmax, m_lg_block_dim, n_lg_block_dim, gen=None):
@@ -321,14 +340,31 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
         lse = torch.empty((heads, total_q), dtype=torch.float32, device=q.device)
         p = torch.empty((0,), dtype=dtype, device=q.device)
         rng_state = torch.zeros((2,), dtype=torch.int64, device=q.device)
-        a = AttnFwdArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
-                        moba_col_offsets.data_ptr(), moba_col_nnz.data_ptr(), moba_row_indices.data_ptr(),
-                        cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(),
-                        batch, total_q, total_k, heads, heads_k, d, int(max_seqlen_q), int(max_seqlen_k), max_cols,
-                        int(m_lg_block_dim), int(n_lg_block_dim), int(bool(is_causal)), _dt(q), float(softmax_scale),
-                        q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
-                        out.stride(0), out.stride(1))
-        _check(load_library().fmoba_attn_fwd(ctypes.byref(a), _stream()))
+        lib = load_library()
+        hint = getattr(_hint, "value", None)
+        _hint.value = None
+
+        def args(ws_ptr, ws_bytes, visits):
+            return AttnFwdArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                               moba_col_offsets.data_ptr(), moba_col_nnz.data_ptr(), moba_row_indices.data_ptr(),
+                               cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ws_ptr, ws_bytes,
+                               batch, total_q, total_k, heads, heads_k, d, int(max_seqlen_q), int(max_seqlen_k), max_cols,
+                               int(m_lg_block_dim), int(n_lg_block_dim), int(bool(is_causal)), _dt(q), visits,
+                               float(softmax_scale),
+                               q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+                               out.stride(0), out.stride(1))
+
+        visits = hint
+        if visits is None and total_q > 0 and total_k > 0 and max_cols > 0:
+            counts = torch.empty((total_q * heads + 1,), dtype=torch.int32, device=q.device)
+            a0 = args(None, 0, 0)
+            _check(lib.fmoba_csc_max_row_visits(ctypes.byref(a0), counts.data_ptr(), counts[total_q * heads:].data_ptr(), _stream()))
+            visits = int(counts[total_q * heads].item())
+        visits = max(1, int(visits or 1))
+        ws_bytes = lib.fmoba_attn_fwd_workspace_bytes(total_q, heads, d, visits)
+        ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=q.device)
+        a = args(ws.data_ptr(), ws_bytes, visits)
+        _check(lib.fmoba_attn_fwd(ctypes.byref(a), _stream()))
     return [out, lse, p, rng_state]
 
 

@@ -306,6 +306,9 @@ def flash_moba_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
         q, k, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
         moba_topk, moba_chunk_size, causal=causal)
     lg_block_m = decide_lg_block_m(moba_topk, moba_chunk_size, max_seqlen_k, causal)
+    if moba_chunk_size % 64 == 0:
+        # a gated row visits at most top-k chunks: the forward needs no pass over the pattern to size its scratch
+        flash_moba_gpu.set_visits_hint(moba_topk * (moba_chunk_size // flash_moba_gpu.fwd_key_block(moba_chunk_size)))
     return flash_moba_attn_varlen_func(
         q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
         col_offsets, col_nnz, indices, lg_block_m, moba_chunk_size, dropout_p=0.0, causal=causal)

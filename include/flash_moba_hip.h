@@ -107,7 +107,14 @@ int fmoba_varlen_sort(const int64_t *seg_starts, const int64_t *seg_ends, int64_
  * Sparse attention forward over a CSC pattern.
  * Replaces moba_varlen_fwd (csrc/flash_moba/flash_moba_api.cpp:375-596).
  *   out (total_q, heads, head_dim) dtype, softmax_lse (heads, total_q) fp32.
- * Rows that see no key get out = 0, lse = +inf.  No scratch memory is needed.
+ * Rows that see no key get out = 0, lse = +inf.
+ * The forward is column-stationary: every visit of a (query row, key block) pair leaves a
+ * partial result in `workspace`, and a second launch merges the partials of each row.  A key
+ * block is fmoba_attn_fwd_key_block(lg_block_n) keys (128 if lg_block_n is a multiple of 128,
+ * else 64).  max_visits_per_row bounds the number of visits of any (row, head): for a pattern
+ * from the gating, topk * lg_block_n / key_block; for an arbitrary pattern,
+ * fmoba_csc_max_row_visits() computes it.  Visits beyond the bound are dropped.
+ * workspace: fmoba_attn_fwd_workspace_bytes() bytes, contents undefined on entry and return.
  * ---------------------------------------------------------------------------------- */
 typedef struct {
   const void *q, *k, *v;
@@ -117,14 +124,23 @@ typedef struct {
   const int32_t *col_nnz;       /* (batch, heads, max_cols) */
   const int32_t *row_indices;   /* flat row lists */
   const int32_t *cu_seqlens_q, *cu_seqlens_k;
+  void *workspace;
+  size_t workspace_bytes;
   int32_t batch, total_q, total_k, heads, heads_k, head_dim;
   int32_t max_seqlen_q, max_seqlen_k, max_cols;
   int32_t lg_block_m, lg_block_n;
   int32_t is_causal, dtype;
+  int32_t max_visits_per_row;
   float softmax_scale;
   int64_t q_row_stride, q_head_stride, k_row_stride, k_head_stride;
   int64_t v_row_stride, v_head_stride, o_row_stride, o_head_stride;
 } fmoba_attn_fwd_args;
+int32_t fmoba_attn_fwd_key_block(int32_t lg_block_n);
+size_t fmoba_attn_fwd_workspace_bytes(int32_t total_q, int32_t heads, int32_t head_dim, int32_t max_visits_per_row);
+/* counts (total_q * heads) int32 and max_out (1) int32 are device outputs: visits per (row, head) and
+ * their maximum for the pattern in `a` (q/k/v/out/workspace of `a` are not read).  No counterpart in the
+ * reference, whose row-wise scratch needs no bound. */
+int fmoba_csc_max_row_visits(const fmoba_attn_fwd_args *a, int32_t *counts, int32_t *max_out, void *stream);
 int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream);
 
 /* ------------------------------------------------------------------------------------
