@@ -236,15 +236,19 @@ def main():
             for name, mask in (("prep", 1), ("dkdv", 2), ("dq", 4)):
                 phase_ms[name] = time_events(lambda: run(mask), it)
 
-        hip.moba_varlen_bwd(dout, qd, kd, vd, out, lse, dq, dk, dv, co, cn, ind, cu, cu, None, max_len, max_len, 0.0, scale,
-                            False, True, 0.0, False, lg_m, chunk, None, None, _phases=run_phases)
-        t_bwd = time_events(lambda: hip.moba_varlen_bwd(dout, qd, kd, vd, out, lse, dq, dk, dv, co, cn, ind, cu, cu, None, max_len,
-                                                        max_len, 0.0, scale, False, True, 0.0, False, lg_m, chunk, None, None), it)
+        bwd_visits = visits * (hip.fwd_key_block(chunk) // 64)
+
+        def bwd(**kw):
+            hip.set_bwd_visits_hint(bwd_visits)
+            return hip.moba_varlen_bwd(dout, qd, kd, vd, out, lse, dq, dk, dv, co, cn, ind, cu, cu, None, max_len, max_len, 0.0,
+                                       scale, False, True, 0.0, False, lg_m, chunk, None, None, **kw)
+
+        bwd(_phases=run_phases)
+        t_bwd = time_events(bwd, it)
         stages["attn_bwd"] = {"ms": t_bwd, "TFLOPs": bwd_flops / t_bwd / 1e9, "frac_mfma": bwd_flops / t_bwd / 1e9 / PEAK_BF16_TFLOPS,
                               "phases_ms": phase_ms}
-        # the dK/dV kernel runs four of the five backward GEMMs (S, dP, dV, dK), the dQ kernel the fifth
-        kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 8.0 * D * pairs, "mfma")
-        kernels["attn_bwd_dq_kernel"] = (phase_ms["dq"], 2.0 * D * pairs, "mfma")
+        # the dK/dV kernel runs all five backward GEMMs (S, dP, dV, dK, dQ partials); the dQ phase only adds partial rows
+        kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 10.0 * D * pairs, "mfma")
     # sort alone, on the CSC the gating produced (already sorted input; same traffic)
     t_sort = time_events(lambda: torch.ops.flash_moba._varlen_sort(co, cn, ind), it)
     sort_bytes = 2 * int(cn.sum().item()) * 4 + 2 * cn.numel() * 8

@@ -2,24 +2,23 @@
 //
 //   bwd_prep_kernel      : delta[row] = sum_d dO*O (fp32).
 //   attn_bwd_dkdv_kernel : COLUMN-stationary.  One workgroup per (64-key block, head,
-//                          sequence) keeps K and V of the block in LDS and in operand
-//                          registers and walks the block's ascending row list in gathered
-//                          32-row tiles:
-//                            S = Q K^T, dP = dO V^T             (A = gathered rows, B = K / V halves in registers)
+//                          sequence) keeps K and V of the block in LDS and walks the block's
+//                          ascending row list in gathered 32-row tiles:
+//                            S = Q K^T, dP = dO V^T             (A = gathered rows, B = K / V halves)
 //                            P = exp2(S*scale*log2e - LSE*log2e), dS = P o (dP - delta)
 //                            dV^T += dO^T P, dK^T += Q^T dS     (P, dS feed the MFMA from registers;
 //                                                                dO^T, Q^T via transposing LDS reads)
+//                            dQ^T_partial = K^T dS^T            (per visit of a (row, key block) pair)
 //                          dK/dV live in accumulator registers for the whole list and are written
-//                          once.  The dS tiles (bf16) are streamed to a workspace indexed by the
-//                          row-list position, i.e. written linearly per column.
-//   attn_bwd_dq_kernel   : ROW-stationary.  One workgroup owns 128 consecutive query rows and
-//                          their fp32 dQ accumulators in LDS; for every column it reads the
-//                          contiguous slice of dS rows its superblock owns and adds dS K:
-//                          dQ = scale * sum_columns dS K, one GEMM, no recomputation.
-// In both kernels half of the waves compute and the other half only move data (global ->
-// registers -> LDS) one to two steps ahead of the compute waves.  The dK/dV kernel runs four
-// waves of 512 registers: a compute wave keeps 32 keys x head_dim of dK^T and dV^T plus its K and
-// V operands in registers, which does not fit in the 256 registers an eight-wave workgroup gets.
+//                          once.  Every visit leaves a dQ partial row (16-bit, unscaled) in a slot
+//                          that the row hands out from a counter.
+//   attn_bwd_dq_combine_kernel : one wave per (row, head) adds the row's partials in ascending
+//                          key-block order and scales: dQ.  Work and traffic are proportional to
+//                          the number of visits, whatever the number of chunks per sequence.
+// In the dK/dV kernel half of the waves compute and the other half only move data (global ->
+// registers -> LDS) two rounds ahead of the compute waves.  It runs four waves of 512 registers: a
+// compute wave keeps 32 keys x head_dim of dK^T and dV^T in registers, which does not fit in the 256
+// registers an eight-wave workgroup gets.
 #include "fmoba_common.h"
 
 #include <type_traits>
@@ -40,8 +39,11 @@ struct BwdSmem {
   static constexpr size_t oV = oK + (size_t)64 * LDQ * 2;
   static constexpr size_t oQ = oV + (size_t)64 * LDQ * 2;          // [2 buffers][2 tile slots][32][LDQ]
   static constexpr size_t odO = oQ + (size_t)4 * 32 * LDQ * 2;
-  static constexpr size_t odS = odO + (size_t)4 * 32 * LDQ * 2;    // [2 waves][32][LDS_]
-  static constexpr size_t oRow = odS + (size_t)2 * 32 * LDS_ * 2;  // int[2 buffers][64]
+  static constexpr size_t odS = odO + (size_t)4 * 32 * LDQ * 2;    // [2 tile slots][64 keys][LDS_]: dS^T of both key halves
+  static constexpr int LDH = HD / 2 + 8;                           // elements, per-wave dQ half-row tile [32 rows][LDH]
+  static constexpr size_t odQ = odS + (size_t)2 * 64 * LDS_ * 2;   // [2 waves][32][LDH]
+  static constexpr size_t oSlot = odQ + (size_t)2 * 32 * LDH * 2;  // int[2 buffers][64]
+  static constexpr size_t oRow = oSlot + 4 * 32 * 4;               // int[2 buffers][64]
   static constexpr size_t oLse = oRow + 4 * 32 * 4;                // LSE * log2(e)
   static constexpr size_t oDelta = oLse + 4 * 32 * 4;
   static constexpr size_t oList = oDelta + 4 * 32 * 4;             // int[kListCap]
@@ -73,10 +75,20 @@ __device__ __forceinline__ int lower_bound_i32b(const int32_t *p, int n, int v) 
   return lo;
 }
 
-template <typename T, int HD>
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args a, uint16_t *ds_ws) {
+struct BwdWs {
+  int32_t *cnt;    // [total_q * heads] visits handed out per (row, head)
+  int32_t *pid;    // [total_q * heads * cap] key block id of each partial
+  uint16_t *part;  // [total_q * heads * cap][head_dim] dQ partials (unscaled)
+  int32_t cap;
+  uint16_t *ds;    // [row list entry][lg_block_n] dS tiles (row-stationary dQ form)
+};
+
+// DQP = true: dQ partials per visit (for the combine kernel); false: dS^T tiles to ws.ds (for the row-stationary dQ kernel)
+template <typename T, int HD, bool DQP>
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args a, BwdWs ws) {
   typedef BwdSmem<HD> SM;
-  constexpr int KS = HD / 16, LDQ = SM::LDQ, LDS_ = SM::LDS_, NDT = HD / 32, VPR = HD / 8, LDR = SM::LDR;
+  constexpr int KS = HD / 16, LDQ = SM::LDQ, LDS_ = SM::LDS_, NDT = HD / 32, VPR = HD / 8, LDR = SM::LDR, LDH = SM::LDH;
+  constexpr int NDH = NDT / 2;  // feature tiles of dQ per compute wave
   constexpr int NV = 2 * 32 * VPR / 128;  // 16-byte vectors of the two gathered Q (or dO) tiles of a round per loader thread
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint16_t *sK = reinterpret_cast<uint16_t *>(smem + SM::oK);
@@ -84,6 +96,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   uint16_t *sQ = reinterpret_cast<uint16_t *>(smem + SM::oQ);
   uint16_t *sdO = reinterpret_cast<uint16_t *>(smem + SM::odO);
   int *sRow = reinterpret_cast<int *>(smem + SM::oRow);
+  int *sSlot = reinterpret_cast<int *>(smem + SM::oSlot);
   float *sLse = reinterpret_cast<float *>(smem + SM::oLse);
   float *sDelta = reinterpret_cast<float *>(smem + SM::oDelta);
   int *sList = reinterpret_cast<int *>(smem + SM::oList);
@@ -103,7 +116,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   const bool causal = a.is_causal != 0;
   const float scale_log2 = a.softmax_scale * 1.4426950408889634f;
   constexpr float kLog2e = 1.4426950408889634f;
-  uint16_t *sdS = reinterpret_cast<uint16_t *>(smem + SM::odS) + (size_t)(wave & 1) * 32 * LDS_;
+  uint16_t *sdS = reinterpret_cast<uint16_t *>(smem + SM::odS);  // + tile slot * 64 * LDS_ + key * LDS_ + row
 
   // ---- the key block stays in LDS ---------------------------------------------------------
   {
@@ -125,7 +138,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   // ---- this block's column list --------------------------------------------------------------
   const int Bn = a.lg_block_n;
   const int c = key0 / Bn;
-  const int koff = key0 - c * Bn;  // offset of this 64-key block inside its column
   const int64_t bh = (int64_t)b * a.heads + h;
   int nnz = 0;
   int64_t lbase = 0;
@@ -137,11 +149,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     if (causal && nnz > 0) start = lower_bound_i32b(a.row_indices + lbase, nnz, key0 - off);
   }
   const int32_t *list = a.row_indices + lbase;
+  const int koff = key0 - c * Bn;  // offset of this 64-key block inside its column
 
   const uint16_t *qg = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)q0 * a.q_row_stride + (int64_t)h * a.q_head_stride;
   const uint16_t *dog = reinterpret_cast<const uint16_t *>(a.dout) + (int64_t)q0 * a.do_row_stride + (int64_t)h * a.do_head_stride;
   const float *lseg = a.softmax_lse + (int64_t)h * a.total_q + q0;
   const float *delg = a.softmax_d + (int64_t)h * ((int64_t)a.total_q + 128 * (int64_t)a.batch) + q0 + 128 * b;
+  int32_t *cntg = ws.cnt + (int64_t)q0 * a.heads + h;  // counter of local row r: cntg[r * heads]
 
   auto fill_list = [&](int seg0, int seg_len) {
     __syncthreads();
@@ -156,90 +170,87 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   // The two roles run separate code with the same barrier sequence, so that the loaders' rings and the
   // compute waves' accumulators and operands do not add up in the register allocation.
   if (is_loader) {
-    // loader state: two-deep rings (compile-time parity) of the gathered rows of two rounds
-    Pack8 lq0[NV], lq1[NV], ld0[NV], ld1[NV];
-    int lrow0 = -1, lrow1 = -1;
-    float llse0 = INFINITY, llse1 = INFINITY, ldel0 = 0.f, ldel1 = 0.f;
+    // two-deep rings (compile-time parity) of the gathered rows of two rounds.  Loads are unconditional
+    // (indices clamped, the surplus zeroed when stored) so that the compiler counts outstanding loads exactly.
+    typedef std::integral_constant<int, 0> P0;
+    typedef std::integral_constant<int, 1> P1;
+    Pack8 lq[2][NV], ld[2][NV];
+    int lrow[2] = {-1, -1}, lslot[2] = {0, 0};
+    float llse[2] = {INFINITY, INFINITY}, ldel[2] = {0.f, 0.f};
 
     for (int seg0 = start; seg0 < nnz; seg0 += kListCap) {
       const int seg_len = min(kListCap, nnz - seg0);
       fill_list(seg0, seg_len);
-      const int ntile = (seg_len + 31) >> 5;
-      const int nround = (ntile + 1) >> 1;
+      const int nround = (seg_len + 63) >> 6;
       auto load_round = [&](auto par, int r) {
         constexpr int P = decltype(par)::value;
-  #pragma unroll
+#pragma unroll
         for (int i = 0; i < NV; ++i) {
           const int v = lt + 128 * i;
-          const int row = v / VPR, e = (v - row * VPR) * 8;  // row 0..63 over the two tiles of the round
-          const int j = r * 64 + row;
-          const int rid = j < seg_len ? sList[j] : -1;
-          Pack8 xq = zero_pack8(), xo = zero_pack8();
-          if (rid >= 0 && e < D) {
-            xq = ld_global16(qg + (int64_t)rid * a.q_row_stride + e);
-            xo = ld_global16(dog + (int64_t)rid * a.do_row_stride + e);
-          }
-          if constexpr (P == 0) {
-            lq0[i] = xq;
-            ld0[i] = xo;
-          } else {
-            lq1[i] = xq;
-            ld1[i] = xo;
-          }
+          const int row = v / VPR, e = min((v - row * VPR) * 8, D - 8);  // row 0..63 over the two tiles of the round
+          const int rid = max(sList[min(r * 64 + row, seg_len - 1)], 0);
+          lq[P][i] = ld_global16(qg + (int64_t)rid * a.q_row_stride + e);
+          ld[P][i] = ld_global16(dog + (int64_t)rid * a.do_row_stride + e);
         }
         if (lt < 64) {
           const int j = r * 64 + lt;
           const int rid = j < seg_len ? sList[j] : -1;
-          float xl = INFINITY, xd = 0.f;
-          if (rid >= 0) {
-            xl = lseg[rid];
-            xd = delg[rid];
-          }
-          if constexpr (P == 0) {
-            lrow0 = rid;
-            llse0 = xl;
-            ldel0 = xd;
-          } else {
-            lrow1 = rid;
-            llse1 = xl;
-            ldel1 = xd;
+          const int rc = max(rid, 0);
+          lrow[P] = rid;
+          llse[P] = lseg[rc];
+          ldel[P] = delg[rc];
+          // every visit of a (row, key block) pair takes one dQ-partial slot of the row (the only conditional
+          // memory operation of the loader)
+          if constexpr (DQP) {
+            if (rid >= 0) lslot[P] = atomicAdd(cntg + (int64_t)rid * a.heads, 1);
           }
         }
       };
-      auto store_round = [&](auto par) {
+      auto store_round = [&](auto par, int r) {
         constexpr int P = decltype(par)::value;
-  #pragma unroll
+#pragma unroll
         for (int i = 0; i < NV; ++i) {
           const int v = lt + 128 * i;
           const int row = v / VPR, e = (v - row * VPR) * 8;
-          *reinterpret_cast<Pack8 *>(sQ + (P * 64 + row) * LDQ + e) = P == 0 ? lq0[i] : lq1[i];
-          *reinterpret_cast<Pack8 *>(sdO + (P * 64 + row) * LDQ + e) = P == 0 ? ld0[i] : ld1[i];
+          const int j = r * 64 + row;
+          const bool ok = e < D && j < seg_len && sList[min(j, seg_len - 1)] >= 0;
+          Pack8 xq = lq[P][i], xo = ld[P][i];
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            xq.w[w] = ok ? xq.w[w] : 0u;
+            xo.w[w] = ok ? xo.w[w] : 0u;
+          }
+          *reinterpret_cast<Pack8 *>(sQ + (P * 64 + row) * LDQ + e) = xq;
+          *reinterpret_cast<Pack8 *>(sdO + (P * 64 + row) * LDQ + e) = xo;
         }
         if (lt < 64) {
-          sRow[P * 64 + lt] = P == 0 ? lrow0 : lrow1;
-          sLse[P * 64 + lt] = (P == 0 ? llse0 : llse1) * kLog2e;
-          sDelta[P * 64 + lt] = P == 0 ? ldel0 : ldel1;
+          const bool ok = lrow[P] >= 0;
+          sRow[P * 64 + lt] = lrow[P];
+          sSlot[P * 64 + lt] = lslot[P];
+          sLse[P * 64 + lt] = ok ? llse[P] * kLog2e : INFINITY;  // absent rows: exp2(x - inf) = 0
+          sDelta[P * 64 + lt] = ok ? ldel[P] : 0.f;
         }
       };
 
-      typedef std::integral_constant<int, 0> P0;
-      typedef std::integral_constant<int, 1> P1;
       // Tiles are double buffered in LDS by round parity, and so are the rings: during round r the loaders
       // put round r+1 into the other buffer and fetch round r+3 into the registers that this frees.
       load_round(P0{}, 0);
-      if (nround > 1) load_round(P1{}, 1);
-      store_round(P0{});
-      if (nround > 2) load_round(P0{}, 2);
+      load_round(P1{}, 1);  // past the end: rows clamp to the last one, nothing of it is used
+      store_round(P0{}, 0);
+      load_round(P0{}, 2);
       auto loader_round = [&](auto par, int r) {  // par: parity of round r + 1
+        // The compute waves exchange dS^T of the round's two tiles through LDS, which takes two more
+        // barriers per round; the loaders' work is spread between them so that nobody waits for it.
         __syncthreads();  // round r is in LDS; the readers of round r-1 are done with the other buffer
-        if (r + 1 < nround) {
-          store_round(par);
-          if (r + 3 < nround) load_round(par, r + 3);
-        }
+        if (r + 1 < nround) store_round(par, r + 1);
+        if constexpr (DQP) __syncthreads();
+        load_round(par, r + 3);
+        if constexpr (DQP) __syncthreads();
       };
-      for (int r = 0; r < nround; r += 2) {
+      const int nround_pad = (nround + 1) & ~1;
+      for (int r = 0; r < nround_pad; r += 2) {
         loader_round(P1{}, r);
-        if (r + 1 < nround) loader_round(P0{}, r + 1);
+        loader_round(P0{}, r + 1);
       }
     }
     __syncthreads();
@@ -269,15 +280,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       constexpr int KC = KS / 4;       // k-steps of S / dP per chunk
       constexpr int BC = NDT / 2;      // (d-tile, row-half) operand pairs of dV / dK per chunk
       lds_cu16 *trQ = tr_lane_base(sQ, LDQ, lane) + 4 * hh * LDQ, *trdO = tr_lane_base(sdO, LDQ, lane) + 4 * hh * LDQ;
-      lds_cu16 *trdS = tr_lane_base(sdS, LDS_, lane) + 8 * hh * LDS_;
+      lds_cu16 *trdS = tr_lane_base(sdS, LDS_, lane) + 8 * hh * LDS_;  // dS^T tile: 8 consecutive keys per read
+      lds_cu16 *trK = tr_lane_base(sK, LDQ, lane) + 8 * hh * LDQ;      // K^T with the same key order
+      uint16_t *sdQ = reinterpret_cast<uint16_t *>(smem + SM::odQ) + (size_t)kh * 32 * LDH;
       Pack8 qa[2][KC], doa[2][KC];     // A operands of S and dP (this lane's row, its half of the head dim), double-buffered by chunk
       Pack8 kb[2][KC], vb[2][KC];      // B operands: this lane's key, same slices of the head dim
       Pack8 dot[2][BC], qt[2][BC];     // dO^T / Q^T operands of the dV / dK products, double-buffered by chunk
       f32x4 lse4[2], del4[2];          // softmax inputs of a chunk's four rows
       int4 row4[2];
       Pack8 pf[2][2], dsf[2][2];       // P and dS of both tiles of the round as MFMA operands
-      Pack8 dsx[2];                    // dS rows on their way to the workspace
-      int dsrow = -1;
+      Pack8 dsx[4];                    // dS^T of all 64 keys as the B operand of the dQ products
+      Pack8 kt[NDH][4];                // K^T of this wave's half of the features
+      f32x16 dqa[NDH];
       f32x16 s[2], dp[2];
       auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
       auto ld_a = [&](auto pc, auto tsc, auto gc) {
@@ -353,31 +367,88 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         dsf[TS][G >> 1].w[2 * (G & 1)] = pack2<T>(ds[0], ds[1]);
         dsf[TS][G >> 1].w[2 * (G & 1) + 1] = pack2<T>(ds[2], ds[3]);
       };
-      // dS^T of this wave's 32 keys goes through its LDS tile [key][row] and comes back as rows: lane
-      // (row, hh) gets 8 consecutive keys per read and stores them to the workspace.  The transposing read
-      // exchanges data between lanes: every lane takes part, only the store is predicated.
+      // dQ of the tile: both waves put dS^T of their 32 keys into one LDS tile [64 keys][32 rows]; after a
+      // barrier each wave computes dQ^T = K^T dS^T over all 64 keys for ITS half of the features (K^T and
+      // dS^T through transposing reads, which exchange data between lanes: every lane takes part).  The
+      // half rows (16-bit, unscaled) go to the partial slot that the row handed out for this visit.
       auto ds_write = [&](auto tsc) {
         constexpr int TS = decltype(tsc)::value;
-  #pragma unroll
+        // DQP: tile slot TS, rows of both key halves; else: this wave's private half of tile slot 0
+        uint16_t *t = sdS + (size_t)((DQP ? TS * 64 : 0) + kh * 32 + (lane & 31)) * LDS_;
+#pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
-          *reinterpret_cast<uint2 *>(sdS + (lane & 31) * LDS_ + 16 * s2 + 4 * hh) = make_uint2(dsf[TS][s2].w[0], dsf[TS][s2].w[1]);
-          *reinterpret_cast<uint2 *>(sdS + (lane & 31) * LDS_ + 16 * s2 + 8 + 4 * hh) = make_uint2(dsf[TS][s2].w[2], dsf[TS][s2].w[3]);
+          *reinterpret_cast<uint2 *>(t + 16 * s2 + 4 * hh) = make_uint2(dsf[TS][s2].w[0], dsf[TS][s2].w[1]);
+          *reinterpret_cast<uint2 *>(t + 16 * s2 + 8 + 4 * hh) = make_uint2(dsf[TS][s2].w[2], dsf[TS][s2].w[3]);
         }
-        wave_lds_fence();
+        if constexpr (DQP)
+          __syncthreads();
+        else
+          wave_lds_fence();
       };
+      // dS form: the wave's 32 keys of every row go to the dS tile of the row's list entry
+      int dsrow = -1;
       auto ds_read = [&](auto pc, auto tsc) {
         constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value;
         dsrow = sRow[TS * 32 + (lane & 31)];
-  #pragma unroll
-        for (int s4 = 0; s4 < 2; ++s4) dsx[s4] = tr_frag8_at(trdS, 16 * s4 * LDS_, (16 * s4 + 4) * LDS_);
+#pragma unroll
+        for (int s4 = 0; s4 < 2; ++s4) dsx[s4] = tr_frag8_at(trdS, (kh * 32 + 16 * s4) * LDS_, (kh * 32 + 16 * s4 + 4) * LDS_);
         wave_lds_fence();
       };
       auto ds_store = [&](int tile) {
         if (dsrow >= 0) {
-          uint16_t *wp = ds_ws + (lbase + seg0 + tile * 32 + (lane & 31)) * Bn + koff + kh * 32;
-  #pragma unroll
+          uint16_t *wp = ws.ds + (lbase + seg0 + tile * 32 + (lane & 31)) * Bn + koff + kh * 32;
+#pragma unroll
           for (int s4 = 0; s4 < 2; ++s4) *reinterpret_cast<Pack8 *>(wp + 16 * s4 + 8 * hh) = dsx[s4];
         }
+      };
+      auto dq_load = [&](auto tsc) {
+        constexpr int TS = decltype(tsc)::value;
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) {
+          dsx[s4] = tr_frag8_at(trdS, (TS * 64 + 16 * s4) * LDS_, (TS * 64 + 16 * s4 + 4) * LDS_);
+#pragma unroll
+          for (int d2 = 0; d2 < NDH; ++d2) {
+            const int lo = 16 * s4 * LDQ + (kh * NDH + d2) * 32;
+            kt[d2][s4] = tr_frag8_at(trK, lo, lo + 4 * LDQ);
+          }
+        }
+      };
+      auto dq_mma = [&](auto gc) {  // a quarter of the products per chunk
+        constexpr int G = decltype(gc)::value;
+#pragma unroll
+        for (int d2 = 0; d2 < NDH; ++d2) {
+          if constexpr (G == 0) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dqa[d2][i] = 0.f;
+          }
+          dqa[d2] = mfma32<T>(kt[d2][G], dsx[G], dqa[d2]);
+        }
+      };
+      const int64_t trash = (int64_t)a.total_q * a.heads * ws.cap;  // spare row: takes the writes of absent rows, no branch
+      auto dq_store = [&](auto pc, auto tsc) {
+        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value;
+        // register i of feature tile d2 <-> feature d2*32 + acc_row(i, hh) of this wave's half, this lane's row
+#pragma unroll
+        for (int d2 = 0; d2 < NDH; ++d2)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            *reinterpret_cast<uint2 *>(sdQ + (lane & 31) * LDH + d2 * 32 + 8 * g + 4 * hh) =
+                make_uint2(pack2<T>(dqa[d2][4 * g], dqa[d2][4 * g + 1]), pack2<T>(dqa[d2][4 * g + 2], dqa[d2][4 * g + 3]));
+        wave_lds_fence();
+        constexpr int LPR = HD / 16;        // lanes per half row (16 bytes each)
+        constexpr int RPP = 64 / LPR;       // rows per pass
+        const int col = (lane % LPR) * 8;
+#pragma unroll
+        for (int k = 0; k < 32 / RPP; ++k) {
+          const int row = k * RPP + lane / LPR;
+          const int r2 = sRow[TS * 32 + row], s2 = sSlot[TS * 32 + row];
+          const Pack8 x = *reinterpret_cast<const Pack8 *>(sdQ + row * LDH + col);
+          const bool ok = r2 >= 0 && s2 < ws.cap;
+          const int64_t pidx = ok ? ((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2 : trash;
+          if (kh * (HD / 2) + col < D) *reinterpret_cast<Pack8 *>(ws.part + pidx * D + kh * (HD / 2) + col) = x;
+          if (kh == 0 && col == 0) ws.pid[pidx] = nb;
+        }
+        wave_lds_fence();
       };
       // One round = tiles 2r and 2r+1, both already in LDS.  A list with an odd number of tiles ends with a tile
       // of absent rows (row id -1, zero data): it runs through the same code and adds nothing.
@@ -405,11 +476,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           smx(C0{}, gc);
           fence();
         });
-        // dV, dK of the first tile between the softmax rows of the second
+        // dV, dK, dQ of the first tile between the softmax rows of the second
         ds_write(C0{});
         ld_b(pc, C0{}, C0{});
         ld_s(pc, C1{}, C0{});
-        ds_read(pc, C0{});
+        if constexpr (DQP)
+          dq_load(C0{});
+        else
+          ds_read(pc, C0{});
         fence();
         static_for<4>([&](auto gc) {
           constexpr int G = decltype(gc)::value;
@@ -418,30 +492,41 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
             ld_s(pc, C1{}, std::integral_constant<int, G + 1>{});
           }
           mm_b(C0{}, gc);
+          if constexpr (DQP) dq_mma(gc);
           smx(C1{}, gc);
-          if constexpr (G == 1) ds_store(2 * r);
+          if constexpr (!DQP && G == 1) ds_store(2 * r);
           fence();
         });
-        // dV, dK of the second tile
+        if constexpr (DQP) dq_store(pc, C0{});
+        // dV, dK, dQ of the second tile
         ds_write(C1{});
         ld_b(pc, C1{}, C0{});
-        ds_read(pc, C1{});
+        if constexpr (DQP)
+          dq_load(C1{});
+        else
+          ds_read(pc, C1{});
         fence();
         static_for<4>([&](auto gc) {
           constexpr int G = decltype(gc)::value;
           if constexpr (G < 3) ld_b(pc, C1{}, std::integral_constant<int, G + 1>{});
           mm_b(C1{}, gc);
-          if constexpr (G == 1) ds_store(2 * r + 1);
+          if constexpr (DQP) dq_mma(gc);
+          if constexpr (!DQP && G == 1) ds_store(2 * r + 1);
           fence();
         });
+        if constexpr (DQP) dq_store(pc, C1{});
       };
 
-      for (int r = 0; r < nround; r += 2) {
+      const int nround_pad = (nround + 1) & ~1;
+      for (int r = 0; r < nround_pad; r += 2) {
         __syncthreads();  // round r is in LDS
         process_round(C0{}, r);
+        __syncthreads();
         if (r + 1 < nround) {
-          __syncthreads();
           process_round(C1{}, r + 1);
+        } else if constexpr (DQP) {  // padding round: only the barriers
+          __syncthreads();
+          __syncthreads();
         }
       }
     }
@@ -759,6 +844,59 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
   }
 }
 
+// ------------------------------------------------------------------------------------
+// dQ, second form: one wave per (row, head) adds the row's partials in ascending key-block order (sorted by
+// block id: the slot a visit got is arbitrary, the sum must not depend on it) and scales.
+// ------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void attn_bwd_dq_combine_kernel(fmoba_attn_bwd_args a, BwdWs ws) {
+  __shared__ int sOrd[4][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t rh = (int64_t)blockIdx.x * 4 + wv;  // (global row) * heads + head
+  if (rh >= (int64_t)a.total_q * a.heads) return;
+  const int64_t row = rh / a.heads;
+  const int h = (int)(rh - row * a.heads);
+  const int D = a.head_dim;
+  const int n = min(ws.cnt[rh], ws.cap);
+  const bool mine = 2 * lane < D;
+  const int32_t *pid = ws.pid + rh * ws.cap;
+  const uint16_t *part = ws.part + rh * ws.cap * D;
+  float acc0 = 0.f, acc1 = 0.f;
+  for (int base = 0; base < n; base += 64) {
+    const int cntb = min(64, n - base);
+    const int cj = lane < cntb ? pid[base + lane] : 0x7fffffff;
+    int rank = 0;
+    for (int i = 0; i < cntb; ++i) {
+      const int ci = __shfl(cj, i, 64);
+      rank += (ci < cj || (ci == cj && i < lane)) ? 1 : 0;
+    }
+    wave_lds_fence();
+    if (lane < cntb) sOrd[wv][rank] = lane;
+    wave_lds_fence();
+    if (mine) {
+      int t = 0;
+      for (; t + 4 <= cntb; t += 4) {
+        uint32_t x[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const uint32_t *>(part + (int64_t)(base + sOrd[wv][t + u]) * D + 2 * lane);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          acc0 += elem_to_float<T>((uint16_t)(x[u] & 0xffffu));
+          acc1 += elem_to_float<T>((uint16_t)(x[u] >> 16));
+        }
+      }
+      for (; t < cntb; ++t) {
+        const uint32_t x = *reinterpret_cast<const uint32_t *>(part + (int64_t)(base + sOrd[wv][t]) * D + 2 * lane);
+        acc0 += elem_to_float<T>((uint16_t)(x & 0xffffu));
+        acc1 += elem_to_float<T>((uint16_t)(x >> 16));
+      }
+    }
+  }
+  if (mine)
+    *reinterpret_cast<uint32_t *>(reinterpret_cast<uint16_t *>(a.dq) + row * a.dq_row_stride + (int64_t)h * a.dq_head_stride + 2 * lane) =
+        pack2<T>(acc0 * a.softmax_scale, acc1 * a.softmax_scale);
+}
+
 // grid (ceil(max_seqlen_q / rows_per_block), heads, batch), block 256.
 // LPR lanes cooperate on one row (LPR = power of two >= head_dim / 8).
 template <typename T>
@@ -797,13 +935,17 @@ __global__ void zero_rows_kernel(void *p, int64_t rows, int64_t row_stride, int 
   }
 }
 
+__global__ void zero_i32_kernel(int32_t *p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
 __global__ void zero_f32_kernel(float *p, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.f;
 }
 
-template <typename T, int HD>
-static int launch_dkdv(const fmoba_attn_bwd_args &a, uint16_t *ws, hipStream_t s) {
-  auto kern = attn_bwd_dkdv_kernel<T, HD>;
+template <typename T, int HD, bool DQP>
+static int launch_dkdv(const fmoba_attn_bwd_args &a, const BwdWs &ws, hipStream_t s) {
+  auto kern = attn_bwd_dkdv_kernel<T, HD, DQP>;
   const size_t smem = BwdSmem<HD>::bytes;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("attn_bwd: cannot reserve %zu bytes of LDS", smem);
@@ -833,8 +975,20 @@ static int launch_dq(const fmoba_attn_bwd_args &a, const uint16_t *ws, hipStream
   return 0;
 }
 
+// Which form of the dQ computation a call uses.  The row-stationary form works on (128-row block, key block) steps
+// and is the faster one while a step has a dozen rows or more; with many chunks per sequence a step has one or
+// two rows and only the per-visit partials scale.  rows per step ~ 128 * (chunks a row selects) / (chunks per sequence).
+static int bwd_dq_partials(const fmoba_attn_bwd_args &a) {
+  if (a.dq_mode == 1) return 0;
+  if (a.dq_mode == 2) return 1;
+  const double chunks_per_seq = (double)a.total_k / a.batch / a.lg_block_n;
+  const double chunks_per_row = (double)a.max_visits_per_row * 64.0 / a.lg_block_n;
+  return 128.0 * chunks_per_row < 12.0 * chunks_per_seq;
+}
+
 template <typename T>
-static int run_bwd(const fmoba_attn_bwd_args &a, uint16_t *ws, int phases, hipStream_t s) {
+static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hipStream_t s) {
+  const bool partials = bwd_dq_partials(a);
   if (phases & FMOBA_BWD_PREP) {
     int lpr = 1;
     while (lpr * 8 < a.head_dim) lpr <<= 1;
@@ -842,21 +996,43 @@ static int run_bwd(const fmoba_attn_bwd_args &a, uint16_t *ws, int phases, hipSt
     hipLaunchKernelGGL(bwd_prep_kernel<T>, dim3(ceil_div(a.max_seqlen_q, rows_per_block), a.heads, a.batch), dim3(256), 0, s, a, lpr);
   }
   if (phases & FMOBA_BWD_DKDV) {
-    int rc = a.head_dim <= 64 ? launch_dkdv<T, 64>(a, ws, s) : launch_dkdv<T, 128>(a, ws, s);
+    int rc;
+    if (partials) {
+      hipLaunchKernelGGL(zero_i32_kernel, dim3(512), dim3(256), 0, s, ws.cnt, (int64_t)a.total_q * a.heads);
+      rc = a.head_dim <= 64 ? launch_dkdv<T, 64, true>(a, ws, s) : launch_dkdv<T, 128, true>(a, ws, s);
+    } else {
+      rc = a.head_dim <= 64 ? launch_dkdv<T, 64, false>(a, ws, s) : launch_dkdv<T, 128, false>(a, ws, s);
+    }
     if (rc) return rc;
   }
   if (phases & FMOBA_BWD_DQ) {
-    int rc = a.head_dim <= 64 ? launch_dq<T, 64>(a, ws, s) : launch_dq<T, 128>(a, ws, s);
-    if (rc) return rc;
+    if (partials) {
+      const int64_t rows = (int64_t)a.total_q * a.heads;
+      hipLaunchKernelGGL(attn_bwd_dq_combine_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, a, ws);
+    } else {
+      int rc = a.head_dim <= 64 ? launch_dq<T, 64>(a, ws.ds, s) : launch_dq<T, 128>(a, ws.ds, s);
+      if (rc) return rc;
+    }
   }
   return 0;
 }
 
+static inline size_t bwd_align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
 }  // namespace fmoba
 
-extern "C" size_t fmoba_attn_bwd_workspace_bytes(int64_t num_row_indices, int32_t lg_block_n) {
-  if (num_row_indices <= 0 || lg_block_n <= 0) return 256;
-  return (size_t)num_row_indices * lg_block_n * 2 + 256;
+extern "C" int32_t fmoba_attn_bwd_uses_partials(const fmoba_attn_bwd_args *a) {
+  if (a == nullptr || a->batch <= 0 || a->lg_block_n <= 0) return 0;
+  return fmoba::bwd_dq_partials(*a);
+}
+
+extern "C" size_t fmoba_attn_bwd_workspace_bytes(const fmoba_attn_bwd_args *a) {
+  using namespace fmoba;
+  if (a == nullptr || a->total_q <= 0 || a->heads <= 0 || a->head_dim <= 0 || a->batch <= 0 || a->lg_block_n <= 0) return 256;
+  if (!bwd_dq_partials(*a)) return (size_t)(a->num_row_indices > 0 ? a->num_row_indices : 0) * a->lg_block_n * 2 + 256;
+  const size_t rows = (size_t)a->total_q * a->heads, cap = (size_t)(a->max_visits_per_row > 0 ? a->max_visits_per_row : 1);
+  // one spare partial row / block id at the end takes the writes of absent rows
+  return bwd_align256(rows * 4) + bwd_align256((rows * cap + 1) * 4) + bwd_align256((rows * cap + 1) * a->head_dim * 2) + 256;
 }
 
 extern "C" int fmoba_attn_bwd(const fmoba_attn_bwd_args *a, void *stream) { return fmoba_attn_bwd_phases(a, 7, stream); }
@@ -874,7 +1050,7 @@ extern "C" int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phase
   FMOBA_REQUIRE(a->lg_block_m % 64 == 0, "m_lg_block_dim must be a multiple of 64");
   FMOBA_REQUIRE(a->lg_block_n > 0 && a->lg_block_n % 64 == 0, "n_lg_block_dim must be a multiple of 64");
   FMOBA_REQUIRE(a->lg_block_n <= 64 * 256, "attn_bwd: n_lg_block_dim above 16384 is not supported");
-  FMOBA_REQUIRE(a->total_q >= 0 && a->total_k >= 0 && a->max_seqlen_q >= 0 && a->max_seqlen_k >= 0 && a->max_cols >= 0 && a->num_row_indices >= 0,
+  FMOBA_REQUIRE(a->total_q >= 0 && a->total_k >= 0 && a->max_seqlen_q >= 0 && a->max_seqlen_k >= 0 && a->max_cols >= 0 && a->max_visits_per_row >= 0 && a->num_row_indices >= 0,
                 "negative size");
   FMOBA_REQUIRE(a->cu_seqlens_q && a->cu_seqlens_k, "attn_bwd: null cu_seqlens pointer");
   FMOBA_REQUIRE(a->batch <= 65535 && a->heads <= 65535, "attn_bwd: batch/heads too large for the launch grid");
@@ -909,9 +1085,19 @@ extern "C" int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phase
     return 0;
   }
   FMOBA_REQUIRE(a->k && a->v && a->col_offsets && a->col_nnz && a->row_indices, "attn_bwd: null k/v/CSC pointer");
-  FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= fmoba_attn_bwd_workspace_bytes(a->num_row_indices, a->lg_block_n),
-                "attn_bwd: workspace too small");
-  uint16_t *ws = reinterpret_cast<uint16_t *>(((uintptr_t)a->workspace + 255) & ~(uintptr_t)255);
+  FMOBA_REQUIRE(a->max_visits_per_row > 0, "attn_bwd: max_visits_per_row must be positive");
+  FMOBA_REQUIRE(a->dq_mode >= 0 && a->dq_mode <= 2, "attn_bwd: dq_mode must be 0 (automatic), 1 (row blocks) or 2 (partials)");
+  FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= fmoba_attn_bwd_workspace_bytes(a), "attn_bwd: workspace too small");
+  const size_t rows = (size_t)a->total_q * a->heads;
+  uintptr_t wp = ((uintptr_t)a->workspace + 255) & ~(uintptr_t)255;
+  BwdWs ws;
+  ws.cap = a->max_visits_per_row;
+  ws.ds = reinterpret_cast<uint16_t *>(wp);
+  ws.cnt = reinterpret_cast<int32_t *>(wp);
+  wp += bwd_align256(rows * 4);
+  ws.pid = reinterpret_cast<int32_t *>(wp);
+  wp += bwd_align256((rows * ws.cap + 1) * 4);
+  ws.part = reinterpret_cast<uint16_t *>(wp);
   int rc = a->dtype == FMOBA_DTYPE_BF16 ? run_bwd<bf16_t>(*a, ws, phases, s) : run_bwd<f16_t>(*a, ws, phases, s);
   if (rc) return rc;
   FMOBA_LAUNCH_CHECK("attn_bwd");

@@ -71,7 +71,7 @@ class AttnBwdArgs(ctypes.Structure):
                 ("batch", c_i32), ("total_q", c_i32), ("total_k", c_i32), ("heads", c_i32), ("heads_k", c_i32),
                 ("head_dim", c_i32), ("max_seqlen_q", c_i32), ("max_seqlen_k", c_i32), ("max_cols", c_i32),
                 ("lg_block_m", c_i32), ("lg_block_n", c_i32), ("is_causal", c_i32), ("dtype", c_i32),
-                ("deterministic", c_i32), ("softmax_scale", c_f32),
+                ("deterministic", c_i32), ("max_visits_per_row", c_i32), ("dq_mode", c_i32), ("softmax_scale", c_f32),
                 ("q_row_stride", c_i64), ("q_head_stride", c_i64), ("k_row_stride", c_i64), ("k_head_stride", c_i64),
                 ("v_row_stride", c_i64), ("v_head_stride", c_i64), ("o_row_stride", c_i64), ("o_head_stride", c_i64),
                 ("do_row_stride", c_i64), ("do_head_stride", c_i64),
@@ -92,7 +92,8 @@ EXPORTS = {
     "fmoba_attn_fwd_workspace_bytes": (c_sz, [c_i32, c_i32, c_i32, c_i32]),
     "fmoba_csc_max_row_visits": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp, c_vp, c_vp]),
     "fmoba_attn_fwd": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp]),
-    "fmoba_attn_bwd_workspace_bytes": (c_sz, [c_i64, c_i32]),
+    "fmoba_attn_bwd_workspace_bytes": (c_sz, [ctypes.POINTER(AttnBwdArgs)]),
+    "fmoba_attn_bwd_uses_partials": (c_i32, [ctypes.POINTER(AttnBwdArgs)]),
     "fmoba_attn_bwd": (c_i32, [ctypes.POINTER(AttnBwdArgs), c_vp]),
     "fmoba_attn_bwd_phases": (c_i32, [ctypes.POINTER(AttnBwdArgs), c_i32, c_vp]),
 }
@@ -291,7 +292,33 @@ _hint = threading.local()
 
 
 def set_visits_hint(n):
+    """Bound (in forward key blocks) for the next forward call of this thread."""
     _hint.value = None if n is None else int(n)
+
+
+def set_bwd_visits_hint(n):
+    """Bound (in 64-key blocks) for the next backward call of this thread."""
+    _hint.bwd = None if n is None else int(n)
+
+
+def last_fwd_visits():
+    """The bound the last forward call of this thread used, in forward key blocks."""
+    return getattr(_hint, "last", None)
+
+
+def _count_visits(lib, q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k, batch, total_q, total_k,
+                  heads, heads_k, d, max_seqlen_q, max_seqlen_k, max_cols, m_lg_block_dim, n_lg_block_dim):
+    """Largest number of (row, forward key block) visits of any (row, head) of the pattern: one pass + one read."""
+    if total_q == 0 or total_k == 0 or max_cols == 0:
+        return 1
+    counts = torch.empty((total_q * heads + 1,), dtype=torch.int32, device=q.device)
+    a0 = AttnFwdArgs(None, None, None, None, None,
+                     moba_col_offsets.data_ptr(), moba_col_nnz.data_ptr(), moba_row_indices.data_ptr(),
+                     cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), None, 0,
+                     batch, total_q, total_k, heads, heads_k, d, int(max_seqlen_q), int(max_seqlen_k), max_cols,
+                     int(m_lg_block_dim), int(n_lg_block_dim), 0, _dt(q), 0, 1.0, 0, 0, 0, 0, 0, 0, 0, 0)
+    _check(lib.fmoba_csc_max_row_visits(ctypes.byref(a0), counts.data_ptr(), counts[total_q * heads:].data_ptr(), _stream()))
+    return max(1, int(counts[total_q * heads].item()))
 
 
 def fwd_key_block(n_lg_block_dim):
@@ -355,12 +382,12 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
                                out.stride(0), out.stride(1))
 
         visits = hint
-        if visits is None and total_q > 0 and total_k > 0 and max_cols > 0:
-            counts = torch.empty((total_q * heads + 1,), dtype=torch.int32, device=q.device)
-            a0 = args(None, 0, 0)
-            _check(lib.fmoba_csc_max_row_visits(ctypes.byref(a0), counts.data_ptr(), counts[total_q * heads:].data_ptr(), _stream()))
-            visits = int(counts[total_q * heads].item())
-        visits = max(1, int(visits or 1))
+        if visits is None:
+            visits = _count_visits(lib, q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k, batch,
+                                   total_q, total_k, heads, heads_k, d, max_seqlen_q, max_seqlen_k, max_cols,
+                                   m_lg_block_dim, n_lg_block_dim)
+        visits = max(1, int(visits))
+        _hint.last = visits
         ws_bytes = lib.fmoba_attn_fwd_workspace_bytes(total_q, heads, d, visits)
         ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=q.device)
         a = args(ws.data_ptr(), ws_bytes, visits)
@@ -374,7 +401,7 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
 def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_offsets, moba_col_nnz, moba_row_indices,
                     cu_seqlens_q, cu_seqlens_k, alibi_slopes, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                     zero_tensors, is_causal, softcap, deterministic, m_lg_block_dim, n_lg_block_dim, gen=None,
-                    rng_state=None, _phases=None):
+                    rng_state=None, _phases=None, _dq_mode=0):
     """Returns [dq, dk, dv, softmax_d (H, total_q + 128*batch) fp32]."""
     dtype = q.dtype
     _require(dtype in (torch.float16, torch.bfloat16), "FlashMoBA only support fp16 and bf16 data type")
@@ -430,19 +457,27 @@ def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_off
         else:
             dk_e, dv_e = dk, dv
         lib = load_library()
-        n_idx = int(moba_row_indices.numel())
-        ws_bytes = lib.fmoba_attn_bwd_workspace_bytes(n_idx, int(n_lg_block_dim))
-        ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+        visits = getattr(_hint, "bwd", None)
+        _hint.bwd = None
+        if visits is None:
+            kb = int(lib.fmoba_attn_fwd_key_block(int(n_lg_block_dim)))
+            visits = (kb // 64) * _count_visits(lib, q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q,
+                                                cu_seqlens_k, batch, total_q, total_k, heads, heads_k, d, max_seqlen_q,
+                                                max_seqlen_k, max_cols, 128, n_lg_block_dim)
+        visits = max(1, int(visits))
         a = AttnBwdArgs(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), softmax_lse.data_ptr(),
                         dq.data_ptr(), dk_e.data_ptr(), dv_e.data_ptr(), softmax_d.data_ptr(),
                         moba_col_offsets.data_ptr(), moba_col_nnz.data_ptr(), moba_row_indices.data_ptr(),
-                        cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ws.data_ptr(), ws_bytes, n_idx,
+                        cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), None, 0, int(moba_row_indices.numel()),
                         batch, total_q, total_k, heads, heads_k, d, int(max_seqlen_q), int(max_seqlen_k), max_cols,
                         int(m_lg_block_dim), int(n_lg_block_dim), int(bool(is_causal)), _dt(q), int(bool(deterministic)),
-                        float(softmax_scale),
+                        visits, int(_dq_mode), float(softmax_scale),
                         q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                         out.stride(0), out.stride(1), dout.stride(0), dout.stride(1),
                         dq.stride(0), dq.stride(1), dk_e.stride(0), dk_e.stride(1), dv_e.stride(0), dv_e.stride(1))
+        ws_bytes = lib.fmoba_attn_bwd_workspace_bytes(ctypes.byref(a))
+        ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
         if _phases is None:
             _check(lib.fmoba_attn_bwd(ctypes.byref(a), _stream()))
         else:  # measurement hook: callable(run) receives run(mask) launching the chosen phases

@@ -223,6 +223,9 @@ class FlashMobaAttnVarlenFunc(torch.autograd.Function):
             dropout_p, softmax_scale, causal=causal, softcap=softcap, alibi_slopes=alibi_slopes,
             return_softmax=return_softmax and dropout_p > 0)
         if needs_grad:
+            # visits bound the forward worked with, converted to the backward's 64-key blocks
+            fwd_visits = flash_moba_gpu.last_fwd_visits()
+            ctx.bwd_visits = None if fwd_visits is None else fwd_visits * (flash_moba_gpu.fwd_key_block(lg_block_n) // 64)
             ctx.save_for_backward(q, k, v, out_padded, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state,
                                   moba_col_offsets, moba_col_nnz, moba_row_indices)
             ctx.cfg = (max_seqlen_q, max_seqlen_k, lg_block_m, lg_block_n, dropout_p, softmax_scale, causal,
@@ -238,6 +241,7 @@ class FlashMobaAttnVarlenFunc(torch.autograd.Function):
          softcap, alibi_slopes, deterministic) = ctx.cfg
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         (dout_padded,) = _pad8(dout)
+        flash_moba_gpu.set_bwd_visits_hint(ctx.bwd_visits)
         _wrapped_flash_moba_attn_varlen_backward(
             dout_padded, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
             max_seqlen_q, max_seqlen_k, col_offsets, col_nnz, row_indices, lg_block_m, lg_block_n,

@@ -150,12 +150,22 @@ int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream);
  *   GQA/MQA the caller sums groups of heads/heads_k (flash_moba_api.cpp:842-845).
  *   softmax_d (heads, total_q + 128*batch) fp32: row (b, r) of head h is stored at
  *   h*(total_q + 128*batch) + cu_q[b] + 128*b + r (flash_bwd_preprocess_kernel.h:86).
- *   workspace: the dS tiles (16-bit, one row of lg_block_n entries per entry of
- *   row_indices) that carry the result of the column-stationary dK/dV pass to the
- *   row-stationary dQ pass; fmoba_attn_bwd_workspace_bytes() bytes, contents undefined on
- *   entry and on return.  num_row_indices = number of int32 entries of row_indices
- *   (every col_offsets[i] + col_nnz[i] must be <= it).  No atomics: results are
- *   bitwise reproducible whatever `deterministic` says.
+ *   dK/dV come from one column-stationary pass.  dQ has two forms (dq_mode: 0 = the library
+ *   chooses, 1 = row blocks, 2 = partials; fmoba_attn_bwd_uses_partials() tells the choice):
+ *     row blocks: the dK/dV pass leaves the dS tiles (16-bit, lg_block_n entries per entry of
+ *       row_indices) in the workspace and a row-stationary pass (128 query rows per workgroup,
+ *       accumulators in LDS) multiplies them with K;
+ *     partials: the dK/dV pass leaves one dQ partial row (16-bit) per visit of a (query row,
+ *       64-key block) pair, a second launch adds the partials of each row in key order.  This is
+ *       the form that scales when sequences have thousands of chunks.
+ *   workspace: fmoba_attn_bwd_workspace_bytes(args) bytes (only the sizes, dq_mode,
+ *   num_row_indices and max_visits_per_row of args are read), contents undefined on entry and on
+ *   return.  num_row_indices = number of int32 entries of row_indices (every col_offsets[i] +
+ *   col_nnz[i] must be <= it).  max_visits_per_row bounds the visits of any (row, head): for a
+ *   pattern from the gating topk * lg_block_n / 64; for an arbitrary pattern
+ *   fmoba_csc_max_row_visits() counts them in forward key blocks, multiply by
+ *   fmoba_attn_fwd_key_block(lg_block_n) / 64.  Visits beyond the bound are dropped.
+ *   No floating-point atomics: results are bitwise reproducible whatever `deterministic` says.
  * ---------------------------------------------------------------------------------- */
 typedef struct {
   const void *dout, *q, *k, *v, *out;
@@ -173,6 +183,7 @@ typedef struct {
   int32_t max_seqlen_q, max_seqlen_k, max_cols;
   int32_t lg_block_m, lg_block_n;
   int32_t is_causal, dtype, deterministic;
+  int32_t max_visits_per_row, dq_mode;
   float softmax_scale;
   int64_t q_row_stride, q_head_stride, k_row_stride, k_head_stride;
   int64_t v_row_stride, v_head_stride, o_row_stride, o_head_stride;
@@ -180,13 +191,13 @@ typedef struct {
   int64_t dq_row_stride, dq_head_stride, dk_row_stride, dk_head_stride;
   int64_t dv_row_stride, dv_head_stride;
 } fmoba_attn_bwd_args;
-size_t fmoba_attn_bwd_workspace_bytes(int64_t num_row_indices, int32_t lg_block_n);
+int32_t fmoba_attn_bwd_uses_partials(const fmoba_attn_bwd_args *a);
+size_t fmoba_attn_bwd_workspace_bytes(const fmoba_attn_bwd_args *a);
 int fmoba_attn_bwd(const fmoba_attn_bwd_args *a, void *stream);
 /* The same call split into its three launches so that each can be timed on its own:
  * phases is a bit mask, 1 = dot(dO, O) (flash_bwd_launch_template.h:70-74), 2 = the
- * column-stationary dK/dV kernel, which also fills the workspace (:76-96), 4 = the
- * row-stationary dQ kernel, which reads it (stands where the reference converts its fp32
- * dQ accumulator, :98-104).  fmoba_attn_bwd(a, s) == fmoba_attn_bwd_phases(a, 7, s). */
+ * column-stationary dK/dV kernel, which also fills the workspace (:76-96), 4 = the dQ pass
+ * in either form (stands where the reference converts its fp32 dQ accumulator, :98-104).  fmoba_attn_bwd(a, s) == fmoba_attn_bwd_phases(a, 7, s). */
 #define FMOBA_BWD_PREP 1
 #define FMOBA_BWD_DKDV 2
 #define FMOBA_BWD_DQ 4

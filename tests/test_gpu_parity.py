@@ -346,6 +346,29 @@ def test_attention_random_pattern(fm, sq, sk, d, mha, causal, dtype):
     _check_attention(fm, q, k, v, dout, cuq, cuk, co, cn, ind, 64, causal)
 
 
+@pytest.mark.parametrize("dq_mode", [1, 2])
+@pytest.mark.parametrize("d,chunk", [(128, 64), (64, 128), (96, 64)])
+def test_backward_both_dq_forms(fm, dq_mode, d, chunk):
+    # the library picks the dQ form by shape; both are checked here whatever it would pick
+    lens = [300, 0, 77, 650]
+    q, k, v, cu, dout = O.make_inputs(lens, 4, d, chunk, 33, torch.bfloat16, with_dout=True)
+    Q, K, V, CU, DO = q.cuda(), k.cuda(), v.cuda(), cu.cuda(), dout.cuda()
+    co, cn, ind = fm.api.flash_topk_varlen_func(Q, K, CU, CU, max(lens), max(lens), 3, chunk, causal=True)
+    scale = d ** -0.5
+    out, lse, _, _ = fm.hip.moba_varlen_fwd(Q, K, V, None, co, cn, ind, CU, CU, None, None, None, max(lens), max(lens), 0.0, scale,
+                                            False, True, 0.0, False, 128, chunk, None)
+    dq, dk, dv, _ = fm.hip.moba_varlen_bwd(DO, Q, K, V, out, lse, None, None, None, co, cn, ind, CU, CU, None, max(lens), max(lens),
+                                           0.0, scale, False, True, 0.0, False, 128, chunk, None, None, _dq_mode=dq_mode)
+    _, _, dq_ref, dk_ref, dv_ref = O.attn_fwd_bwd(q, k, v, dout, cu, cu, co.cpu(), cn.cpu(), ind.cpu(), chunk, None, True)
+    assert_close("dq", dq, dq_ref, 2e-2, 1e-2)
+    assert_close("dk", dk, dk_ref, 2e-2, 1e-2)
+    assert_close("dv", dv, dv_ref, 2e-2, 1e-2)
+    # no floating-point atomics in either form: a second run gives the same bits
+    dq2, dk2, dv2, _ = fm.hip.moba_varlen_bwd(DO, Q, K, V, out, lse, None, None, None, co, cn, ind, CU, CU, None, max(lens), max(lens),
+                                              0.0, scale, False, True, 0.0, False, 128, chunk, None, None, _dq_mode=dq_mode)
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+
+
 @pytest.mark.parametrize("chunk,topk", [(64, 4), (128, 3), (64, 32)])
 def test_attention_on_gated_pattern(fm, chunk, topk):
     lens = [640, 1, 0, 1300]

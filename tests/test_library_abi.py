@@ -42,7 +42,14 @@ def test_workspace_queries_are_pure_host_functions():
     assert b >= 16 * 7 * 65536 * 4 + 8 * 16 * 7 * 224 * 4
     assert lib.fmoba_fused_topk_workspace_bytes(0, 0, 0, 0, 0, 0) == 0
     assert lib.fmoba_varlen_sort_workspace_bytes(1000) == 4000
-    assert lib.fmoba_attn_bwd_workspace_bytes(1024, 128) >= 1024 * 128 * 2
+    a = H.AttnBwdArgs()
+    a.total_q, a.heads, a.head_dim, a.batch, a.total_k, a.lg_block_n, a.max_visits_per_row, a.num_row_indices = 1024, 4, 128, 1, 1024, 64, 8, 32768
+    a.dq_mode = 2
+    assert lib.fmoba_attn_bwd_workspace_bytes(ctypes.byref(a)) >= 1024 * 4 * 8 * 128 * 2
+    a.dq_mode = 1
+    assert lib.fmoba_attn_bwd_workspace_bytes(ctypes.byref(a)) >= 32768 * 64 * 2
+    assert lib.fmoba_attn_fwd_workspace_bytes(1024, 4, 128, 8) >= 1024 * 4 * 8 * (128 * 2 + 16)
+    assert lib.fmoba_attn_fwd_key_block(64) == 64 and lib.fmoba_attn_fwd_key_block(128) == 128 and lib.fmoba_attn_fwd_key_block(192) == 64
 
 
 def test_struct_sizes_match_the_header_layout():
