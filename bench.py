@@ -100,9 +100,10 @@ def time_events(fn, iters, warmup=1):
 # what the same counter reads for a plain 1 GiB copy (the summary of those runs is kept under profiles/).
 # Counter runs cannot be made from inside this script, so the figures are the committed measurement.
 MEASURED_TRAFFIC_BYTES = {
-    ("headline", "attn_fwd_kernel"): 1.712e9,
-    ("headline", "attn_bwd_dkdv_kernel"): 18.588e9,
-    ("headline", "attn_bwd_dq_kernel"): 4.774e9,
+    ("headline", "attn_fwd_col_kernel"): 16.307e9,
+    ("headline", "attn_fwd_combine_kernel"): 8.346e9,
+    ("headline", "attn_bwd_dkdv_kernel"): 18.632e9,
+    ("headline", "attn_bwd_dq_kernel"): 4.790e9,
 }
 
 
@@ -113,29 +114,36 @@ def cpu_baseline(q, k, v, cu, seqlens, chunk, topk, budget_s=12.0):
     from oracle import moba_oracle as O  # checker only: never on the product path
 
     torch.set_num_threads(os.cpu_count())
-    b = max(range(len(seqlens)), key=lambda i: seqlens[i])  # the longest sequence of the batch
-    L, start = seqlens[b], sum(seqlens[:b])
-    qs, ks, vs = (t[start:start + L].float().cpu() for t in (q, k, v))
-    cu0 = torch.tensor([0, L], dtype=torch.int32)
     H, D = q.shape[1], q.shape[2]
+    order = sorted(range(len(seqlens)), key=lambda i: -seqlens[i])  # longest sequences first
     t0 = time.perf_counter()
-    heads = 0
-    while heads < H and (time.perf_counter() - t0) < budget_s:
-        O.moba_dense_ref(qs[:, heads:heads + 1], ks[:, heads:heads + 1], vs[:, heads:heads + 1], cu0, cu0, chunk, topk, True,
-                         row_block=1024)
-        heads += 1
+    pairs, done = 0, []
+    for b in order:
+        L, start = seqlens[b], sum(seqlens[:b])
+        qs, ks, vs = (t[start:start + L].float().cpu() for t in (q, k, v))
+        cu0 = torch.tensor([0, L], dtype=torch.int32)
+        C = (L + chunk - 1) // chunk
+        per_head = (sum(min(chunk, L - c * chunk) * (min(chunk, L - c * chunk) + 1) // 2 for c in range(C))
+                    + chunk * chunk * sum(min(topk - 1, c) for c in range(C)))
+        heads = 0
+        while heads < H and (time.perf_counter() - t0) < budget_s:
+            O.moba_dense_ref(qs[:, heads:heads + 1], ks[:, heads:heads + 1], vs[:, heads:heads + 1], cu0, cu0, chunk, topk, True,
+                             row_block=1024)
+            heads += 1
+            pairs += per_head
+        if heads:
+            done.append(f"sequence {b} ({L} tokens) x {heads} heads")
+        if (time.perf_counter() - t0) >= budget_s:
+            break
     dt = time.perf_counter() - t0
-    C = (L + chunk - 1) // chunk
-    pairs = heads * (sum(min(chunk, L - c * chunk) * (min(chunk, L - c * chunk) + 1) // 2 for c in range(C))
-                     + chunk * chunk * sum(min(topk - 1, c) for c in range(C)))
     flops = 4.0 * D * pairs
     return {
         "value": flops / dt / 1e12,
         "unit": "TFLOP/s",
         "cores": os.cpu_count(),
         "kind": "port",
-        "sample": f"forward only, fp32, sequence {b} ({L} tokens, the longest) x {heads} of {H} heads, row-blocked dense-masked "
-                  f"attention; {dt:.1f} s of CPU time; effective sparse FLOPs / time",
+        "sample": "forward only, fp32, row-blocked dense-masked attention on " + ", ".join(done)
+                  + f"; {dt:.1f} s of CPU time; effective sparse FLOPs / time",
         "seconds": dt,
     }
 
@@ -214,19 +222,30 @@ def main():
     t_gate = time_events(lambda: hip.moba_fused_topk(qd, km, cu, cu, cu_km, max_len, max_len, topk, chunk, True, return_raw=False), it)
     visits = topk * (chunk // hip.fwd_key_block(chunk))  # the bound the gated path hands to the forward
 
-    def fwd():
+    def fwd(**kw):
         hip.set_visits_hint(visits)
         return hip.moba_varlen_fwd(qd, kd, vd, None, co, cn, ind, cu, cu, None, None, None, max_len, max_len, 0.0, scale,
-                                   False, True, 0.0, False, lg_m, chunk, None)
+                                   False, True, 0.0, False, lg_m, chunk, None, **kw)
+
+    fwd_phase_ms = {}
+
+    def run_fwd_phases(run):
+        run(3)
+        for name, mask in (("columns", 1), ("combine", 2)):
+            fwd_phase_ms[name] = time_events(lambda: run(mask), it)
+
+    fwd(_phases=run_fwd_phases)
 
     out, lse, _, _ = fwd()
     t_fwd = time_events(fwd, it)
     stages = {
         "mean_pool": {"ms": t_pool, "GBps": pool_bytes / t_pool / 1e6, "frac_hbm": pool_bytes / t_pool / 1e6 / PEAK_HBM_GBS},
         "topk_csc": {"ms": t_gate, "GBps": gate_bytes / t_gate / 1e6, "frac_hbm": gate_bytes / t_gate / 1e6 / PEAK_HBM_GBS},
-        "attn_fwd": {"ms": t_fwd, "TFLOPs": fwd_flops / t_fwd / 1e9, "frac_mfma": fwd_flops / t_fwd / 1e9 / PEAK_BF16_TFLOPS},
+        "attn_fwd": {"ms": t_fwd, "TFLOPs": fwd_flops / t_fwd / 1e9, "frac_mfma": fwd_flops / t_fwd / 1e9 / PEAK_BF16_TFLOPS,
+                     "phases_ms": fwd_phase_ms},
     }
-    kernels = {"attn_fwd_kernel": (t_fwd, fwd_flops, "mfma")}
+    # the column pass runs both forward GEMMs; the combine only merges partial rows
+    kernels = {"attn_fwd_col_kernel": (fwd_phase_ms["columns"], fwd_flops, "mfma")}
     if backward:
         dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
         phase_ms = {}
@@ -247,8 +266,9 @@ def main():
         t_bwd = time_events(bwd, it)
         stages["attn_bwd"] = {"ms": t_bwd, "TFLOPs": bwd_flops / t_bwd / 1e9, "frac_mfma": bwd_flops / t_bwd / 1e9 / PEAK_BF16_TFLOPS,
                               "phases_ms": phase_ms}
-        # the dK/dV kernel runs all five backward GEMMs (S, dP, dV, dK, dQ partials); the dQ phase only adds partial rows
-        kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 10.0 * D * pairs, "mfma")
+        # the dK/dV kernel runs four of the five backward GEMMs (S, dP, dV, dK); the fifth is in it as well when the
+        # library picks the partial-sum form of dQ (long sequences), else in the dQ kernel (this figure assumes the latter)
+        kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 8.0 * D * pairs, "mfma")
     # sort alone, on the CSC the gating produced (already sorted input; same traffic)
     t_sort = time_events(lambda: torch.ops.flash_moba._varlen_sort(co, cn, ind), it)
     sort_bytes = 2 * int(cn.sum().item()) * 4 + 2 * cn.numel() * 8

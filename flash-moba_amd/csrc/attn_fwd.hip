@@ -492,16 +492,20 @@ static int launch_fwd_col(const fmoba_attn_fwd_args &a, const FwdWs &ws, hipStre
   return 0;
 }
 template <typename T>
-static int run_fwd(const fmoba_attn_fwd_args &a, const FwdWs &ws, hipStream_t s) {
-  const int kb = fwd_key_block(a.lg_block_n);
-  int rc;
-  if (a.head_dim <= 64)
-    rc = kb == 128 ? launch_fwd_col<T, 64, 128>(a, ws, s) : launch_fwd_col<T, 64, 64>(a, ws, s);
-  else
-    rc = kb == 128 ? launch_fwd_col<T, 128, 128>(a, ws, s) : launch_fwd_col<T, 128, 64>(a, ws, s);
-  if (rc) return rc;
+static int run_fwd(const fmoba_attn_fwd_args &a, const FwdWs &ws, int phases, hipStream_t s) {
   const int64_t rows = (int64_t)a.total_q * a.heads;
-  hipLaunchKernelGGL(attn_fwd_combine_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, a, ws);
+  if (phases & FMOBA_FWD_COLUMNS) {
+    hipLaunchKernelGGL(fwd_zero_i32_kernel, dim3(512), dim3(256), 0, s, ws.cnt, rows);
+    const int kb = fwd_key_block(a.lg_block_n);
+    int rc;
+    if (a.head_dim <= 64)
+      rc = kb == 128 ? launch_fwd_col<T, 64, 128>(a, ws, s) : launch_fwd_col<T, 64, 64>(a, ws, s);
+    else
+      rc = kb == 128 ? launch_fwd_col<T, 128, 128>(a, ws, s) : launch_fwd_col<T, 128, 64>(a, ws, s);
+    if (rc) return rc;
+  }
+  if (phases & FMOBA_FWD_COMBINE)
+    hipLaunchKernelGGL(attn_fwd_combine_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, a, ws);
   return 0;
 }
 
@@ -551,9 +555,12 @@ extern "C" int fmoba_csc_max_row_visits(const fmoba_attn_fwd_args *a, int32_t *c
   return 0;
 }
 
-extern "C" int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream) {
+extern "C" int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream) { return fmoba_attn_fwd_phases(a, 3, stream); }
+
+extern "C" int fmoba_attn_fwd_phases(const fmoba_attn_fwd_args *a, int32_t phases, void *stream) {
   using namespace fmoba;
   if (int rc = fwd_check_common(a)) return rc;
+  FMOBA_REQUIRE(phases > 0 && phases <= 3, "attn_fwd: phases must be a mask of bits 1, 2");
   hipStream_t s = (hipStream_t)stream;
   if (a->total_q == 0 || a->max_seqlen_q == 0) return 0;
   FMOBA_REQUIRE(a->q && a->out && a->softmax_lse, "attn_fwd: null q/out/lse pointer");
@@ -584,8 +591,7 @@ extern "C" int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream) {
   ws.hdr = reinterpret_cast<float4 *>(p);
   p += fwd_align256(rows * ws.cap * 16);
   ws.part = reinterpret_cast<uint16_t *>(p);
-  hipLaunchKernelGGL(fwd_zero_i32_kernel, dim3(512), dim3(256), 0, s, ws.cnt, (int64_t)rows + 1);
-  int rc = a->dtype == FMOBA_DTYPE_BF16 ? run_fwd<bf16_t>(*a, ws, s) : run_fwd<f16_t>(*a, ws, s);
+  int rc = a->dtype == FMOBA_DTYPE_BF16 ? run_fwd<bf16_t>(*a, ws, phases, s) : run_fwd<f16_t>(*a, ws, phases, s);
   if (rc) return rc;
   FMOBA_LAUNCH_CHECK("attn_fwd");
   return 0;

@@ -92,6 +92,7 @@ EXPORTS = {
     "fmoba_attn_fwd_workspace_bytes": (c_sz, [c_i32, c_i32, c_i32, c_i32]),
     "fmoba_csc_max_row_visits": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp, c_vp, c_vp]),
     "fmoba_attn_fwd": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp]),
+    "fmoba_attn_fwd_phases": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_i32, c_vp]),
     "fmoba_attn_bwd_workspace_bytes": (c_sz, [ctypes.POINTER(AttnBwdArgs)]),
     "fmoba_attn_bwd_uses_partials": (c_i32, [ctypes.POINTER(AttnBwdArgs)]),
     "fmoba_attn_bwd": (c_i32, [ctypes.POINTER(AttnBwdArgs), c_vp]),
@@ -327,7 +328,7 @@ def fwd_key_block(n_lg_block_dim):
 
 def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k,
                     seqused_k, leftpad_k, alibi_slopes, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-                    zero_tensors, is_causal, softcap, return_softmax, m_lg_block_dim, n_lg_block_dim, gen=None):
+                    zero_tensors, is_causal, softcap, return_softmax, m_lg_block_dim, n_lg_block_dim, gen=None, _phases=None):
     """Returns [out, softmax_lse (H, total_q) fp32, p (empty), rng_state (2,) int64]."""
     dtype = q.dtype
     _require(dtype in (torch.float16, torch.bfloat16), "FlashMoBA only support fp16 and bf16 data type")
@@ -391,7 +392,10 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
         ws_bytes = lib.fmoba_attn_fwd_workspace_bytes(total_q, heads, d, visits)
         ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=q.device)
         a = args(ws.data_ptr(), ws_bytes, visits)
-        _check(lib.fmoba_attn_fwd(ctypes.byref(a), _stream()))
+        if _phases is None:
+            _check(lib.fmoba_attn_fwd(ctypes.byref(a), _stream()))
+        else:  # measurement hook: callable(run) receives run(mask) launching the chosen phases
+            _phases(lambda mask: _check(lib.fmoba_attn_fwd_phases(ctypes.byref(a), mask, _stream())))
     return [out, lse, p, rng_state]
 
 

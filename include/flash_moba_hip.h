@@ -142,6 +142,12 @@ size_t fmoba_attn_fwd_workspace_bytes(int32_t total_q, int32_t heads, int32_t he
  * reference, whose row-wise scratch needs no bound. */
 int fmoba_csc_max_row_visits(const fmoba_attn_fwd_args *a, int32_t *counts, int32_t *max_out, void *stream);
 int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream);
+/* The same call split into its two launches so that each can be timed on its own: phases is a bit
+ * mask, 1 = the column pass (clears the visit counters first), 2 = the per-row combine.
+ * fmoba_attn_fwd(a, s) == fmoba_attn_fwd_phases(a, 3, s). */
+#define FMOBA_FWD_COLUMNS 1
+#define FMOBA_FWD_COMBINE 2
+int fmoba_attn_fwd_phases(const fmoba_attn_fwd_args *a, int32_t phases, void *stream);
 
 /* ------------------------------------------------------------------------------------
  * Sparse attention backward.
