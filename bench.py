@@ -155,6 +155,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="headline", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--fwd-mode", type=int, default=0, choices=(0, 1, 2),
+                    help="forward form of the per-stage timings: 0 = the library's choice (what the timed steps run), 1 = columns, 2 = row blocks")
     ap.add_argument("--calib-copy", action="store_true",
                     help="run one plain 1 GiB device copy first, so that a counter run has a kernel of known traffic to scale by")
     args = ap.parse_args()
@@ -202,7 +204,9 @@ def main():
 
     # ---- algorithmic work -------------------------------------------------------------
     with torch.no_grad():
+        hip.keep_next_gate_selection()  # as flash_moba_varlen_func does: the forward may use the gating's selection bits
         co, cn, ind = flash_moba.flash_topk_varlen_func(q, k, cu, cu, max_len, max_len, topk, chunk, causal=True)
+        selection = hip.take_gate_selection()
     pairs = count_pairs(seqlens, cn, chunk, H)
     fwd_flops = 4.0 * D * pairs
     bwd_flops = 2.5 * fwd_flops
@@ -223,15 +227,18 @@ def main():
     visits = topk * (chunk // hip.fwd_key_block(chunk))  # the bound the gated path hands to the forward
 
     def fwd(**kw):
-        hip.set_visits_hint(visits)
+        hip.set_visits_hint(visits, selection=selection)
         return hip.moba_varlen_fwd(qd, kd, vd, None, co, cn, ind, cu, cu, None, None, None, max_len, max_len, 0.0, scale,
-                                   False, True, 0.0, False, lg_m, chunk, None, **kw)
+                                   False, True, 0.0, False, lg_m, chunk, None, _fwd_mode=args.fwd_mode, **kw)
 
     fwd_phase_ms = {}
+    fwd()
+    row_blocks = bool(hip.last_fwd_row_blocks())  # which of the two forward forms the library picks for this shape
+    fwd_names = ("selection_bits", "row_blocks") if row_blocks else ("columns", "combine")
 
     def run_fwd_phases(run):
         run(3)
-        for name, mask in (("columns", 1), ("combine", 2)):
+        for name, mask in zip(fwd_names, (1, 2)):
             fwd_phase_ms[name] = time_events(lambda: run(mask), it)
 
     fwd(_phases=run_fwd_phases)
@@ -244,8 +251,11 @@ def main():
         "attn_fwd": {"ms": t_fwd, "TFLOPs": fwd_flops / t_fwd / 1e9, "frac_mfma": fwd_flops / t_fwd / 1e9 / PEAK_BF16_TFLOPS,
                      "phases_ms": fwd_phase_ms},
     }
-    # the column pass runs both forward GEMMs; the combine only merges partial rows
-    kernels = {"attn_fwd_col_kernel": (fwd_phase_ms["columns"], fwd_flops, "mfma")}
+    # one kernel runs both forward GEMMs: the row-block pass, or the column pass (its combine only merges partial rows)
+    if row_blocks:
+        kernels = {"attn_fwd_rows_kernel": (fwd_phase_ms["row_blocks"], fwd_flops, "mfma")}
+    else:
+        kernels = {"attn_fwd_col_kernel": (fwd_phase_ms["columns"], fwd_flops, "mfma")}
     if backward:
         dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
         phase_ms = {}

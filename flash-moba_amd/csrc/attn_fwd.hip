@@ -21,12 +21,14 @@
 // (global -> registers -> LDS), two rounds ahead.
 #include "fmoba_common.h"
 
+#include <algorithm>
 #include <type_traits>
 #include <utility>
 
 namespace fmoba {
 
 constexpr int kFwdListCap = 4096;  // rows of a column list held in LDS at a time
+constexpr int kFwdRowsDensity = 6;  // row-block form when a row selects at least 1/6 of the chunks it may see
 
 // NCW compute waves (one 32-row tile each per round) + 2 loader waves
 template <int HD, int KB, int NCW>
@@ -477,6 +479,24 @@ __global__ __launch_bounds__(256) void max_i32_kernel(const int32_t *p, int64_t 
 static inline size_t fwd_align256(size_t x) { return (x + 255) & ~(size_t)255; }
 static inline int fwd_key_block(int lg_block_n) { return lg_block_n % 128 == 0 ? 128 : 64; }
 
+// the row-block form (attn_fwd_rows.hip)
+bool fwd_rows_feasible(const fmoba_attn_fwd_args &a);
+size_t fwd_rows_workspace_bytes(const fmoba_attn_fwd_args &a);
+int run_fwd_rows(const fmoba_attn_fwd_args &a, int phases, hipStream_t s);
+
+// Which form runs.  The row-block form multiplies every row of a 128-row block with every chunk that
+// any of its rows selected, the column form only the selected pairs but pays a partial result per
+// visit: the first wins while a row selects more than about a sixth of the chunks it may see.
+static bool fwd_use_rows(const fmoba_attn_fwd_args &a) {
+  if (a.fwd_mode == 1) return false;
+  if (!fwd_rows_feasible(a)) return false;
+  if (a.fwd_mode == 2) return true;
+  const int64_t chunks_per_seq = std::max<int64_t>(1, ceil_div64(ceil_div64(std::max(a.total_k, 1), a.batch), a.lg_block_n));
+  const int64_t chunks_per_row = std::max<int64_t>(1, (int64_t)a.max_visits_per_row * fwd_key_block(a.lg_block_n) / a.lg_block_n);
+  const int64_t seen = a.is_causal ? (chunks_per_seq + 1) / 2 : chunks_per_seq;
+  return chunks_per_row * kFwdRowsDensity >= seen;
+}
+
 template <typename T, int HD, int KB>
 static int launch_fwd_col(const fmoba_attn_fwd_args &a, const FwdWs &ws, hipStream_t s) {
   // 64-key blocks leave room (registers, LDS) for four compute waves; 128-key blocks for two
@@ -513,11 +533,24 @@ static int run_fwd(const fmoba_attn_fwd_args &a, const FwdWs &ws, int phases, hi
 
 extern "C" int32_t fmoba_attn_fwd_key_block(int32_t lg_block_n) { return fmoba::fwd_key_block(lg_block_n); }
 
-extern "C" size_t fmoba_attn_fwd_workspace_bytes(int32_t total_q, int32_t heads, int32_t head_dim, int32_t max_visits_per_row) {
+static size_t fwd_cols_workspace_bytes(int32_t total_q, int32_t heads, int32_t head_dim, int32_t max_visits_per_row) {
   using namespace fmoba;
   if (total_q <= 0 || heads <= 0 || head_dim <= 0 || max_visits_per_row <= 0) return 256;
   const size_t rows = (size_t)total_q * heads;
   return fwd_align256((rows + 1) * 4) + fwd_align256(rows * max_visits_per_row * 16) + fwd_align256(rows * max_visits_per_row * head_dim * 2) + 256;
+}
+
+extern "C" size_t fmoba_attn_fwd_workspace_bytes(const fmoba_attn_fwd_args *a) {
+  using namespace fmoba;
+  if (a == nullptr || a->total_q <= 0 || a->heads <= 0 || a->head_dim <= 0 || a->batch <= 0 || a->lg_block_n <= 0) return 256;
+  if (fwd_use_rows(*a)) return fwd_rows_workspace_bytes(*a);
+  return fwd_cols_workspace_bytes(a->total_q, a->heads, a->head_dim, a->max_visits_per_row);
+}
+
+extern "C" int32_t fmoba_attn_fwd_uses_row_blocks(const fmoba_attn_fwd_args *a) {
+  using namespace fmoba;
+  if (a == nullptr || a->total_q <= 0 || a->heads <= 0 || a->head_dim <= 0 || a->batch <= 0 || a->lg_block_n <= 0) return 0;
+  return fwd_use_rows(*a) ? 1 : 0;
 }
 
 static int fwd_check_common(const fmoba_attn_fwd_args *a) {
@@ -580,8 +613,16 @@ extern "C" int fmoba_attn_fwd_phases(const fmoba_attn_fwd_args *a, int32_t phase
   FMOBA_REQUIRE(((uintptr_t)a->q % 16) == 0 && ((uintptr_t)a->k % 16) == 0 && ((uintptr_t)a->v % 16) == 0 && ((uintptr_t)a->out % 16) == 0,
                 "attn_fwd: q, k, v and out must be 16-byte aligned");
   FMOBA_REQUIRE(a->max_visits_per_row > 0, "attn_fwd: max_visits_per_row must be positive");
-  const size_t need = fmoba_attn_fwd_workspace_bytes(a->total_q, a->heads, a->head_dim, a->max_visits_per_row);
+  FMOBA_REQUIRE(a->fwd_mode >= 0 && a->fwd_mode <= 2, "attn_fwd: fwd_mode must be 0 (automatic), 1 (columns) or 2 (row blocks)");
+  FMOBA_REQUIRE(a->fwd_mode != 2 || fwd_rows_feasible(*a), "attn_fwd: the row-block form does not take this shape (more than %d chunks or %d keys per sequence)",
+                32 * 128, 64 * 4096);
+  const size_t need = fmoba_attn_fwd_workspace_bytes(a);
   FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, "attn_fwd: workspace too small (%zu < %zu)", a->workspace_bytes, need);
+  if (fwd_use_rows(*a)) {
+    if (int rc = run_fwd_rows(*a, phases, s)) return rc;
+    FMOBA_LAUNCH_CHECK("attn_fwd");
+    return 0;
+  }
   const size_t rows = (size_t)a->total_q * a->heads;
   uintptr_t p = ((uintptr_t)a->workspace + 255) & ~(uintptr_t)255;
   FwdWs ws;

@@ -52,12 +52,12 @@ class FusedTopkArgs(ctypes.Structure):
 class AttnFwdArgs(ctypes.Structure):
     _fields_ = [("q", c_vp), ("k", c_vp), ("v", c_vp), ("out", c_vp), ("softmax_lse", c_vp),
                 ("col_offsets", c_vp), ("col_nnz", c_vp), ("row_indices", c_vp),
-                ("cu_seqlens_q", c_vp), ("cu_seqlens_k", c_vp),
+                ("cu_seqlens_q", c_vp), ("cu_seqlens_k", c_vp), ("selection_bits", c_vp),
                 ("workspace", c_vp), ("workspace_bytes", c_sz),
                 ("batch", c_i32), ("total_q", c_i32), ("total_k", c_i32), ("heads", c_i32), ("heads_k", c_i32),
                 ("head_dim", c_i32), ("max_seqlen_q", c_i32), ("max_seqlen_k", c_i32), ("max_cols", c_i32),
                 ("lg_block_m", c_i32), ("lg_block_n", c_i32), ("is_causal", c_i32), ("dtype", c_i32),
-                ("max_visits_per_row", c_i32), ("softmax_scale", c_f32),
+                ("max_visits_per_row", c_i32), ("fwd_mode", c_i32), ("softmax_scale", c_f32),
                 ("q_row_stride", c_i64), ("q_head_stride", c_i64), ("k_row_stride", c_i64), ("k_head_stride", c_i64),
                 ("v_row_stride", c_i64), ("v_head_stride", c_i64), ("o_row_stride", c_i64), ("o_head_stride", c_i64)]
 
@@ -89,7 +89,8 @@ EXPORTS = {
     "fmoba_varlen_sort_workspace_bytes": (c_sz, [c_i64]),
     "fmoba_varlen_sort": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_sz, c_vp]),
     "fmoba_attn_fwd_key_block": (c_i32, [c_i32]),
-    "fmoba_attn_fwd_workspace_bytes": (c_sz, [c_i32, c_i32, c_i32, c_i32]),
+    "fmoba_attn_fwd_workspace_bytes": (c_sz, [ctypes.POINTER(AttnFwdArgs)]),
+    "fmoba_attn_fwd_uses_row_blocks": (c_i32, [ctypes.POINTER(AttnFwdArgs)]),
     "fmoba_csc_max_row_visits": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp, c_vp, c_vp]),
     "fmoba_attn_fwd": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_vp]),
     "fmoba_attn_fwd_phases": (c_i32, [ctypes.POINTER(AttnFwdArgs), c_i32, c_vp]),
@@ -231,6 +232,10 @@ def moba_fused_topk(q: torch.Tensor, km: torch.Tensor, cu_seqlens_q: torch.Tenso
                           int(moba_topk), int(moba_chunk_size), int(bool(is_causal)), _dt(q),
                           q.stride(0), q.stride(1), km.stride(0), km.stride(1))
         _check(lib.fmoba_fused_topk(ctypes.byref(a), _stream()))
+        if getattr(_hint, "keep_selection", False):
+            # the selection bits sit at the first 256-byte boundary of the workspace: (heads, ceil(max_cols/32), total_q) words
+            _hint.keep_selection = False
+            _hint.selection = (ws, heads, (max_cols + 31) // 32, total_q)
     return [col_offsets, col_nnz, flat, values, indices]
 
 
@@ -292,9 +297,25 @@ def _reject_unsupported(p_dropout, softcap, alibi_slopes, seqused_k=None, leftpa
 _hint = threading.local()
 
 
-def set_visits_hint(n):
-    """Bound (in forward key blocks) for the next forward call of this thread."""
+def set_visits_hint(n, selection=None):
+    """Bound (in forward key blocks) for the next forward call of this thread, and optionally the
+    selection bits of the gating call that produced its pattern (take_gate_selection())."""
     _hint.value = None if n is None else int(n)
+    _hint.fwd_selection = selection
+
+
+def keep_next_gate_selection():
+    """The next gating call of this thread keeps its workspace, whose head is the selection as one bit
+    per (row, head, chunk); take_gate_selection() hands it over once."""
+    _hint.keep_selection = True
+    _hint.selection = None
+
+
+def take_gate_selection():
+    sel = getattr(_hint, "selection", None)
+    _hint.selection = None
+    _hint.keep_selection = False
+    return sel
 
 
 def set_bwd_visits_hint(n):
@@ -315,11 +336,16 @@ def _count_visits(lib, q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_s
     counts = torch.empty((total_q * heads + 1,), dtype=torch.int32, device=q.device)
     a0 = AttnFwdArgs(None, None, None, None, None,
                      moba_col_offsets.data_ptr(), moba_col_nnz.data_ptr(), moba_row_indices.data_ptr(),
-                     cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), None, 0,
+                     cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), None, None, 0,
                      batch, total_q, total_k, heads, heads_k, d, int(max_seqlen_q), int(max_seqlen_k), max_cols,
-                     int(m_lg_block_dim), int(n_lg_block_dim), 0, _dt(q), 0, 1.0, 0, 0, 0, 0, 0, 0, 0, 0)
+                     int(m_lg_block_dim), int(n_lg_block_dim), 0, _dt(q), 0, 0, 1.0, 0, 0, 0, 0, 0, 0, 0, 0)
     _check(lib.fmoba_csc_max_row_visits(ctypes.byref(a0), counts.data_ptr(), counts[total_q * heads:].data_ptr(), _stream()))
     return max(1, int(counts[total_q * heads].item()))
+
+
+def last_fwd_row_blocks():
+    """1 if the last forward of this thread ran the row-block form, 0 for the column form."""
+    return int(getattr(_hint, "last_form", 0))
 
 
 def fwd_key_block(n_lg_block_dim):
@@ -328,7 +354,8 @@ def fwd_key_block(n_lg_block_dim):
 
 def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k,
                     seqused_k, leftpad_k, alibi_slopes, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-                    zero_tensors, is_causal, softcap, return_softmax, m_lg_block_dim, n_lg_block_dim, gen=None, _phases=None):
+                    zero_tensors, is_causal, softcap, return_softmax, m_lg_block_dim, n_lg_block_dim, gen=None, _phases=None,
+                    _fwd_mode=0):
     """Returns [out, softmax_lse (H, total_q) fp32, p (empty), rng_state (2,) int64]."""
     dtype = q.dtype
     _require(dtype in (torch.float16, torch.bfloat16), "FlashMoBA only support fp16 and bf16 data type")
@@ -371,14 +398,19 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
         lib = load_library()
         hint = getattr(_hint, "value", None)
         _hint.value = None
+        sel = getattr(_hint, "fwd_selection", None)
+        _hint.fwd_selection = None
+        sel_ptr = None
+        if sel is not None and sel[1:] == (heads, (max_cols + 31) // 32, total_q) and sel[0].device == q.device:
+            sel_ptr = (sel[0].data_ptr() + 255) & ~255
 
         def args(ws_ptr, ws_bytes, visits):
             return AttnFwdArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
                                moba_col_offsets.data_ptr(), moba_col_nnz.data_ptr(), moba_row_indices.data_ptr(),
-                               cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), ws_ptr, ws_bytes,
+                               cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), sel_ptr, ws_ptr, ws_bytes,
                                batch, total_q, total_k, heads, heads_k, d, int(max_seqlen_q), int(max_seqlen_k), max_cols,
                                int(m_lg_block_dim), int(n_lg_block_dim), int(bool(is_causal)), _dt(q), visits,
-                               float(softmax_scale),
+                               int(_fwd_mode), float(softmax_scale),
                                q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                                out.stride(0), out.stride(1))
 
@@ -389,7 +421,9 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
                                    m_lg_block_dim, n_lg_block_dim)
         visits = max(1, int(visits))
         _hint.last = visits
-        ws_bytes = lib.fmoba_attn_fwd_workspace_bytes(total_q, heads, d, visits)
+        a = args(None, 0, visits)
+        ws_bytes = lib.fmoba_attn_fwd_workspace_bytes(ctypes.byref(a))
+        _hint.last_form = int(lib.fmoba_attn_fwd_uses_row_blocks(ctypes.byref(a)))
         ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=q.device)
         a = args(ws.data_ptr(), ws_bytes, visits)
         if _phases is None:

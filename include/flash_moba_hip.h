@@ -108,7 +108,10 @@ int fmoba_varlen_sort(const int64_t *seg_starts, const int64_t *seg_ends, int64_
  * Replaces moba_varlen_fwd (csrc/flash_moba/flash_moba_api.cpp:375-596).
  *   out (total_q, heads, head_dim) dtype, softmax_lse (heads, total_q) fp32.
  * Rows that see no key get out = 0, lse = +inf.
- * The forward is column-stationary: every visit of a (query row, key block) pair leaves a
+ * Two forms.  Row blocks (patterns in which a row selects a good part of the chunks it may see):
+ * one workgroup per 128 query rows walks every chunk any of its rows selected, with the running
+ * softmax state in registers; `workspace` then holds one selection bit per (row, head, chunk).
+ * Columns (sparser patterns): every visit of a (query row, key block) pair leaves a
  * partial result in `workspace`, and a second launch merges the partials of each row.  A key
  * block is fmoba_attn_fwd_key_block(lg_block_n) keys (128 if lg_block_n is a multiple of 128,
  * else 64).  max_visits_per_row bounds the number of visits of any (row, head): for a pattern
@@ -124,6 +127,11 @@ typedef struct {
   const int32_t *col_nnz;       /* (batch, heads, max_cols) */
   const int32_t *row_indices;   /* flat row lists */
   const int32_t *cu_seqlens_q, *cu_seqlens_k;
+  /* optional (may be NULL): the same pattern as one bit per (row, head, chunk), word
+   * [(h * ceil(max_cols/32) + c/32) * total_q + global row] bit c%32 -- what fmoba_fused_topk leaves
+   * at the first 256-byte boundary of its workspace.  Only the row-block form reads it; without it
+   * that form derives the bits from the lists first. */
+  const uint32_t *selection_bits;
   void *workspace;
   size_t workspace_bytes;
   int32_t batch, total_q, total_k, heads, heads_k, head_dim;
@@ -131,19 +139,24 @@ typedef struct {
   int32_t lg_block_m, lg_block_n;
   int32_t is_causal, dtype;
   int32_t max_visits_per_row;
+  int32_t fwd_mode;             /* 0 = the library chooses, 1 = column form, 2 = row-block form */
   float softmax_scale;
   int64_t q_row_stride, q_head_stride, k_row_stride, k_head_stride;
   int64_t v_row_stride, v_head_stride, o_row_stride, o_head_stride;
 } fmoba_attn_fwd_args;
 int32_t fmoba_attn_fwd_key_block(int32_t lg_block_n);
-size_t fmoba_attn_fwd_workspace_bytes(int32_t total_q, int32_t heads, int32_t head_dim, int32_t max_visits_per_row);
+/* Bytes of workspace for the call described by `a` (sizes, max_visits_per_row and fwd_mode are read,
+ * pointers are not), and which form it will run (1 = row blocks, 0 = columns). */
+size_t fmoba_attn_fwd_workspace_bytes(const fmoba_attn_fwd_args *a);
+int32_t fmoba_attn_fwd_uses_row_blocks(const fmoba_attn_fwd_args *a);
 /* counts (total_q * heads) int32 and max_out (1) int32 are device outputs: visits per (row, head) and
  * their maximum for the pattern in `a` (q/k/v/out/workspace of `a` are not read).  No counterpart in the
  * reference, whose row-wise scratch needs no bound. */
 int fmoba_csc_max_row_visits(const fmoba_attn_fwd_args *a, int32_t *counts, int32_t *max_out, void *stream);
 int fmoba_attn_fwd(const fmoba_attn_fwd_args *a, void *stream);
 /* The same call split into its two launches so that each can be timed on its own: phases is a bit
- * mask, 1 = the column pass (clears the visit counters first), 2 = the per-row combine.
+ * mask, 1 = the column pass (clears the visit counters first), 2 = the per-row combine; in the
+ * row-block form 1 = building the selection bits, 2 = the attention pass.
  * fmoba_attn_fwd(a, s) == fmoba_attn_fwd_phases(a, 3, s). */
 #define FMOBA_FWD_COLUMNS 1
 #define FMOBA_FWD_COMBINE 2

@@ -346,6 +346,63 @@ def test_attention_random_pattern(fm, sq, sk, d, mha, causal, dtype):
     _check_attention(fm, q, k, v, dout, cuq, cuk, co, cn, ind, 64, causal)
 
 
+@pytest.mark.parametrize("form", [1, 2])
+@pytest.mark.parametrize("sq,sk,d,Hk,chunk,topk,causal,dtype", [
+    (300, 300, 128, 4, 64, 3, True, torch.bfloat16),
+    (1023, 1024, 128, 4, 64, 6, True, torch.bfloat16),
+    (513, 700, 64, 2, 64, 4, True, torch.bfloat16),      # len_k > len_q, GQA
+    (700, 513, 96, 1, 64, 4, True, torch.float16),       # len_q > len_k: leading rows see nothing; MQA; padded head dim
+    (384, 640, 128, 4, 128, 2, True, torch.bfloat16),    # 128-key chunks: two 64-key steps per chunk
+    (257, 390, 128, 4, 64, 3, False, torch.bfloat16),    # non-causal
+    (129, 1, 64, 4, 64, 1, False, torch.float16),
+])
+def test_forward_both_forms(fm, form, sq, sk, d, Hk, chunk, topk, causal, dtype):
+    # the library picks the forward form (columns / row blocks) by the density of the pattern; both are
+    # checked here whatever it would pick
+    H = 4
+    rng = np.random.RandomState(sq * 7 + sk)
+    lens_q = [max(1, sq - int(x)) for x in rng.randint(0, 150, 3)]
+    lens_k = [max(1, sk - int(x)) for x in rng.randint(0, 150, 3)] if sk > 1 else [1, 1, 1]
+    q, k, v, dout, cuq, cuk = _attn_inputs(5, lens_q, lens_k, H, Hk, d, dtype)
+    co, cn, ind = _random_csc(2, lens_q, lens_k, H, chunk, topk, causal)
+    scale = d ** -0.5
+    dp = (8 - d % 8) % 8
+    pad = (lambda t: torch.nn.functional.pad(t, (0, dp))) if dp else (lambda t: t)
+    out, lse, _, _ = fm.hip.moba_varlen_fwd(pad(q).cuda(), pad(k).cuda(), pad(v).cuda(), None, co.cuda(), cn.cuda(), ind.cuda(),
+                                            cuq.cuda(), cuk.cuda(), None, None, None, max(lens_q), max(lens_k), 0.0, scale,
+                                            False, causal, 0.0, False, 128, chunk, None, _fwd_mode=form)
+    o_ref, lse_ref, _, _, _ = O.attn_fwd_bwd(q, k, v, dout, cuq, cuk, co, cn, ind, chunk, scale, causal)
+    assert_close("out", out[..., :d], o_ref, 2e-2, 1e-2)
+    fin = torch.isfinite(lse_ref)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    assert (lse.cpu()[~fin] == float("inf")).all()
+    assert_close("lse", lse.cpu()[fin], lse_ref[fin], 2e-2, 1e-2)
+    out2, lse2, _, _ = fm.hip.moba_varlen_fwd(pad(q).cuda(), pad(k).cuda(), pad(v).cuda(), None, co.cuda(), cn.cuda(), ind.cuda(),
+                                              cuq.cuda(), cuk.cuda(), None, None, None, max(lens_q), max(lens_k), 0.0, scale,
+                                              False, causal, 0.0, False, 128, chunk, None, _fwd_mode=form)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+
+
+@pytest.mark.parametrize("lens,chunk,topk,Hk", [([640, 1, 0, 1300], 64, 6, 4), ([2100, 900], 128, 5, 2), ([300 * 64 + 17], 64, 33, 1)])
+def test_fused_path_hands_the_gating_selection_to_the_forward(fm, lens, chunk, topk, Hk):
+    # flash_moba_varlen_func passes the gating's selection bits on; the attention entry point alone derives them from
+    # the lists: same bits, same result
+    H, D = 4, 128
+    g = torch.Generator().manual_seed(9)
+    T = sum(lens)
+    q = torch.randn((T, H, D), generator=g).to(torch.bfloat16).cuda()
+    k = torch.randn((T, Hk, D), generator=g).to(torch.bfloat16).cuda()
+    v = torch.randn((T, Hk, D), generator=g).to(torch.bfloat16).cuda()
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32).cuda()
+    out = fm.api.flash_moba_varlen_func(q, k, v, cu, cu, max(lens), max(lens), chunk, topk, causal=True)
+    assert fm.hip.last_fwd_row_blocks() == 1
+    co, cn, ind = fm.api.flash_topk_varlen_func(q, k, cu, cu, max(lens), max(lens), topk, chunk, causal=True)
+    lg_m = fm.iface.decide_lg_block_m(topk, chunk, max(lens), True)
+    out2 = fm.api.flash_moba_attn_varlen_func(q, k, v, cu, cu, max(lens), max(lens), co, cn, ind, lg_m, chunk, causal=True)
+    assert fm.hip.last_fwd_row_blocks() == 1
+    assert torch.equal(out, out2)
+
+
 @pytest.mark.parametrize("dq_mode", [1, 2])
 @pytest.mark.parametrize("d,chunk", [(128, 64), (64, 128), (96, 64)])
 def test_backward_both_dq_forms(fm, dq_mode, d, chunk):

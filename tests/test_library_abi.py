@@ -48,7 +48,21 @@ def test_workspace_queries_are_pure_host_functions():
     assert lib.fmoba_attn_bwd_workspace_bytes(ctypes.byref(a)) >= 1024 * 4 * 8 * 128 * 2
     a.dq_mode = 1
     assert lib.fmoba_attn_bwd_workspace_bytes(ctypes.byref(a)) >= 32768 * 64 * 2
-    assert lib.fmoba_attn_fwd_workspace_bytes(1024, 4, 128, 8) >= 1024 * 4 * 8 * (128 * 2 + 16)
+    f = H.AttnFwdArgs()
+    f.total_q, f.heads, f.heads_k, f.head_dim, f.batch, f.total_k, f.lg_block_n, f.max_visits_per_row = 1024, 4, 4, 128, 1, 1024, 64, 8
+    f.max_seqlen_q = f.max_seqlen_k = 1024
+    f.max_cols, f.is_causal = 16, 1
+    f.fwd_mode = 1  # columns: one partial row + header per visit
+    assert lib.fmoba_attn_fwd_uses_row_blocks(ctypes.byref(f)) == 0
+    assert lib.fmoba_attn_fwd_workspace_bytes(ctypes.byref(f)) >= 1024 * 4 * 8 * (128 * 2 + 16)
+    f.fwd_mode = 2  # row blocks: one selection bit per (row, head, chunk)
+    assert lib.fmoba_attn_fwd_uses_row_blocks(ctypes.byref(f)) == 1
+    assert 1024 * 4 * 4 <= lib.fmoba_attn_fwd_workspace_bytes(ctypes.byref(f)) < 1024 * 4 * 4 + 1024
+    f.fwd_mode = 0  # 8 of at most 16 chunks per row: dense enough for row blocks
+    assert lib.fmoba_attn_fwd_uses_row_blocks(ctypes.byref(f)) == 1
+    f.total_k = f.max_seqlen_k = 1 << 20  # 16384 chunks: columns
+    f.max_cols = 16384
+    assert lib.fmoba_attn_fwd_uses_row_blocks(ctypes.byref(f)) == 0
     assert lib.fmoba_attn_fwd_key_block(64) == 64 and lib.fmoba_attn_fwd_key_block(128) == 128 and lib.fmoba_attn_fwd_key_block(192) == 64
 
 
