@@ -567,7 +567,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 }
 
 // ------------------------------------------------------------------------------------
-// dQ: row-stationary
+// dQ, first form: row blocks.  One workgroup owns 128 consecutive query rows of one (sequence, head) and walks the
+// 64-key blocks of every column in which one of its rows appears.  The dS rows of a step (written by the dK/dV
+// pass in list order) are put at the place of their query row in LDS, rows that are absent keep a stale tag and
+// contribute zeros, so every compute wave multiplies its own 32 rows and keeps dQ in registers for the whole walk.
 // ------------------------------------------------------------------------------------
 constexpr int kDqRows = 128;
 constexpr int kDqColBatch = 256;
@@ -576,19 +579,19 @@ constexpr int kDqMaxSteps = 512;
 template <int HD>
 struct DqSmem {
   static constexpr int LDQ = HD + 16;  // elements, K tile
-  static constexpr int LDA = HD + 4;   // floats, dQ accumulators
   static constexpr int LDD = 64 + 8;   // elements, dS rows [128][64 keys]
-  static constexpr size_t oA = 0;
-  static constexpr size_t oK = oA + (size_t)kDqRows * LDA * 4;     // [2][64][LDQ]
+  static constexpr int LDO = HD + 8;   // elements, per-wave output tile [32 rows][LDO] (reuses the K tiles at the end)
+  static constexpr size_t oK = 0;                                   // [2][64][LDQ]
   static constexpr size_t oD = oK + (size_t)2 * 64 * LDQ * 2;      // [2][128][LDD]
-  static constexpr size_t oRows = oD + (size_t)2 * kDqRows * LDD * 2;  // int[2][128]
-  static constexpr size_t oLo = oRows + 2 * kDqRows * 4;
+  static constexpr size_t oTag = oD + (size_t)2 * kDqRows * LDD * 2;  // int[2][128]: step that last wrote the row
+  static constexpr size_t oLo = oTag + 2 * kDqRows * 4;
   static constexpr size_t oCnt = oLo + kDqColBatch * 4;
   static constexpr size_t oStep = oCnt + kDqColBatch * 4;
   static constexpr size_t oOff = oStep + kDqMaxSteps * 4;          // int64[kDqColBatch]
   static constexpr size_t oInfo = oOff + kDqColBatch * 8;          // int4[kDqMaxSteps]: key0, rows, list position (lo, hi)
   static constexpr size_t oMisc = oInfo + kDqMaxSteps * 16;
   static constexpr size_t bytes = oMisc + 64;
+  static_assert((size_t)4 * 32 * LDO * 2 <= (size_t)2 * 64 * LDQ * 2, "output tiles must fit the K tiles");
 };
 
 struct DqItem {
@@ -608,14 +611,13 @@ __device__ __forceinline__ DqItem dq_decode_item(int id, int npairs, int nsb_max
 template <typename T, int HD>
 __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a, const uint16_t *ds_ws, int nsb_max) {
   typedef DqSmem<HD> SM;
-  constexpr int LDQ = SM::LDQ, LDA = SM::LDA, LDD = SM::LDD, NDT = HD / 32, VPR = HD / 8;
+  constexpr int LDQ = SM::LDQ, LDD = SM::LDD, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
   constexpr int KVV = 64 * VPR / 256;  // K-tile vectors per loader thread
   constexpr int DVV = kDqRows * 8 / 256;  // dS-row vectors (64 keys = 8 vectors per row) per loader thread
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float *sA = reinterpret_cast<float *>(smem + SM::oA);
   uint16_t *sK = reinterpret_cast<uint16_t *>(smem + SM::oK);
   uint16_t *sD = reinterpret_cast<uint16_t *>(smem + SM::oD);
-  int *sRows = reinterpret_cast<int *>(smem + SM::oRows);
+  int *sTag = reinterpret_cast<int *>(smem + SM::oTag);
   int *sLo = reinterpret_cast<int *>(smem + SM::oLo);
   int *sCnt = reinterpret_cast<int *>(smem + SM::oCnt);
   int *sStep = reinterpret_cast<int *>(smem + SM::oStep);
@@ -640,7 +642,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
   const int ltid = tid & 255;
   const bool causal = a.is_causal != 0;
 
-  for (int v = tid; v < kDqRows * LDA; v += 512) sA[v] = 0.f;
+  for (int v = tid; v < 2 * kDqRows; v += 512) sTag[v] = 0;  // step tags start at 1
 
   int ncols = min((Lk + Bn - 1) / Bn, a.max_cols);
   const int last_rowpos = m0 + rows_sb - 1 + off;
@@ -650,12 +652,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
   const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + (int64_t)k0 * a.k_row_stride + (int64_t)hk * a.k_head_stride;
   const int cols_per_batch = min(kDqColBatch, kDqMaxSteps / nsub);
 
-  // loader rings, four steps deep: the dS rows come from HBM (about 2 us under load), a step takes well under 1 us
-  Pack8 pk[4][KVV], pd[4][DVV];
-  int prow[4] = {0, 0, 0, 0};
-
-  for (int cb = 0; cb < ncols; cb += cols_per_batch) {
-    const int cend = min(ncols, cb + cols_per_batch);
+  // The steps of one batch of columns: for every column the part of its list that falls into this row block, then
+  // one record per (column, 64-key block) that has rows and visible keys.  Both roles run it (same barriers).
+  auto prepare_batch = [&](int cb, int cend) {
     __syncthreads();
     for (int c = cb + tid; c < cend; c += 512) {
       const int nnz = a.col_nnz[bh * a.max_cols + c];
@@ -691,8 +690,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
     }
     __syncthreads();
     const int nsteps = sMisc[0];
-    if (nsteps == 0) continue;
-
     // one record per step, so that a loader needs a single LDS read before it can issue its loads
     for (int st = tid; st < nsteps; st += 512) {
       const int code = sStep[st];
@@ -701,106 +698,104 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
       sInfo[st] = make_int4((cb + cl) * Bn + kb * 64, sCnt[cl], (int)(uint32_t)(pos0 & 0xffffffffll), (int)(pos0 >> 32));
     }
     __syncthreads();
+    return nsteps;
+  };
 
-    // Loads are unconditional (indices clamped into the valid range, the surplus zeroed when it is stored):
-    // without branches around them the compiler counts outstanding loads exactly, so storing one ring
-    // entry does not wait for the loads of the next one.
-    auto load_step = [&](auto par, int step) {
-      constexpr int P = decltype(par)::value;
-      const int4 info = sInfo[min(step, nsteps - 1)];  // past the end: a redundant load, never stored
-      const int key0 = info.x, n = info.y;
-      const int64_t pos0 = (int64_t)(uint32_t)info.z | ((int64_t)info.w << 32);
-      const int koff = key0 - (key0 / Bn) * Bn;  // offset of the 64-key block inside its column
+  typedef std::integral_constant<int, 0> P0;
+  typedef std::integral_constant<int, 1> P1;
+  typedef std::integral_constant<int, 2> P2;
+  typedef std::integral_constant<int, 3> P3;
+  // LDS is double buffered by step parity: while the compute waves work on step s the loaders put
+  // step s+1 into the other buffer and then fetch step s+5 into the ring entry that this frees.
+  // The two roles run separate code with the same barrier sequence.  Every load_step is issued
+  // unconditionally and no control flow joins the loader path: the compiler sizes each wait by the
+  // smallest number of younger loads over all paths that reach it, and a path without loads (or one
+  // skipped load) would make every store wait for the whole ring.
+  if (is_loader) {
+    // loader rings, four steps deep: the dS rows come from HBM (about 2 us under load), a step takes well under 1 us
+    Pack8 pk[4][KVV], pd[4][DVV];
+    int prid[4][DVV];
+    int tag_base = 0;
+    // per-lane parts of the K-tile addresses: vector i of this thread is key ltid / VPR + i * (256 / VPR), features (ltid % VPR) * 8
+    uint32_t kvo[KVV];
 #pragma unroll
-      for (int i = 0; i < KVV; ++i) {
-        const int v = ltid + i * 256;
-        const int key = min(key0 + v / VPR, Lk - 1), e = min((v % VPR) * 8, D - 8);
-        const Pack8 x = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
-        pk[P][i] = x;
-      }
+    for (int i = 0; i < KVV; ++i) kvo[i] = (uint32_t)((ltid / VPR + i * (256 / VPR)) * (int)a.k_row_stride + min((ltid % VPR) * 8, D - 8));
+    const int klo = (ltid / VPR) * LDQ + (ltid % VPR) * 8;
+    for (int cb = 0; cb < ncols; cb += cols_per_batch) {
+      const int nsteps = prepare_batch(cb, min(ncols, cb + cols_per_batch));
+      if (nsteps == 0) continue;
+      // Loads are unconditional (indices clamped into the valid range, the surplus dropped when it is stored).
+      // Addresses are a uniform base (scalar registers) plus a 32-bit offset per lane that does not depend on
+      // the step: the loaders share their SIMDs with the compute waves, every instruction they issue is taken
+      // from those.
+      auto load_step = [&](auto par, int step) {
+        constexpr int P = decltype(par)::value;
+        const int4 info = sInfo[min(step, nsteps - 1)];  // past the end: a redundant load, never stored
+        const int key0 = __builtin_amdgcn_readfirstlane(info.x), n = __builtin_amdgcn_readfirstlane(info.y);
+        const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
+        const int koff = key0 - (key0 / Bn) * Bn;  // offset of the 64-key block inside its column
+        if (key0 + 64 <= Lk) {
+          const uint16_t *kb0 = kp + (int64_t)key0 * a.k_row_stride;
 #pragma unroll
-      for (int i = 0; i < DVV; ++i) {
-        const int v = ltid + i * 256;
-        const int row = min(v >> 3, n - 1), e = (v & 7) * 8;
-        const Pack8 x = ld_global16(ds_ws + (pos0 + row) * Bn + koff + e);
-        pd[P][i] = x;
-      }
-      prow[P] = a.row_indices[pos0 + min(ltid, n - 1)];
-    };
-    auto store_step = [&](auto par, int step) {
-      constexpr int P = decltype(par)::value;
-      const int buf = step & 1;
-      const int4 info = sInfo[step];
-      const int key0 = info.x, n = info.y;
+          for (int i = 0; i < KVV; ++i) pk[P][i] = ld_global16(kb0 + kvo[i]);
+        } else {
 #pragma unroll
-      for (int i = 0; i < KVV; ++i) {
-        const int v = ltid + i * 256;
-        const int key = v / VPR, e = (v - key * VPR) * 8;
-        const bool ok = key0 + key < Lk && e < D;
-        Pack8 x = pk[P][i];
-#pragma unroll
-        for (int w = 0; w < 4; ++w) x.w[w] = ok ? x.w[w] : 0u;
-        *reinterpret_cast<Pack8 *>(sK + ((size_t)buf * 64 + key) * LDQ + e) = x;
-      }
-#pragma unroll
-      for (int i = 0; i < DVV; ++i) {
-        const int v = ltid + i * 256;
-        const int row = v >> 3, e = (v & 7) * 8;
-        Pack8 x = pd[P][i];
-#pragma unroll
-        for (int w = 0; w < 4; ++w) x.w[w] = row < n ? x.w[w] : 0u;
-        *reinterpret_cast<Pack8 *>(sD + ((size_t)buf * kDqRows + row) * LDD + e) = x;
-      }
-      if (ltid < kDqRows) {
-        // the dK/dV pass wrote dS only for rows of this sequence that can see a key of the block
-        const int rr = prow[P];
-        const bool ok = ltid < n && rr >= m0 && rr < m0 + rows_sb && !(causal && rr + off < key0);
-        sRows[buf * kDqRows + ltid] = ok ? rr - m0 : -1;
-      }
-    };
-    auto compute_step = [&](int step) {
-      const int buf = step & 1;
-      const int n = sInfo[step].y;
-      const uint16_t *tK = sK + (size_t)buf * 64 * LDQ;
-      const int dt = wave % NDT;
-      for (int tile = wave / NDT; tile * 32 < n; tile += 4 / NDT) {
-        const int slot = tile * 32 + (lane & 31);
-        const int rid = sRows[buf * kDqRows + slot];
-        Pack8 df[4], kf[4];
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) {
-          df[s4] = *reinterpret_cast<const Pack8 *>(sD + ((size_t)buf * kDqRows + slot) * LDD + 16 * s4 + 8 * hh);
-          kf[s4] = tr_frag8(tK, LDQ, 16 * s4 + 8 * hh, 16 * s4 + 8 * hh + 4, dt * 32, lane);
-        }
-        f32x16 dq;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) dq[i] = 0.f;
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) dq = mfma32<T>(kf[s4], df[s4], dq);  // dQ^T[d][row] += K^T[d][key] dS^T[key][row]
-        if (rid >= 0 && rid < kDqRows) {
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            float *ap = sA + rid * LDA + dt * 32 + 8 * g + 4 * hh;
-            f32x4 old = *reinterpret_cast<f32x4 *>(ap);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) old[j] += dq[4 * g + j];
-            *reinterpret_cast<f32x4 *>(ap) = old;
+          for (int i = 0; i < KVV; ++i) {
+            const int v = ltid + i * 256;
+            const int key = min(key0 + v / VPR, Lk - 1), e = min((v % VPR) * 8, D - 8);
+            pk[P][i] = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
           }
         }
-      }
-    };
-
-    typedef std::integral_constant<int, 0> P0;
-    typedef std::integral_constant<int, 1> P1;
-    typedef std::integral_constant<int, 2> P2;
-    typedef std::integral_constant<int, 3> P3;
-    // LDS is double buffered by step parity: while the compute waves work on step s the loaders put
-    // step s+1 into the other buffer and then fetch step s+5 into the ring entry that this frees
-    // The two roles run separate loops with the same barrier sequence.  Every load_step is issued
-    // unconditionally and no control flow joins the loader path: the compiler sizes each wait by the
-    // smallest number of younger loads over all paths that reach it, and a path without loads (or one
-    // skipped load) would make every store wait for the whole ring.
-    if (is_loader) {
+        const uint16_t *db0 = ds_ws + pos0 * Bn + koff + (ltid & 7) * 8;
+        const int32_t *rb0 = a.row_indices + pos0;
+        // rows 32 i .. 32 i + 31 of the step's dS tile; a group past the last row is not fetched (the first always is:
+        // the waits the compiler places count the loads that every path issues)
+#pragma unroll
+        for (int i = 0; i < DVV; ++i) {
+          if (i == 0 || 32 * i < n) {
+            const uint32_t row = (uint32_t)min((ltid >> 3) + 32 * i, n - 1);
+            pd[P][i] = ld_global16(db0 + row * (uint32_t)Bn);
+            prid[P][i] = rb0[row];
+          }
+        }
+      };
+      auto store_step = [&](auto par, int step) {
+        constexpr int P = decltype(par)::value;
+        const int buf = step & 1;
+        const int4 info = sInfo[step];
+        const int key0 = __builtin_amdgcn_readfirstlane(info.x), n = __builtin_amdgcn_readfirstlane(info.y);
+        uint16_t *tK = sK + (size_t)buf * 64 * LDQ;
+        if (D == HD && key0 + 64 <= Lk) {
+#pragma unroll
+          for (int i = 0; i < KVV; ++i) *reinterpret_cast<Pack8 *>(tK + klo + i * (256 / VPR) * LDQ) = pk[P][i];
+        } else {
+#pragma unroll
+          for (int i = 0; i < KVV; ++i) {
+            const int v = ltid + i * 256;
+            const int key = v / VPR, e = (v - key * VPR) * 8;
+            const bool ok = key0 + key < Lk && e < D;
+            Pack8 x = pk[P][i];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) x.w[w] = ok ? x.w[w] : 0u;
+            *reinterpret_cast<Pack8 *>(tK + key * LDQ + e) = x;
+          }
+        }
+        // the dK/dV pass wrote dS only for rows of this sequence that can see a key of the block
+        const int first_rel = causal ? key0 - off - m0 : -0x40000000;  // rows before it see no key of the block
+        uint16_t *tD = sD + (size_t)buf * kDqRows * LDD + (ltid & 7) * 8;
+        int *tT = sTag + buf * kDqRows;
+        const int tag = tag_base + step + 1;
+#pragma unroll
+        for (int i = 0; i < DVV; ++i) {
+          if (32 * i >= n) break;
+          const int rel = prid[P][i] - m0;
+          const bool ok = (ltid >> 3) + 32 * i < n && (uint32_t)rel < (uint32_t)rows_sb && rel >= first_rel;
+          if (ok) {
+            *reinterpret_cast<Pack8 *>(tD + rel * LDD) = pd[P][i];
+            if ((ltid & 7) == 0) tT[rel] = tag;
+          }
+        }
+      };
       load_step(P0{}, 0);
       load_step(P1{}, 1);
       load_step(P2{}, 2);
@@ -819,27 +814,76 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
         loader_step(P3{}, step + 2);
         loader_step(P0{}, step + 3);
       }
-    } else {
+      tag_base += nsteps;
+    }
+    __syncthreads();  // the compute waves are done with the K tiles
+  } else {
+    // dQ^T of this wave's 32 rows: register i of feature tile dt <-> feature dt*32 + acc_row(i, hh), this lane's row
+    f32x16 acc[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
+    const int myrow = wave * 32 + (lane & 31);
+    int tag_base = 0;
+    for (int cb = 0; cb < ncols; cb += cols_per_batch) {
+      const int nsteps = prepare_batch(cb, min(ncols, cb + cols_per_batch));
+      if (nsteps == 0) continue;
       const int nsteps_pad = (nsteps + 3) & ~3;
       for (int step = 0; step < nsteps_pad; ++step) {
         __syncthreads();
-        if (step < nsteps) compute_step(step);
-      }
-    }
-  }
-  __syncthreads();
-
-  // dQ = scale * accumulator
-  {
-    uint16_t *op = reinterpret_cast<uint16_t *>(a.dq) + (int64_t)(q0 + m0) * a.dq_row_stride + (int64_t)h * a.dq_head_stride;
-    for (int v = tid; v < rows_sb * VPR; v += 512) {
-      const int row = v / VPR, e = (v - row * VPR) * 8;
-      if (e >= D) continue;
-      const float *src = sA + row * LDA + e;
-      Pack8 o;
+        if (step >= nsteps) continue;
+        const int buf = step & 1;
+        const bool present = sTag[buf * kDqRows + myrow] == tag_base + step + 1;
+        if (!__any(present)) continue;
+        // this lane's dS row as the B operand (zeros for a row that is not in the step)
+        Pack8 df[4];
 #pragma unroll
-      for (int w = 0; w < 4; ++w) o.w[w] = pack2<T>(src[2 * w] * a.softmax_scale, src[2 * w + 1] * a.softmax_scale);
-      *reinterpret_cast<Pack8 *>(op + (int64_t)row * a.dq_row_stride + e) = o;
+        for (int s4 = 0; s4 < 4; ++s4) {
+          df[s4] = *reinterpret_cast<const Pack8 *>(sD + ((size_t)buf * kDqRows + myrow) * LDD + 16 * s4 + 8 * hh);
+#pragma unroll
+          for (int w = 0; w < 4; ++w) df[s4].w[w] = present ? df[s4].w[w] : 0u;
+        }
+        lds_cu16 *trK = tr_lane_base(sK + (size_t)buf * 64 * LDQ, LDQ, lane) + 8 * hh * LDQ;
+        // K^T operands one feature tile ahead of the products that use them
+        Pack8 kf[2][4];
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) kf[0][s4] = tr_frag8_at(trK, 16 * s4 * LDQ, (16 * s4 + 4) * LDQ);
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+          if (dt + 1 < NDT) {
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4) kf[(dt + 1) & 1][s4] = tr_frag8_at(trK, 16 * s4 * LDQ + (dt + 1) * 32, (16 * s4 + 4) * LDQ + (dt + 1) * 32);
+          }
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4) acc[dt] = mfma32<T>(kf[dt & 1][s4], df[s4], acc[dt]);  // dQ^T[d][row] += K^T[d][key] dS^T[key][row]
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      tag_base += nsteps;
+    }
+    __syncthreads();  // every wave is done with the K tiles: they now hold the output tiles
+
+    // dQ = scale * accumulator, through a per-wave row-major tile
+    uint16_t *sOut = reinterpret_cast<uint16_t *>(smem + SM::oK) + (size_t)wave * 32 * LDO;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<uint2 *>(sOut + (lane & 31) * LDO + dt * 32 + 8 * g + 4 * hh) =
+            make_uint2(pack2<T>(acc[dt][4 * g] * a.softmax_scale, acc[dt][4 * g + 1] * a.softmax_scale),
+                       pack2<T>(acc[dt][4 * g + 2] * a.softmax_scale, acc[dt][4 * g + 3] * a.softmax_scale));
+    wave_lds_fence();
+    // rows leave as 16-byte pieces: lane -> (row 4k + lane / 16, features 8 * (lane % 16))
+    if ((lane & 15) * 8 < D) {
+      uint16_t *op = reinterpret_cast<uint16_t *>(a.dq) + (int64_t)(q0 + m0) * a.dq_row_stride + (int64_t)h * a.dq_head_stride;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int rl = 4 * k + (lane >> 4);
+        const int r2 = wave * 32 + rl;
+        if (r2 < rows_sb)
+          *reinterpret_cast<Pack8 *>(op + (int64_t)r2 * a.dq_row_stride + (lane & 15) * 8) = *reinterpret_cast<const Pack8 *>(sOut + rl * LDO + (lane & 15) * 8);
+      }
     }
   }
 }
