@@ -575,6 +575,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 constexpr int kDqRows = 128;
 constexpr int kDqColBatch = 256;
 constexpr int kDqMaxSteps = 512;
+constexpr int kDqRing = 4;  // steps the loaders run ahead: the dS rows come from HBM
 
 template <int HD>
 struct DqSmem {
@@ -702,19 +703,16 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
   };
 
   typedef std::integral_constant<int, 0> P0;
-  typedef std::integral_constant<int, 1> P1;
-  typedef std::integral_constant<int, 2> P2;
-  typedef std::integral_constant<int, 3> P3;
   // LDS is double buffered by step parity: while the compute waves work on step s the loaders put
-  // step s+1 into the other buffer and then fetch step s+5 into the ring entry that this frees.
+  // step s+1 into the other buffer and then fetch step s+1+kDqRing into the ring entry that this frees.
   // The two roles run separate code with the same barrier sequence.  Every load_step is issued
   // unconditionally and no control flow joins the loader path: the compiler sizes each wait by the
   // smallest number of younger loads over all paths that reach it, and a path without loads (or one
   // skipped load) would make every store wait for the whole ring.
   if (is_loader) {
-    // loader rings, four steps deep: the dS rows come from HBM (about 2 us under load), a step takes well under 1 us
-    Pack8 pk[4][KVV], pd[4][DVV];
-    int prid[4][DVV];
+    // loader rings: the dS rows come from HBM (about 2 us under load), a step takes well under 1 us
+    Pack8 pk[kDqRing][KVV], pd[kDqRing][DVV];
+    int prid[kDqRing][DVV];
     int tag_base = 0;
     // per-lane parts of the K-tile addresses: vector i of this thread is key ltid / VPR + i * (256 / VPR), features (ltid % VPR) * 8
     uint32_t kvo[KVV];
@@ -796,24 +794,17 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
           }
         }
       };
-      load_step(P0{}, 0);
-      load_step(P1{}, 1);
-      load_step(P2{}, 2);
-      load_step(P3{}, 3);
+      static_for<kDqRing>([&](auto e) { load_step(e, decltype(e)::value); });
       store_step(P0{}, 0);
-      load_step(P0{}, 4);
+      load_step(P0{}, kDqRing);
       auto loader_step = [&](auto par, int step) {  // par: ring entry of step + 1, stored during step
         __syncthreads();
         if (step + 1 < nsteps) store_step(par, step + 1);
-        load_step(par, step + 5);
+        load_step(par, step + 1 + kDqRing);
       };
-      // whole groups of four steps (the step count is padded with empty steps: barriers only)
-      for (int step = 0; step < nsteps; step += 4) {
-        loader_step(P1{}, step);
-        loader_step(P2{}, step + 1);
-        loader_step(P3{}, step + 2);
-        loader_step(P0{}, step + 3);
-      }
+      // whole turns of the ring (the step count is padded with empty steps: barriers only)
+      for (int step = 0; step < nsteps; step += kDqRing)
+        static_for<kDqRing>([&](auto e) { loader_step(std::integral_constant<int, (decltype(e)::value + 1) % kDqRing>{}, step + decltype(e)::value); });
       tag_base += nsteps;
     }
     __syncthreads();  // the compute waves are done with the K tiles
@@ -829,7 +820,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
     for (int cb = 0; cb < ncols; cb += cols_per_batch) {
       const int nsteps = prepare_batch(cb, min(ncols, cb + cols_per_batch));
       if (nsteps == 0) continue;
-      const int nsteps_pad = (nsteps + 3) & ~3;
+      const int nsteps_pad = (nsteps + kDqRing - 1) / kDqRing * kDqRing;
       for (int step = 0; step < nsteps_pad; ++step) {
         __syncthreads();
         if (step >= nsteps) continue;
