@@ -101,7 +101,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   float *sDelta = reinterpret_cast<float *>(smem + SM::oDelta);
   int *sList = reinterpret_cast<int *>(smem + SM::oList);
 
-  const int nb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + 63) / 64);
+  const int nb = item.idx, b = item.pair / a.heads, h = item.pair - b * a.heads;
   const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
   const int key0 = nb * 64;
   if (key0 >= Lk) return;
@@ -599,13 +600,11 @@ struct DqItem {
   int pair, sb;
 };
 __device__ __forceinline__ DqItem dq_decode_item(int id, int npairs, int nsb_max) {
-  // all superblocks of a (sequence, head) pair on one XCD (pair p on XCD p % 8), late ones first
-  const int x = id & 7, s = id >> 3;
-  const int pl = s / nsb_max, sbi = s - pl * nsb_max;
+  // late row blocks (the longest walks) first
+  const PairItem item = xcd_pair_item(id, npairs, nsb_max);
   DqItem w;
-  w.pair = pl * 8 + x;
-  w.sb = nsb_max - 1 - sbi;
-  if (w.pair >= npairs) w.pair = -1;
+  w.pair = item.pair < npairs ? item.pair : -1;
+  w.sb = nsb_max - 1 - item.idx;
   return w;
 }
 
@@ -986,8 +985,12 @@ static int launch_dkdv(const fmoba_attn_bwd_args &a, const BwdWs &ws, hipStream_
     set_error("attn_bwd: cannot reserve %zu bytes of LDS", smem);
     return 2;
   }
-  dim3 grid(ceil_div(a.max_seqlen_k, 64), a.heads, a.batch);
-  hipLaunchKernelGGL(kern, grid, dim3(256), smem, s, a, ws);
+  const int64_t items = (int64_t)a.batch * a.heads * ceil_div(a.max_seqlen_k, 64);
+  if (items >= ((int64_t)1 << 31)) {
+    set_error("attn_bwd: too many (sequence, head, key block) work items");
+    return 1;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)items), dim3(256), smem, s, a, ws);
   return 0;
 }
 
@@ -1000,8 +1003,7 @@ static int launch_dq(const fmoba_attn_bwd_args &a, const uint16_t *ws, hipStream
     return 2;
   }
   const int nsb_max = ceil_div(a.max_seqlen_q, kDqRows);
-  const int64_t pairs_per_xcd = ((int64_t)a.heads * a.batch + 7) / 8;
-  const int64_t items = 8 * pairs_per_xcd * nsb_max;
+  const int64_t items = (int64_t)a.heads * a.batch * nsb_max;
   if (items >= ((int64_t)1 << 31)) {
     set_error("attn_bwd: too many (sequence, head, superblock) work items");
     return 1;

@@ -89,7 +89,8 @@ __global__ __launch_bounds__((NCW + 2) * 64) void attn_fwd_col_kernel(fmoba_attn
   int *sSlot = reinterpret_cast<int *>(smem + SM::oSlot);
   int *sList = reinterpret_cast<int *>(smem + SM::oList);
 
-  const int nb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + KB - 1) / KB);
+  const int nb = item.idx, b = item.pair / a.heads, h = item.pair - b * a.heads;
   const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
   const int key0 = nb * KB;
   if (key0 >= Lk) return;
@@ -507,8 +508,12 @@ static int launch_fwd_col(const fmoba_attn_fwd_args &a, const FwdWs &ws, hipStre
     set_error("attn_fwd: cannot reserve %zu bytes of LDS", smem);
     return 2;
   }
-  dim3 grid(ceil_div(a.max_seqlen_k, KB), a.heads, a.batch);
-  hipLaunchKernelGGL(kern, grid, dim3((NCW + 2) * 64), smem, s, a, ws);
+  const int64_t items = (int64_t)a.batch * a.heads * ceil_div(a.max_seqlen_k, KB);
+  if (items >= ((int64_t)1 << 31)) {
+    set_error("attn_fwd: too many (sequence, head, key block) work items");
+    return 1;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)items), dim3((NCW + 2) * 64), smem, s, a, ws);
   return 0;
 }
 template <typename T>

@@ -75,9 +75,11 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
   uint32_t *sUnion = reinterpret_cast<uint32_t *>(smem + SM::oUnion);
   int *sOff = reinterpret_cast<int *>(smem + SM::oOff);
 
-  const int h = blockIdx.y, b = blockIdx.z;
+  const int nrb = (a.max_seqlen_q + 127) / 128;
+  const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, nrb);
+  const int b = item.pair / a.heads, h = item.pair - b * a.heads;
   const int q0 = a.cu_seqlens_q[b], Lq = a.cu_seqlens_q[b + 1] - q0;
-  const int rb = (int)gridDim.x - 1 - (int)blockIdx.x;  // the longest walks (last rows of a causal sequence) start first
+  const int rb = nrb - 1 - item.idx;  // the longest walks (last rows of a causal sequence) start first
   const int r0 = rb * 128;
   if (r0 >= Lq) return;
   const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
@@ -414,8 +416,12 @@ static int launch_rows(const fmoba_attn_fwd_args &a, const uint32_t *bm, int nw,
     set_error("attn_fwd: cannot reserve %zu bytes of LDS", smem);
     return 2;
   }
-  dim3 grid(ceil_div(a.max_seqlen_q, 128), a.heads, a.batch);
-  hipLaunchKernelGGL(kern, grid, dim3(512), smem, s, a, bm, nw);
+  const int64_t items = (int64_t)a.batch * a.heads * ceil_div(a.max_seqlen_q, 128);
+  if (items >= ((int64_t)1 << 31)) {
+    set_error("attn_fwd: too many (sequence, head, row block) work items");
+    return 1;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)items), dim3(512), smem, s, a, bm, nw);
   return 0;
 }
 

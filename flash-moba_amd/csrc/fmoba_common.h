@@ -293,6 +293,29 @@ __device__ __forceinline__ float order_key_float(uint32_t k) {
   return __uint_as_float(u);
 }
 
+// ------------------------------------------------------------------------------------
+// Work items of a 1-D grid of npairs * nper workgroups, nper items per (sequence, head) pair.
+// Workgroup i runs on XCD i % 8.  With a multiple of 8 pairs, pair p gets XCD p % 8 for all its
+// items, so what the items of a pair share (its K / V, or the Q / dO rows that its key blocks
+// gather again and again) stays in one L2; otherwise the items of a pair are simply consecutive.
+// ------------------------------------------------------------------------------------
+struct PairItem {
+  int pair, idx;
+};
+__device__ __forceinline__ PairItem xcd_pair_item(int id, int npairs, int nper) {
+  PairItem w;
+  if (npairs % 8 == 0) {
+    const int s = id >> 3;
+    const int pl = s / nper;
+    w.pair = pl * 8 + (id & 7);
+    w.idx = s - pl * nper;
+  } else {
+    w.pair = id / nper;
+    w.idx = id - w.pair * nper;
+  }
+  return w;
+}
+
 __device__ __forceinline__ Pack8 ld_global16(const void *p) { return *reinterpret_cast<const Pack8 *>(p); }
 __device__ __forceinline__ Pack8 zero_pack8() {
   Pack8 r;
