@@ -100,10 +100,9 @@ def time_events(fn, iters, warmup=1):
 # what the same counter reads for a plain 1 GiB copy (the summary of those runs is kept under profiles/).
 # Counter runs cannot be made from inside this script, so the figures are the committed measurement.
 MEASURED_TRAFFIC_BYTES = {
-    ("headline", "attn_fwd_col_kernel"): 16.307e9,
-    ("headline", "attn_fwd_combine_kernel"): 8.346e9,
-    ("headline", "attn_bwd_dkdv_kernel"): 18.632e9,
-    ("headline", "attn_bwd_dq_kernel"): 4.790e9,
+    ("headline", "attn_fwd_rows_kernel"): 1.500e9,
+    ("headline", "attn_bwd_dkdv_kernel"): 6.769e9,
+    ("headline", "attn_bwd_dq_kernel"): 4.801e9,
 }
 
 
@@ -279,6 +278,8 @@ def main():
         # the dK/dV kernel runs four of the five backward GEMMs (S, dP, dV, dK); the fifth is in it as well when the
         # library picks the partial-sum form of dQ (long sequences), else in the dQ kernel (this figure assumes the latter)
         kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 8.0 * D * pairs, "mfma")
+        if not hip.last_bwd_partials():
+            kernels["attn_bwd_dq_kernel"] = (phase_ms["dq"], 2.0 * D * pairs, "mfma")
     # sort alone, on the CSC the gating produced (already sorted input; same traffic)
     t_sort = time_events(lambda: torch.ops.flash_moba._varlen_sort(co, cn, ind), it)
     sort_bytes = 2 * int(cn.sum().item()) * 4 + 2 * cn.numel() * 8

@@ -1096,6 +1096,7 @@ extern "C" int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phase
                         a->o_row_stride,  a->o_head_stride,  a->do_row_stride, a->do_head_stride, a->dq_row_stride, a->dq_head_stride,
                         a->dk_row_stride, a->dk_head_stride, a->dv_row_stride, a->dv_head_stride};
   for (int64_t x : st) FMOBA_REQUIRE(x % 8 == 0, "attn_bwd: strides must be multiples of 8 elements");
+  FMOBA_REQUIRE(a->k_row_stride < ((int64_t)1 << 24), "attn_bwd: k_row_stride must be below 2^24 elements");
   const void *ptrs[] = {a->dout, a->q, a->k, a->v, a->out, a->dq, a->dk, a->dv};
   for (const void *p : ptrs) FMOBA_REQUIRE(((uintptr_t)p % 16) == 0, "attn_bwd: tensors must be 16-byte aligned");
 

@@ -348,6 +348,11 @@ def last_fwd_row_blocks():
     return int(getattr(_hint, "last_form", 0))
 
 
+def last_bwd_partials():
+    """1 if the last backward of this thread formed dQ from per-visit partials, 0 for the row-block form."""
+    return int(getattr(_hint, "last_bwd_partials", 0))
+
+
 def fwd_key_block(n_lg_block_dim):
     return int(load_library().fmoba_attn_fwd_key_block(int(n_lg_block_dim)))
 
@@ -514,6 +519,7 @@ def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_off
                         out.stride(0), out.stride(1), dout.stride(0), dout.stride(1),
                         dq.stride(0), dq.stride(1), dk_e.stride(0), dk_e.stride(1), dv_e.stride(0), dv_e.stride(1))
         ws_bytes = lib.fmoba_attn_bwd_workspace_bytes(ctypes.byref(a))
+        _hint.last_bwd_partials = int(lib.fmoba_attn_bwd_uses_partials(ctypes.byref(a)))
         ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
         a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
         if _phases is None:
