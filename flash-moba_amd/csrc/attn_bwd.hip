@@ -285,7 +285,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       lds_cu16 *trK = tr_lane_base(sK, LDQ, lane) + 8 * hh * LDQ;      // K^T with the same key order
       uint16_t *sdQ = reinterpret_cast<uint16_t *>(smem + SM::odQ) + (size_t)kh * 32 * LDH;
       Pack8 qa[2][KC], doa[2][KC];     // A operands of S and dP (this lane's row, its half of the head dim), double-buffered by chunk
-      Pack8 kb[2][KC], vb[2][KC];      // B operands: this lane's key, same slices of the head dim
+      // B operands of S and dP: this lane's key, its half of the head dim; they never change, so they stay in registers
+      Pack8 kb[KS], vb[KS];
+#pragma unroll
+      for (int t = 0; t < KS; ++t) {
+        kb[t] = *reinterpret_cast<const Pack8 *>(sK + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
+        vb[t] = *reinterpret_cast<const Pack8 *>(sV + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
+      }
       Pack8 dot[2][BC], qt[2][BC];     // dO^T / Q^T operands of the dV / dK products, double-buffered by chunk
       f32x4 lse4[2], del4[2];          // softmax inputs of a chunk's four rows
       int4 row4[2];
@@ -302,8 +308,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         for (int t = 0; t < KC; ++t) {
           qa[G & 1][t] = *reinterpret_cast<const Pack8 *>(tQ + (lane & 31) * LDQ + (hh * KS + G * KC + t) * 8);
           doa[G & 1][t] = *reinterpret_cast<const Pack8 *>(tdO + (lane & 31) * LDQ + (hh * KS + G * KC + t) * 8);
-          kb[G & 1][t] = *reinterpret_cast<const Pack8 *>(sK + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + G * KC + t) * 8);
-          vb[G & 1][t] = *reinterpret_cast<const Pack8 *>(sV + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + G * KC + t) * 8);
         }
       };
       auto mm_a = [&](auto tsc, auto gc) {
@@ -317,8 +321,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         }
   #pragma unroll
         for (int t = 0; t < KC; ++t) {
-          s[TS] = mfma32<T>(qa[G & 1][t], kb[G & 1][t], s[TS]);
-          dp[TS] = mfma32<T>(doa[G & 1][t], vb[G & 1][t], dp[TS]);
+          s[TS] = mfma32<T>(qa[G & 1][t], kb[G * KC + t], s[TS]);
+          dp[TS] = mfma32<T>(doa[G & 1][t], vb[G * KC + t], dp[TS]);
         }
       };
       auto ld_b = [&](auto pc, auto tsc, auto gc) {
