@@ -297,7 +297,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       int4 row4[2];
       Pack8 pf[2][2], dsf[2][2];       // P and dS of both tiles of the round as MFMA operands
       Pack8 dsx[4];                    // dS^T of all 64 keys as the B operand of the dQ products
-      Pack8 kt[NDH][4];                // K^T of this wave's half of the features
+      Pack8 kt[NDH][4];                // K^T of this wave's half of the features: never changes, stays in registers
+      if constexpr (DQP) {
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+          for (int d2 = 0; d2 < NDH; ++d2) {
+            const int lo = 16 * s4 * LDQ + (kh * NDH + d2) * 32;
+            kt[d2][s4] = tr_frag8_at(trK, lo, lo + 4 * LDQ);
+          }
+      }
       f32x16 dqa[NDH];
       f32x16 s[2], dp[2];
       auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
@@ -409,14 +418,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       auto dq_load = [&](auto tsc) {
         constexpr int TS = decltype(tsc)::value;
 #pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) {
-          dsx[s4] = tr_frag8_at(trdS, (TS * 64 + 16 * s4) * LDS_, (TS * 64 + 16 * s4 + 4) * LDS_);
-#pragma unroll
-          for (int d2 = 0; d2 < NDH; ++d2) {
-            const int lo = 16 * s4 * LDQ + (kh * NDH + d2) * 32;
-            kt[d2][s4] = tr_frag8_at(trK, lo, lo + 4 * LDQ);
-          }
-        }
+        for (int s4 = 0; s4 < 4; ++s4) dsx[s4] = tr_frag8_at(trdS, (TS * 64 + 16 * s4) * LDS_, (TS * 64 + 16 * s4 + 4) * LDS_);
       };
       auto dq_mma = [&](auto gc) {  // a quarter of the products per chunk
         constexpr int G = decltype(gc)::value;
