@@ -10,10 +10,13 @@
 //                                                                dO^T, Q^T via transposing LDS reads)
 //                            dQ^T_partial = K^T dS^T            (per visit of a (row, key block) pair)
 //                          dK/dV live in accumulator registers for the whole list and are written
-//                          once.  Every visit leaves a dQ partial row (16-bit, unscaled) in a slot
-//                          that the row hands out from a counter.
-//   attn_bwd_dq_combine_kernel : one wave per (row, head) adds the row's partials in ascending
-//                          key-block order and scales: dQ.  Work and traffic are proportional to
+//                          once.  For dQ the kernel leaves either its dS tiles (16-bit, indexed by
+//                          row-list position) or, per visit, a dQ partial row (16-bit, unscaled) in a
+//                          slot that the row hands out from a counter.
+//   attn_bwd_dq_kernel   : dQ from the dS tiles, one workgroup per 128 query rows, dQ in registers
+//                          (patterns in which a 128-row block meets a dozen rows or more per step).
+//   attn_bwd_dq_combine_kernel : dQ from the partials, one wave per (row, head) adds them in ascending
+//                          key-block order and scales.  Work and traffic are proportional to
 //                          the number of visits, whatever the number of chunks per sequence.
 // In the dK/dV kernel half of the waves compute and the other half only move data (global ->
 // registers -> LDS) two rounds ahead of the compute waves.  It runs four waves of 512 registers: a

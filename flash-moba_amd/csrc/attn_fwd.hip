@@ -1,4 +1,5 @@
-// Sparse attention forward over a CSC pattern, column-stationary, in two launches.
+// Sparse attention forward over a CSC pattern: the entry points, and the column-stationary form in two
+// launches (sparse patterns; the row-block form for dense ones is in attn_fwd_rows.hip).
 //
 //   attn_fwd_col_kernel     : one workgroup per (key block of KB = 64 or 128 keys, head,
 //                             sequence).  K of the block lives in MFMA operand registers, V in
@@ -17,7 +18,7 @@
 // Work and traffic are proportional to the number of (row, key block) visits whatever the number of
 // chunks per sequence; a row-stationary formulation degenerates when every 128-row block touches
 // thousands of chunks with one or two rows each.
-// In the first kernel waves 0,1 compute (one tile each per round) and waves 2,3 only move data
+// In the first kernel two or four waves compute (one tile each per round) and two more only move data
 // (global -> registers -> LDS), two rounds ahead.
 #include "fmoba_common.h"
 

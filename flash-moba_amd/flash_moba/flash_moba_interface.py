@@ -307,10 +307,12 @@ def flash_moba_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
                            moba_chunk_size, moba_topk, causal=True):
     """MoBA attention end to end: gate (mean-pool + top-k + CSC), then sparse attention."""
     flash_moba_gpu.keep_next_gate_selection()
-    col_offsets, col_nnz, indices = flash_topk_varlen_func(
-        q, k, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-        moba_topk, moba_chunk_size, causal=causal)
-    selection = flash_moba_gpu.take_gate_selection()
+    try:
+        col_offsets, col_nnz, indices = flash_topk_varlen_func(
+            q, k, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+            moba_topk, moba_chunk_size, causal=causal)
+    finally:
+        selection = flash_moba_gpu.take_gate_selection()
     lg_block_m = decide_lg_block_m(moba_topk, moba_chunk_size, max_seqlen_k, causal)
     if moba_chunk_size % 64 == 0:
         # a gated row visits at most top-k chunks: the forward needs no pass over the pattern to size its scratch,
