@@ -284,6 +284,7 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
   int *sIdx = reinterpret_cast<int *>(sVal + 2 * kGateRows * kBigCap);   // [2][128][kBigCap]
   int *sCnt = sIdx + 2 * kGateRows * kBigCap;                            // [2][128]
   int *sHist = sCnt + 2 * kGateRows;                                     // [max_cols]
+  int *sTrash = sHist + p.max_cols;                                      // [256]: takes the stores of lanes that have nothing to store
 
   const fmoba_fused_topk_args &a = p.a;
   const int mb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -332,6 +333,7 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
   if (tid < 2 * kGateRows) sCnt[tid] = 0;
   int cur = 0;
   const uint16_t *kmp = reinterpret_cast<const uint16_t *>(a.km) + (int64_t)hk * a.km_head_stride;
+#pragma nounroll
   for (int g = 0; g < ngroups; ++g) {
     const int c0 = g * GC;
     const int gsc = min(GC, nsc - c0);
@@ -390,6 +392,89 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
         for (int i = 0; i < 16; ++i) sc[t][i] = -INFINITY;
       }
     }
+    // ---- later groups: streaming update ---------------------------------------------------------
+    // A row that still has candidates in this group had at least GC of them in the first one, so it already holds
+    // kp winners.  Only the new scores that reach its weakest winner can enter (a new chunk has a higher index than
+    // every earlier one, so an equal score wins the tie): they are put into the row's other list, then each takes
+    // the place of the weakest winner if it beats it.  That is the top kp of the union, in the same total order
+    // (score descending, chunk descending) as the bisection below, which stays for the first group and for rows
+    // with more entrants than a list holds.
+    if (g > 0 && __all(m_prev == kp || nc <= c0)) {
+      float pmin = INFINITY;
+#pragma unroll
+      for (int j = 0; j < PL; ++j) pmin = fminf(pmin, pi[j] >= 0 ? pv[j] : INFINITY);
+      pmin = min_xor32_f(pmin);
+      int ne = 0;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) ne += (sc[t][i] >= pmin) ? 1 : 0;
+        }
+      int slot = 0;
+      if (ne > 0) slot = atomicAdd(&sCnt[nxt * kGateRows + rs], ne);
+      wave_lds_fence();
+      const int ne_row = sCnt[nxt * kGateRows + rs];
+      wave_lds_fence();
+      if (__all(ne_row <= kBigCap)) {
+        float *ev = sVal + (size_t)(nxt * kGateRows + rs) * kBigCap;
+        int *ei = sIdx + (size_t)(nxt * kGateRows + rs) * kBigCap;
+        // (no branches: a lane without an entrant at this position stores to its trash word)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          if (t < n_tiles) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const bool w = sc[t][i] >= pmin;
+              *(w ? ev + slot : reinterpret_cast<float *>(sTrash + tid)) = sc[t][i];
+              *(w ? ei + slot : sTrash + tid) = c0 + t * 32 + acc_row(i, hh);
+              slot += w ? 1 : 0;
+            }
+          }
+        wave_lds_fence();
+#pragma nounroll
+        for (int e = 0; __any(e < ne_row); ++e) {
+          const bool has = e < ne_row;
+          const float x = has ? ev[e] : -INFINITY;
+          const int c = has ? ei[e] : -1;
+          // the weakest winner of this lane's half of the list, then of the row
+          float vw = INFINITY;
+          int cw = 0x7fffffff, jw = -1;
+#pragma unroll
+          for (int j = 0; j < PL; ++j) {
+            const bool better = (pi[j] >= 0) & ((pv[j] < vw) | ((pv[j] == vw) & (pi[j] < cw)));
+            vw = better ? pv[j] : vw;
+            cw = better ? pi[j] : cw;
+            jw = better ? j : jw;
+          }
+          const float vo = shfl_xor32_f(vw);
+          const int co = shfl_xor32_i(cw);
+          const bool mine = (jw >= 0) & ((vw < vo) | ((vw == vo) & (cw < co)));
+          const float vr = mine ? vw : vo;
+          const int cr = mine ? cw : co;
+          const bool beats = has & ((x > vr) | ((x == vr) & (c > cr)));
+          const int jr = (beats & mine) ? jw : -1;
+#pragma unroll
+          for (int j = 0; j < PL; ++j) {
+            pv[j] = j == jr ? x : pv[j];
+            pi[j] = j == jr ? c : pi[j];
+          }
+        }
+        // the updated winners go back to where they came from; the list keeps its length
+#pragma unroll
+        for (int j = 0; j < PL; ++j) {
+          const int e = hh * PL + j;
+          if (e < m_prev) {
+            sVal[(cur * kGateRows + rs) * kBigCap + e] = pv[j];
+            sIdx[(cur * kGateRows + rs) * kBigCap + e] = pi[j];
+          }
+        }
+        continue;
+      }
+      // more entrants than a list holds: the general path below recounts from scratch
+      if (hh == 0) sCnt[nxt * kGateRows + rs] = 0;
+      wave_lds_fence();
+    }
     vmin = min_xor32_f(vmin);
     vmax = max_xor32_f(vmax);
     const int ntot = m_prev + max(0, min(nc - c0, GC));  // candidates that compete in this group
@@ -415,6 +500,7 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
       uint32_t hi_k = float_order_key(vmax);
       int c_hi = 0;
       bool open = need;
+#pragma nounroll
       for (int iter = 0;; ++iter) {
         if (open && hi_k - lo_k <= 1u) {
           tau = order_key_float(hi_k);
@@ -455,17 +541,18 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
 #pragma unroll
               for (int i = 0; i < 16; ++i) {
                 const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
-                cnt += (sc[t][i] == tau_eq && c >= trial) ? 1 : 0;
+                cnt += ((sc[t][i] == tau_eq) & (c >= trial)) ? 1 : 0;
               }
             }
 #pragma unroll
-          for (int j = 0; j < PL; ++j) cnt += (pv[j] == tau_eq && (uint32_t)pi[j] >= trial && pi[j] >= 0) ? 1 : 0;
+          for (int j = 0; j < PL; ++j) cnt += ((pv[j] == tau_eq) & ((uint32_t)pi[j] >= trial) & (pi[j] >= 0)) ? 1 : 0;
           return sum_xor32_i(cnt);
         };
         const int ceq = count_eq_ge(0u);
         const bool split = tie && ceq > n_eq;
         if (__any(split)) {
           uint32_t i_acc = 0u;
+#pragma nounroll
           for (int bit = 23; bit >= 0; --bit) {
             const uint32_t trial = i_acc | (1u << bit);
             const int cnt = count_eq_ge(trial);
@@ -486,17 +573,17 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
           for (int i = 0; i < 16; ++i) {
             const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
             const float x = sc[t][i];
-            nwin += ((x > tau) || (x == tau_eq && c >= iota)) ? 1 : 0;
+            nwin += ((x > tau) | ((x == tau_eq) & (c >= iota))) ? 1 : 0;
           }
         }
 #pragma unroll
-      for (int j = 0; j < PL; ++j) nwin += (pi[j] >= 0 && ((pv[j] > tau) || (pv[j] == tau_eq && (uint32_t)pi[j] >= iota))) ? 1 : 0;
+      for (int j = 0; j < PL; ++j) nwin += ((pi[j] >= 0) & ((pv[j] > tau) | ((pv[j] == tau_eq) & ((uint32_t)pi[j] >= iota)))) ? 1 : 0;
     }
     int slot = 0;
     if (nwin > 0) slot = atomicAdd(&sCnt[nxt * kGateRows + rs], nwin);
     float *ov = sVal + (size_t)(nxt * kGateRows + rs) * kBigCap;
     int *oi = sIdx + (size_t)(nxt * kGateRows + rs) * kBigCap;
-    if (nwin > 0) {
+    if (__any(nwin > 0)) {  // (no branches inside: a lane without a winner at a position stores to its trash word)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
         if (t < n_tiles) {
@@ -504,20 +591,19 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
           for (int i = 0; i < 16; ++i) {
             const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
             const float x = sc[t][i];
-            if (((x > tau) || (x == tau_eq && c >= iota)) && slot < kBigCap) {
-              ov[slot] = x;
-              oi[slot] = (int)c;
-              ++slot;
-            }
+            const bool w = (kp > 0) & ((x > tau) | ((x == tau_eq) & (c >= iota))) & (slot < kBigCap);
+            *(w ? ov + slot : reinterpret_cast<float *>(sTrash + tid)) = x;
+            *(w ? oi + slot : sTrash + tid) = (int)c;
+            slot += w ? 1 : 0;
           }
         }
 #pragma unroll
-      for (int j = 0; j < PL; ++j)
-        if (pi[j] >= 0 && ((pv[j] > tau) || (pv[j] == tau_eq && (uint32_t)pi[j] >= iota)) && slot < kBigCap) {
-          ov[slot] = pv[j];
-          oi[slot] = pi[j];
-          ++slot;
-        }
+      for (int j = 0; j < PL; ++j) {
+        const bool w = (kp > 0) & (pi[j] >= 0) & ((pv[j] > tau) | ((pv[j] == tau_eq) & ((uint32_t)pi[j] >= iota))) & (slot < kBigCap);
+        *(w ? ov + slot : reinterpret_cast<float *>(sTrash + tid)) = pv[j];
+        *(w ? oi + slot : sTrash + tid) = pi[j];
+        slot += w ? 1 : 0;
+      }
     }
     cur = nxt;
   }
@@ -763,7 +849,7 @@ static int launch_gate_nt(const TopkParams &p, dim3 grid, hipStream_t s) {
 template <typename T, int HD, int NT>
 static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
   const size_t tile = (size_t)NT * 32 * (HD + 16) * 2;
-  const size_t smem = tile + (size_t)2 * kGateRows * kBigCap * 8 + (size_t)2 * kGateRows * 4 + (size_t)p.max_cols * 4;
+  const size_t smem = tile + (size_t)2 * kGateRows * kBigCap * 8 + (size_t)2 * kGateRows * 4 + (size_t)p.max_cols * 4 + 256 * 4;
   if ((size_t)p.W * kGateRows * 4 > tile || smem > 160 * 1024) {
     set_error("fused_topk: %d key chunks per sequence exceed what the LDS of this build holds", p.max_cols);
     return 1;
