@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(TopkParams p) {
 #pragma unroll
               for (int i = 0; i < 16; ++i) {
                 const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
-                cnt += (sc[t][i] == tau_eq && c >= trial) ? 1 : 0;
+                cnt += ((sc[t][i] == tau_eq) & (c >= trial)) ? 1 : 0;
               }
             }
           cnt = sum_xor32_i(cnt);
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(TopkParams p) {
         for (int i = 0; i < 16; ++i) {
           const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
           const float x = sc[t][i];
-          const bool s = (x > tau) || (x == tau_eq && c >= iota);
+          const bool s = (x > tau) | ((x == tau_eq) & (c >= iota));
           w |= s ? (1u << ((8 * (i >> 2) + (i & 3)) + 4 * hh)) : 0u;
         }
       }
