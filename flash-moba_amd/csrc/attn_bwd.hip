@@ -217,7 +217,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           const int v = lt + 128 * i;
           const int row = v / VPR, e = (v - row * VPR) * 8;
           const int j = r * 64 + row;
-          const bool ok = e < D && j < seg_len && sList[min(j, seg_len - 1)] >= 0;
+          const bool ok = (e < D) & (j < seg_len) & (sList[min(j, seg_len - 1)] >= 0);
           Pack8 xq = lq[P][i], xo = ld[P][i];
 #pragma unroll
           for (int w = 0; w < 4; ++w) {
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           const int row = k * RPP + lane / LPR;
           const int r2 = sRow[TS * 32 + row], s2 = sSlot[TS * 32 + row];
           const Pack8 x = *reinterpret_cast<const Pack8 *>(sdQ + row * LDH + col);
-          const bool ok = r2 >= 0 && s2 < ws.cap;
+          const bool ok = (r2 >= 0) & (s2 < ws.cap);
           const int64_t pidx = ok ? ((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2 : trash;
           if (kh * (HD / 2) + col < D) *reinterpret_cast<Pack8 *>(ws.part + pidx * D + kh * (HD / 2) + col) = x;
           if (kh == 0 && col == 0) ws.pid[pidx] = nb;
@@ -795,7 +795,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
         for (int i = 0; i < DVV; ++i) {
           if (32 * i >= n) break;
           const int rel = prid[P][i] - m0;
-          const bool ok = (ltid >> 3) + 32 * i < n && (uint32_t)rel < (uint32_t)rows_sb && rel >= first_rel;
+          const bool ok = ((ltid >> 3) + 32 * i < n) & ((uint32_t)rel < (uint32_t)rows_sb) & (rel >= first_rel);
           if (ok) {
             *reinterpret_cast<Pack8 *>(tD + rel * LDD) = pd[P][i];
             if ((ltid & 7) == 0) tT[rel] = tag;

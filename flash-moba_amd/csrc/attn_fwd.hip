@@ -185,7 +185,7 @@ __global__ __launch_bounds__((NCW + 2) * 64) void attn_fwd_col_kernel(fmoba_attn
           const int v = lt + 128 * i;
           const int row = v / VPR, e = (v - row * VPR) * 8;
           const int j = r * RR + row;
-          const bool ok = e < D && j < seg_len && sList[min(j, seg_len - 1)] >= 0;
+          const bool ok = (e < D) & (j < seg_len) & (sList[min(j, seg_len - 1)] >= 0);
           Pack8 x = lq[P][i];
 #pragma unroll
           for (int w = 0; w < 4; ++w) x.w[w] = ok ? x.w[w] : 0u;
