@@ -154,6 +154,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="headline", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--dq-mode", type=int, default=0, choices=(0, 1, 2),
+                    help="dQ form of the per-stage timings: 0 = the library's choice (what the timed steps run), 1 = row blocks, 2 = partials")
     ap.add_argument("--fwd-mode", type=int, default=0, choices=(0, 1, 2),
                     help="forward form of the per-stage timings: 0 = the library's choice (what the timed steps run), 1 = columns, 2 = row blocks")
     ap.add_argument("--calib-copy", action="store_true",
@@ -269,7 +271,7 @@ def main():
         def bwd(**kw):
             hip.set_bwd_visits_hint(bwd_visits)
             return hip.moba_varlen_bwd(dout, qd, kd, vd, out, lse, dq, dk, dv, co, cn, ind, cu, cu, None, max_len, max_len, 0.0,
-                                       scale, False, True, 0.0, False, lg_m, chunk, None, None, **kw)
+                                       scale, False, True, 0.0, False, lg_m, chunk, None, None, _dq_mode=args.dq_mode, **kw)
 
         bwd(_phases=run_phases)
         t_bwd = time_events(bwd, it)

@@ -306,7 +306,12 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
 #pragma unroll
         for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, sc[kt][i]);
       mloc = max_xor32_f(mloc);
-      const float m_new = active ? fmaxf(m_run, mloc) : m_run;
+      // The reference point of the row's exponentials only moves when the block's maximum exceeds it by more than
+      // 2^8 after scaling (always on the row's first block): p stays below 256, which the 16-bit P and the fp32 sums
+      // hold easily, out and lse do not depend on the reference point, and O is rescaled a few times per row
+      // instead of whenever one of the wave's 32 rows meets a new maximum.
+      const bool grow = active & ((mloc - m_run) * scale_log2 > 8.f);
+      const float m_new = grow ? mloc : m_run;
       const float alpha = m_new == m_run ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);  // first visit: factor 0 on zeros
       const float neg_mc = active ? -m_new * scale_log2 : -INFINITY;  // rows that did not select the chunk: p = 0
       m_run = m_new;
