@@ -56,28 +56,6 @@ struct BwdSmem {
   static constexpr size_t bytes = mainBytes > redBytes ? mainBytes : redBytes;
 };
 
-template <typename F, int... I>
-__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{})
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F &&f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
-__device__ __forceinline__ int lower_bound_i32b(const int32_t *p, int n, int v) {
-  int lo = 0, hi = n;
-  while (lo < hi) {
-    const int mid = (lo + hi) >> 1;
-    if (p[mid] < v)
-      lo = mid + 1;
-    else
-      hi = mid;
-  }
-  return lo;
-}
-
 struct BwdWs {
   int32_t *cnt;    // [total_q * heads] visits handed out per (row, head)
   int32_t *pid;    // [total_q * heads * cap] key block id of each partial
@@ -150,7 +128,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     nnz = a.col_nnz[bh * a.max_cols + c];
     lbase = a.col_offsets[bh * a.max_cols + c];
     // rows r with r + off < key0 see no key of this block
-    if (causal && nnz > 0) start = lower_bound_i32b(a.row_indices + lbase, nnz, key0 - off);
+    if (causal && nnz > 0) start = lower_bound_i32(a.row_indices + lbase, nnz, key0 - off);
   }
   const int32_t *list = a.row_indices + lbase;
   const int koff = key0 - c * Bn;  // offset of this 64-key block inside its column
@@ -672,8 +650,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
       if (nnz > 0) {
         base = coff[c];
         const int32_t *list = a.row_indices + base;
-        lo = lower_bound_i32b(list, nnz, m0);
-        const int hi = lo + lower_bound_i32b(list + lo, nnz - lo, m0 + kDqRows);
+        lo = lower_bound_i32(list, nnz, m0);
+        const int hi = lo + lower_bound_i32(list + lo, nnz - lo, m0 + kDqRows);
         cnt = min(hi - lo, kDqRows);
       }
       sLo[c - cb] = lo;

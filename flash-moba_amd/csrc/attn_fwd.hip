@@ -47,27 +47,6 @@ struct FwdColSmem {
   static constexpr size_t bytes = oList + (size_t)kFwdListCap * 4;
 };
 
-template <typename F, int... I>
-__device__ __forceinline__ void fwd_static_for_impl(F &&f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void fwd_static_for(F &&f) {
-  fwd_static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
-__device__ __forceinline__ int lower_bound_i32(const int32_t *p, int n, int v) {
-  int lo = 0, hi = n;
-  while (lo < hi) {
-    const int mid = (lo + hi) >> 1;
-    if (p[mid] < v)
-      lo = mid + 1;
-    else
-      hi = mid;
-  }
-  return lo;
-}
-
 struct FwdWs {
   int32_t *cnt;      // [total_q * heads] visits handed out per (row, head)
   float4 *hdr;       // [total_q * heads * cap] {m (log2 domain), l, key block id, -}

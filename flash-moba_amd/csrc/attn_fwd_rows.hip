@@ -35,15 +35,6 @@ struct FwdRowsSmem {
   static_assert((size_t)4 * 32 * LDO * 2 <= 2 * stage, "output tiles must fit the K/V stages");
 };
 
-template <typename F, int... I>
-__device__ __forceinline__ void rows_static_for_impl(F &&f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void rows_static_for(F &&f) {
-  rows_static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
 // one bit per (row, head, chunk): bm[(h * nw + c / 32) * total_q + q0 + r] bit c % 32 (the layout the gating
 // leaves its selection in)
 __global__ __launch_bounds__(256) void csc_bitmap_kernel(fmoba_attn_fwd_args a, uint32_t *bm, int nw) {
@@ -332,7 +323,7 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
       Pack8 vt[2][2];  // V^T operands of one feature tile
       lds_cu16 *trV = tr_lane_base(sV, LDQ, lane) + 4 * hh * LDQ;
       float lsum = 0.f;
-      rows_static_for<16>([&](auto gi) {
+      static_for<16>([&](auto gi) {
         constexpr int g = decltype(gi)::value;
         constexpr int M0 = g * (2 * KS) / 16, M1 = (g + 1) * (2 * KS) / 16;
 #pragma unroll
@@ -359,7 +350,7 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
       });
       l_run += lsum;
       // ---- part 2: O^T += V^T P^T ----
-      rows_static_for<NDT>([&](auto di) {
+      static_for<NDT>([&](auto di) {
         constexpr int dt = decltype(di)::value;
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)

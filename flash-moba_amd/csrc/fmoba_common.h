@@ -3,6 +3,9 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
+#include <utility>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
@@ -291,6 +294,30 @@ __device__ __forceinline__ uint32_t float_order_key(float f) {
 __device__ __forceinline__ float order_key_float(uint32_t k) {
   uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
   return __uint_as_float(u);
+}
+
+// first position of an ascending list whose entry is not below v
+__device__ __forceinline__ int lower_bound_i32(const int32_t *p, int n, int v) {
+  int lo = 0, hi = n;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (p[mid] < v)
+      lo = mid + 1;
+    else
+      hi = mid;
+  }
+  return lo;
+}
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}): a loop whose index is a
+// compile-time constant inside the body (register arrays, template arguments)
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 // ------------------------------------------------------------------------------------
