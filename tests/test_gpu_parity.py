@@ -333,8 +333,6 @@ def _check_attention(fm, q, k, v, dout, cuq, cuk, co, cn, ind, lg_n, causal, sca
 @pytest.mark.parametrize("d", [64, 128, 96, 59])
 @pytest.mark.parametrize("sq,sk", [(113, 203), (128, 217), (256, 512), (512, 256), (1023, 1024)])
 def test_attention_random_pattern(fm, sq, sk, d, mha, causal, dtype):
-    if dtype == torch.float16 and (d != 128 or mha != "mha"):
-        pytest.skip("fp16 is covered at d=128 / mha")
     H = 6
     Hk = {"mha": 6, "gqa": 2, "mqa": 1}[mha]
     # padded batch in the spirit of tests/test_moba_attn.py:103-104: lengths a little below the maximum
