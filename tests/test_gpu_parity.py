@@ -401,6 +401,32 @@ def test_fused_path_hands_the_gating_selection_to_the_forward(fm, lens, chunk, t
     assert torch.equal(out, out2)
 
 
+def test_row_block_forms_over_many_columns(fm):
+    # more than 32 chunks (several selection words per row) in the forward, more than 256 columns (several column
+    # batches per row block) in the row-block dQ pass
+    lens = [300 * 64 + 40, 2500]
+    H, D, chunk, topk = 2, 64, 64, 5
+    q, k, v, cu, dout = O.make_inputs(lens, H, D, chunk, 41, torch.bfloat16, with_dout=True)
+    Q, K, V, CU, DO = q.cuda(), k.cuda(), v.cuda(), cu.cuda(), dout.cuda()
+    co, cn, ind = fm.api.flash_topk_varlen_func(Q, K, CU, CU, max(lens), max(lens), topk, chunk, causal=True)
+    scale = D ** -0.5
+    out, lse, _, _ = fm.hip.moba_varlen_fwd(Q, K, V, None, co, cn, ind, CU, CU, None, None, None, max(lens), max(lens), 0.0, scale,
+                                            False, True, 0.0, False, 128, chunk, None, _fwd_mode=2)
+    assert fm.hip.last_fwd_row_blocks() == 1
+    dq, dk, dv, _ = fm.hip.moba_varlen_bwd(DO, Q, K, V, out, lse, None, None, None, co, cn, ind, CU, CU, None, max(lens), max(lens),
+                                           0.0, scale, False, True, 0.0, False, 128, chunk, None, None, _dq_mode=1)
+    assert fm.hip.last_bwd_partials() == 0
+    # the column form / the partials form of the same call as the reference: they are checked against the oracle elsewhere
+    out1, lse1, _, _ = fm.hip.moba_varlen_fwd(Q, K, V, None, co, cn, ind, CU, CU, None, None, None, max(lens), max(lens), 0.0, scale,
+                                              False, True, 0.0, False, 128, chunk, None, _fwd_mode=1)
+    dq2, dk2, dv2, _ = fm.hip.moba_varlen_bwd(DO, Q, K, V, out, lse, None, None, None, co, cn, ind, CU, CU, None, max(lens), max(lens),
+                                              0.0, scale, False, True, 0.0, False, 128, chunk, None, None, _dq_mode=2)
+    assert_close("out", out, out1.float().cpu(), 2e-2, 1e-2)
+    assert_close("lse", lse, lse1.float().cpu(), 2e-2, 1e-2)
+    assert_close("dq", dq, dq2.float().cpu(), 2e-2, 1e-2)
+    assert torch.equal(dk, dk2) and torch.equal(dv, dv2)
+
+
 @pytest.mark.parametrize("dq_mode", [1, 2])
 @pytest.mark.parametrize("d,chunk", [(128, 64), (64, 128), (96, 64)])
 def test_backward_both_dq_forms(fm, dq_mode, d, chunk):
