@@ -360,7 +360,7 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
     float vmin = INFINITY, vmax = -INFINITY;
 #pragma unroll
     for (int j = 0; j < PL; ++j) {
-      const int e = hh * PL + j;
+      const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
       const bool ok = e < m_prev;
       pv[j] = ok ? sVal[(cur * kGateRows + rs) * kBigCap + e] : -INFINITY;
       pi[j] = ok ? sIdx[(cur * kGateRows + rs) * kBigCap + e] : -1;
@@ -432,38 +432,46 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
             }
           }
         wave_lds_fence();
+        // (with at most 16 winners a lane holds at most 8 of them: the short variant of the loop)
+        auto stream = [&](auto plc) {
+          constexpr int PLX = decltype(plc)::value;
 #pragma nounroll
-        for (int e = 0; __any(e < ne_row); ++e) {
-          const bool has = e < ne_row;
-          const float x = has ? ev[e] : -INFINITY;
-          const int c = has ? ei[e] : -1;
-          // the weakest winner of this lane's half of the list, then of the row
-          float vw = INFINITY;
-          int cw = 0x7fffffff, jw = -1;
+          for (int e = 0; __any(e < ne_row); ++e) {
+            const bool has = e < ne_row;
+            const float x = has ? ev[e] : -INFINITY;
+            const int c = has ? ei[e] : -1;
+            // the weakest winner of this lane's half of the list, then of the row
+            float vw = INFINITY;
+            int cw = 0x7fffffff, jw = -1;
 #pragma unroll
-          for (int j = 0; j < PL; ++j) {
-            const bool better = (pi[j] >= 0) & ((pv[j] < vw) | ((pv[j] == vw) & (pi[j] < cw)));
-            vw = better ? pv[j] : vw;
-            cw = better ? pi[j] : cw;
-            jw = better ? j : jw;
-          }
-          const float vo = shfl_xor32_f(vw);
-          const int co = shfl_xor32_i(cw);
-          const bool mine = (jw >= 0) & ((vw < vo) | ((vw == vo) & (cw < co)));
-          const float vr = mine ? vw : vo;
-          const int cr = mine ? cw : co;
-          const bool beats = has & ((x > vr) | ((x == vr) & (c > cr)));
-          const int jr = (beats & mine) ? jw : -1;
+            for (int j = 0; j < PLX; ++j) {
+              const bool better = (pi[j] >= 0) & ((pv[j] < vw) | ((pv[j] == vw) & (pi[j] < cw)));
+              vw = better ? pv[j] : vw;
+              cw = better ? pi[j] : cw;
+              jw = better ? j : jw;
+            }
+            const float vo = shfl_xor32_f(vw);
+            const int co = shfl_xor32_i(cw);
+            const bool mine = (jw >= 0) & ((vw < vo) | ((vw == vo) & (cw < co)));
+            const float vr = mine ? vw : vo;
+            const int cr = mine ? cw : co;
+            const bool beats = has & ((x > vr) | ((x == vr) & (c > cr)));
+            const int jr = (beats & mine) ? jw : -1;
 #pragma unroll
-          for (int j = 0; j < PL; ++j) {
-            pv[j] = j == jr ? x : pv[j];
-            pi[j] = j == jr ? c : pi[j];
+            for (int j = 0; j < PLX; ++j) {
+              pv[j] = j == jr ? x : pv[j];
+              pi[j] = j == jr ? c : pi[j];
+            }
           }
-        }
+        };
+        if (kp <= PL)
+          stream(std::integral_constant<int, PL / 2>{});
+        else
+          stream(std::integral_constant<int, PL>{});
         // the updated winners go back to where they came from; the list keeps its length
 #pragma unroll
         for (int j = 0; j < PL; ++j) {
-          const int e = hh * PL + j;
+          const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
           if (e < m_prev) {
             sVal[(cur * kGateRows + rs) * kBigCap + e] = pv[j];
             sIdx[(cur * kGateRows + rs) * kBigCap + e] = pi[j];
@@ -617,7 +625,7 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
     const int m = min(sCnt[cur * kGateRows + rs], kBigCap);
 #pragma unroll
     for (int j = 0; j < PL; ++j) {
-      const int e = hh * PL + j;
+      const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
       if (e < m) {
         const int c = sIdx[(cur * kGateRows + rs) * kBigCap + e];
         atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
