@@ -38,6 +38,8 @@ CONFIGS = {
     "c2": ([8192], 16, 128, 128, 8, False),
     "c3": ([32768], 32, 128, 128, 16, True),
     "c5": ([262144], 16, 128, 128, 16, True),
+    # one point of the reference's own sequence-length sweep (benchmarks/bench_flash_moba.py): batch 2, top-k 8
+    "sweep64k": ([65536, 65536], 16, 128, 128, 8, True),
 }
 
 

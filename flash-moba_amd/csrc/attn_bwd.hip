@@ -221,11 +221,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       store_round(P0{}, 0);
       load_round(P0{}, 2);
       auto loader_round = [&](auto par, int r) {  // par: parity of round r + 1
-        // The compute waves exchange dS^T of the round's two tiles through LDS, which takes two more
-        // barriers per round; the loaders' work is spread between them so that nobody waits for it.
+        // The compute waves exchange dS^T of the round's two tiles through LDS, which takes one more
+        // barrier per round.
         __syncthreads();  // round r is in LDS; the readers of round r-1 are done with the other buffer
         if (r + 1 < nround) store_round(par, r + 1);
-        if constexpr (DQP) __syncthreads();
         load_round(par, r + 3);
         if constexpr (DQP) __syncthreads();
       };
@@ -375,10 +374,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           *reinterpret_cast<uint2 *>(t + 16 * s2 + 4 * hh) = make_uint2(dsf[TS][s2].w[0], dsf[TS][s2].w[1]);
           *reinterpret_cast<uint2 *>(t + 16 * s2 + 8 + 4 * hh) = make_uint2(dsf[TS][s2].w[2], dsf[TS][s2].w[3]);
         }
-        if constexpr (DQP)
-          __syncthreads();
-        else
-          wave_lds_fence();
+        if constexpr (!DQP) wave_lds_fence();  // (the partials form waits for both key halves at a workgroup barrier later)
       };
       // dS form: the wave's 32 keys of every row go to the dS tile of the row's list entry
       int dsrow = -1;
@@ -464,14 +460,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           smx(C0{}, gc);
           fence();
         });
-        // dV, dK, dQ of the first tile between the softmax rows of the second
+        // dV, dK of the first tile between the softmax rows of the second
         ds_write(C0{});
         ld_b(pc, C0{}, C0{});
         ld_s(pc, C1{}, C0{});
-        if constexpr (DQP)
-          dq_load(C0{});
-        else
-          ds_read(pc, C0{});
+        if constexpr (!DQP) ds_read(pc, C0{});
         fence();
         static_for<4>([&](auto gc) {
           constexpr int G = decltype(gc)::value;
@@ -480,17 +473,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
             ld_s(pc, C1{}, std::integral_constant<int, G + 1>{});
           }
           mm_b(C0{}, gc);
-          if constexpr (DQP) dq_mma(gc);
           smx(C1{}, gc);
           if constexpr (!DQP && G == 1) ds_store(2 * r);
           fence();
         });
-        if constexpr (DQP) dq_store(pc, C0{});
-        // dV, dK, dQ of the second tile
+        // dV, dK of the second tile; in the partials form dQ of the first one runs between them: by now both key
+        // halves have put dS^T of both tiles into LDS, so the one barrier the exchange needs hardly ever waits
         ds_write(C1{});
+        if constexpr (DQP) __syncthreads();
         ld_b(pc, C1{}, C0{});
         if constexpr (DQP)
-          dq_load(C1{});
+          dq_load(C0{});
         else
           ds_read(pc, C1{});
         fence();
@@ -502,7 +495,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           if constexpr (!DQP && G == 1) ds_store(2 * r + 1);
           fence();
         });
-        if constexpr (DQP) dq_store(pc, C1{});
+        if constexpr (DQP) {
+          dq_store(pc, C0{});
+          // dQ of the second tile
+          dq_load(C1{});
+          fence();
+          static_for<4>([&](auto gc) {
+            dq_mma(gc);
+            fence();
+          });
+          dq_store(pc, C1{});
+        }
       };
 
       const int nround_pad = (nround + 1) & ~1;
@@ -512,8 +515,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         __syncthreads();
         if (r + 1 < nround) {
           process_round(C1{}, r + 1);
-        } else if constexpr (DQP) {  // padding round: only the barriers
-          __syncthreads();
+        } else if constexpr (DQP) {  // padding round: only the barrier
           __syncthreads();
         }
       }
