@@ -559,23 +559,24 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 // ------------------------------------------------------------------------------------
 // dQ, first form: row blocks.  One workgroup owns 128 consecutive query rows of one (sequence, head) and walks the
 // 64-key blocks of every column in which one of its rows appears.  The dS rows of a step (written by the dK/dV
-// pass in list order) are put at the place of their query row in LDS, rows that are absent keep a stale tag and
-// contribute zeros, so every compute wave multiplies its own 32 rows and keeps dQ in registers for the whole walk.
+// pass in list order) go from global memory straight into the registers of the lane that owns the query row; rows
+// that are absent contribute zeros, so every compute wave multiplies its own 32 rows and keeps dQ in registers for
+// the whole walk.  Registers (128) and LDS (about 52 KB) leave room for two workgroups per compute unit: one
+// workgroup's waits at barriers and on LDS are covered by the other.
 // ------------------------------------------------------------------------------------
 constexpr int kDqRows = 128;
 constexpr int kDqColBatch = 256;
 constexpr int kDqMaxSteps = 512;
-constexpr int kDqRing = 4;  // steps the loaders run ahead: the dS rows come from HBM
+constexpr int kDqRing = 4;   // K tiles the loaders keep in flight
+constexpr int kDqRows2 = 2;  // dS rows in flight per compute lane (16 registers each)
 
 template <int HD>
 struct DqSmem {
   static constexpr int LDQ = HD + 16;  // elements, K tile
-  static constexpr int LDD = 64 + 8;   // elements, dS rows [128][64 keys]
   static constexpr int LDO = HD + 8;   // elements, per-wave output tile [32 rows][LDO] (reuses the K tiles at the end)
   static constexpr size_t oK = 0;                                   // [2][64][LDQ]
-  static constexpr size_t oD = oK + (size_t)2 * 64 * LDQ * 2;      // [2][128][LDD]
-  static constexpr size_t oTag = oD + (size_t)2 * kDqRows * LDD * 2;  // int[2][128]: step that last wrote the row
-  static constexpr size_t oLo = oTag + 2 * kDqRows * 4;
+  static constexpr size_t oTag = oK + (size_t)2 * 64 * LDQ * 2;    // int[3][128]: (step tag << 8) | list position of the row in that step
+  static constexpr size_t oLo = oTag + 3 * kDqRows * 4;
   static constexpr size_t oCnt = oLo + kDqColBatch * 4;
   static constexpr size_t oStep = oCnt + kDqColBatch * 4;
   static constexpr size_t oOff = oStep + kDqMaxSteps * 4;          // int64[kDqColBatch]
@@ -598,15 +599,13 @@ __device__ __forceinline__ DqItem dq_decode_item(int id, int npairs, int nsb_max
 }
 
 template <typename T, int HD>
-__global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a, const uint16_t *ds_ws, int nsb_max) {
+__global__ __launch_bounds__(512, 4) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a, const uint16_t *ds_ws, int nsb_max) {
   typedef DqSmem<HD> SM;
-  constexpr int LDQ = SM::LDQ, LDD = SM::LDD, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
+  constexpr int LDQ = SM::LDQ, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
   constexpr int KVV = 64 * VPR / 256;  // K-tile vectors per loader thread
-  constexpr int DVV = kDqRows * 8 / 256;  // dS-row vectors (64 keys = 8 vectors per row) per loader thread
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint16_t *sK = reinterpret_cast<uint16_t *>(smem + SM::oK);
-  uint16_t *sD = reinterpret_cast<uint16_t *>(smem + SM::oD);
-  int *sTag = reinterpret_cast<int *>(smem + SM::oTag);
+  int *sPos = reinterpret_cast<int *>(smem + SM::oTag);
   int *sLo = reinterpret_cast<int *>(smem + SM::oLo);
   int *sCnt = reinterpret_cast<int *>(smem + SM::oCnt);
   int *sStep = reinterpret_cast<int *>(smem + SM::oStep);
@@ -631,7 +630,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
   const int ltid = tid & 255;
   const bool causal = a.is_causal != 0;
 
-  for (int v = tid; v < 2 * kDqRows; v += 512) sTag[v] = 0;  // step tags start at 1
+  for (int v = tid; v < 3 * kDqRows; v += 512) sPos[v] = 0;  // step tags start at 1
 
   int ncols = min((Lk + Bn - 1) / Bn, a.max_cols);
   const int last_rowpos = m0 + rows_sb - 1 + off;
@@ -691,18 +690,21 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
   };
 
   typedef std::integral_constant<int, 0> P0;
-  // LDS is double buffered by step parity: while the compute waves work on step s the loaders put
-  // step s+1 into the other buffer and then fetch step s+1+kDqRing into the ring entry that this frees.
-  // The two roles run separate code with the same barrier sequence.  Every load_step is issued
-  // unconditionally and no control flow joins the loader path: the compiler sizes each wait by the
-  // smallest number of younger loads over all paths that reach it, and a path without loads (or one
-  // skipped load) would make every store wait for the whole ring.
+  // The K tiles are double buffered in LDS by step parity: while the compute waves work on step s the loaders put
+  // step s+1 into the other buffer and then fetch step s+1+RK into the ring entry that this frees.  The loaders also
+  // tell every query row of the block where its dS row of a step lies (position in the step's list segment, tagged
+  // with the step number), NR steps ahead; a compute lane fetches the 128 bytes of its row (one half per lane of the
+  // pair that holds the row) NR-1 steps ahead of their use.  Rows that are not in a step keep a stale tag.
+  // The two roles run separate code with the same barrier sequence.  Every load is issued unconditionally and no
+  // control flow joins a path between a load and its use: the compiler sizes each wait by the smallest number of
+  // younger loads over all paths that reach it, and a path without loads would make every use wait for the whole ring.
+  constexpr int RK = kDqRing;  // ring of the K tiles (and of the row ids, which run NR - 1 steps ahead of them)
+  constexpr int NR = kDqRows2;
+  constexpr int PADTO = (NR % 4 == 0) ? NR : ((NR % 2 == 0) ? 2 * NR : 4 * NR);
   if (is_loader) {
-    // loader rings: the dS rows come from HBM (about 2 us under load), a step takes well under 1 us
-    Pack8 pk[kDqRing][KVV], pd[kDqRing][DVV];
-    int prid[kDqRing][DVV];
+    Pack8 pk[RK][KVV];
+    int prid[RK];
     int tag_base = 0;
-    // per-lane parts of the K-tile addresses: vector i of this thread is key ltid / VPR + i * (256 / VPR), features (ltid % VPR) * 8
     uint32_t kvo[KVV];
 #pragma unroll
     for (int i = 0; i < KVV; ++i) kvo[i] = (uint32_t)((ltid / VPR + i * (256 / VPR)) * (int)a.k_row_stride + min((ltid % VPR) * 8, D - 8));
@@ -710,16 +712,25 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
     for (int cb = 0; cb < ncols; cb += cols_per_batch) {
       const int nsteps = prepare_batch(cb, min(ncols, cb + cols_per_batch));
       if (nsteps == 0) continue;
-      // Loads are unconditional (indices clamped into the valid range, the surplus dropped when it is stored).
-      // Addresses are a uniform base (scalar registers) plus a 32-bit offset per lane that does not depend on
-      // the step: the loaders share their SIMDs with the compute waves, every instruction they issue is taken
-      // from those.
+      auto row_id = [&](int step) {  // row of list position ltid of the step (clamped), for the threads that write positions
+        const int4 info = sInfo[min(step, nsteps - 1)];
+        const int n = __builtin_amdgcn_readfirstlane(info.y);
+        const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
+        return a.row_indices[pos0 + min(ltid & 127, n - 1)];
+      };
+      auto put_pos = [&](int step, int rr) {  // positions of the rows of `step`
+        if (step < nsteps && ltid < kDqRows) {
+          const int4 info = sInfo[step];
+          const int key0 = info.x, n = info.y;
+          const int first_rel = causal ? key0 - off - m0 : -0x40000000;  // rows before it see no key of the block
+          const int rel = rr - m0;
+          if ((ltid < n) & ((uint32_t)rel < (uint32_t)rows_sb) & (rel >= first_rel)) sPos[(step % 3) * kDqRows + rel] = ((tag_base + step + 1) << 8) | ltid;
+        }
+      };
+      // K of `step`, row ids of `step + 2`
       auto load_step = [&](auto par, int step) {
         constexpr int P = decltype(par)::value;
-        const int4 info = sInfo[min(step, nsteps - 1)];  // past the end: a redundant load, never stored
-        const int key0 = __builtin_amdgcn_readfirstlane(info.x), n = __builtin_amdgcn_readfirstlane(info.y);
-        const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
-        const int koff = key0 - (key0 / Bn) * Bn;  // offset of the 64-key block inside its column
+        const int key0 = __builtin_amdgcn_readfirstlane(sInfo[min(step, nsteps - 1)].x);
         if (key0 + 64 <= Lk) {
           const uint16_t *kb0 = kp + (int64_t)key0 * a.k_row_stride;
 #pragma unroll
@@ -732,25 +743,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
             pk[P][i] = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
           }
         }
-        const uint16_t *db0 = ds_ws + pos0 * Bn + koff + (ltid & 7) * 8;
-        const int32_t *rb0 = a.row_indices + pos0;
-        // rows 32 i .. 32 i + 31 of the step's dS tile; a group past the last row is not fetched (the first always is:
-        // the waits the compiler places count the loads that every path issues)
-#pragma unroll
-        for (int i = 0; i < DVV; ++i) {
-          if (i == 0 || 32 * i < n) {
-            const uint32_t row = (uint32_t)min((ltid >> 3) + 32 * i, n - 1);
-            pd[P][i] = ld_global16(db0 + row * (uint32_t)Bn);
-            prid[P][i] = rb0[row];
-          }
-        }
+        prid[P] = row_id(step + NR - 1);
       };
       auto store_step = [&](auto par, int step) {
         constexpr int P = decltype(par)::value;
-        const int buf = step & 1;
-        const int4 info = sInfo[step];
-        const int key0 = __builtin_amdgcn_readfirstlane(info.x), n = __builtin_amdgcn_readfirstlane(info.y);
-        uint16_t *tK = sK + (size_t)buf * 64 * LDQ;
+        const int key0 = __builtin_amdgcn_readfirstlane(sInfo[step].x);
+        uint16_t *tK = sK + (size_t)(step & 1) * 64 * LDQ;
         if (D == HD && key0 + 64 <= Lk) {
 #pragma unroll
           for (int i = 0; i < KVV; ++i) *reinterpret_cast<Pack8 *>(tK + klo + i * (256 / VPR) * LDQ) = pk[P][i];
@@ -759,45 +757,32 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
           for (int i = 0; i < KVV; ++i) {
             const int v = ltid + i * 256;
             const int key = v / VPR, e = (v - key * VPR) * 8;
-            const bool ok = key0 + key < Lk && e < D;
+            const bool ok = (key0 + key < Lk) & (e < D);
             Pack8 x = pk[P][i];
 #pragma unroll
             for (int w = 0; w < 4; ++w) x.w[w] = ok ? x.w[w] : 0u;
             *reinterpret_cast<Pack8 *>(tK + key * LDQ + e) = x;
           }
         }
-        // the dK/dV pass wrote dS only for rows of this sequence that can see a key of the block
-        const int first_rel = causal ? key0 - off - m0 : -0x40000000;  // rows before it see no key of the block
-        uint16_t *tD = sD + (size_t)buf * kDqRows * LDD + (ltid & 7) * 8;
-        int *tT = sTag + buf * kDqRows;
-        const int tag = tag_base + step + 1;
-#pragma unroll
-        for (int i = 0; i < DVV; ++i) {
-          if (32 * i >= n) break;
-          const int rel = prid[P][i] - m0;
-          const bool ok = ((ltid >> 3) + 32 * i < n) & ((uint32_t)rel < (uint32_t)rows_sb) & (rel >= first_rel);
-          if (ok) {
-            *reinterpret_cast<Pack8 *>(tD + rel * LDD) = pd[P][i];
-            if ((ltid & 7) == 0) tT[rel] = tag;
-          }
-        }
+        put_pos(step + NR - 1, prid[P]);
       };
-      static_for<kDqRing>([&](auto e) { load_step(e, decltype(e)::value); });
+      static_for<RK>([&](auto e) { load_step(e, decltype(e)::value); });
+      for (int t = 0; t < NR - 1; ++t) put_pos(t, row_id(t));
       store_step(P0{}, 0);
-      load_step(P0{}, kDqRing);
+      load_step(P0{}, RK);
+      __syncthreads();  // the positions of steps 0, 1, 2 are in LDS
       auto loader_step = [&](auto par, int step) {  // par: ring entry of step + 1, stored during step
         __syncthreads();
         if (step + 1 < nsteps) store_step(par, step + 1);
-        load_step(par, step + 1 + kDqRing);
+        load_step(par, step + 1 + RK);
       };
-      // whole turns of the ring (the step count is padded with empty steps: barriers only)
-      for (int step = 0; step < nsteps; step += kDqRing)
-        static_for<kDqRing>([&](auto e) { loader_step(std::integral_constant<int, (decltype(e)::value + 1) % kDqRing>{}, step + decltype(e)::value); });
+      const int nsteps_pad = (nsteps + PADTO - 1) / PADTO * PADTO;
+      for (int step = 0; step < nsteps_pad; step += RK)
+        static_for<RK>([&](auto e) { loader_step(std::integral_constant<int, (decltype(e)::value + 1) % RK>{}, step + decltype(e)::value); });
       tag_base += nsteps;
     }
     __syncthreads();  // the compute waves are done with the K tiles
   } else {
-    // dQ^T of this wave's 32 rows: register i of feature tile dt <-> feature dt*32 + acc_row(i, hh), this lane's row
     f32x16 acc[NDT];
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
@@ -805,45 +790,66 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
       for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
     const int myrow = wave * 32 + (lane & 31);
     int tag_base = 0;
+    Pack8 df[NR][4];   // this lane's dS row of NR consecutive steps (B operands)
+    bool dfp[NR];
     for (int cb = 0; cb < ncols; cb += cols_per_batch) {
       const int nsteps = prepare_batch(cb, min(ncols, cb + cols_per_batch));
       if (nsteps == 0) continue;
-      const int nsteps_pad = (nsteps + kDqRing - 1) / kDqRing * kDqRing;
-      for (int step = 0; step < nsteps_pad; ++step) {
-        __syncthreads();
-        if (step >= nsteps) continue;
-        const int buf = step & 1;
-        const bool present = sTag[buf * kDqRows + myrow] == tag_base + step + 1;
-        if (!__any(present)) continue;
-        // this lane's dS row as the B operand (zeros for a row that is not in the step)
-        Pack8 df[4];
+      // fetch this lane's dS row of `step` into ring entry R (unconditional: an absent row reads position 0)
+      auto fetch = [&](auto rc, int step) {
+        constexpr int R = decltype(rc)::value;
+        const int sc_ = min(step, nsteps - 1);
+        const int4 info = sInfo[sc_];
+        const int key0 = __builtin_amdgcn_readfirstlane(info.x);
+        const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
+        const int koff = key0 - (key0 / Bn) * Bn;
+        const int v = sPos[(sc_ % 3) * kDqRows + myrow];
+        const bool pres = (step < nsteps) & ((v >> 8) == tag_base + sc_ + 1);
+        const uint32_t j = pres ? (uint32_t)(v & 255) : 0u;
+        const uint16_t *rp = ds_ws + pos0 * Bn + koff + 8 * hh;
 #pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) {
-          df[s4] = *reinterpret_cast<const Pack8 *>(sD + ((size_t)buf * kDqRows + myrow) * LDD + 16 * s4 + 8 * hh);
+        for (int s4 = 0; s4 < 4; ++s4) df[R][s4] = ld_global16(rp + j * (uint32_t)Bn + 16 * s4);
+        dfp[R] = pres;
+      };
+      auto compute = [&](auto rc, int step) {
+        constexpr int R = decltype(rc)::value;
+        const bool present = dfp[R];
+        if (!__any(present)) return;
+        Pack8 dz[4];
 #pragma unroll
-          for (int w = 0; w < 4; ++w) df[s4].w[w] = present ? df[s4].w[w] : 0u;
-        }
-        lds_cu16 *trK = tr_lane_base(sK + (size_t)buf * 64 * LDQ, LDQ, lane) + 8 * hh * LDQ;
-        // K^T operands one feature tile ahead of the products that use them
-        Pack8 kf[2][4];
+        for (int s4 = 0; s4 < 4; ++s4)
 #pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) kf[0][s4] = tr_frag8_at(trK, 16 * s4 * LDQ, (16 * s4 + 4) * LDQ);
+          for (int w = 0; w < 4; ++w) dz[s4].w[w] = present ? df[R][s4].w[w] : 0u;
+        lds_cu16 *trK = tr_lane_base(sK + (size_t)(step & 1) * 64 * LDQ, LDQ, lane) + 8 * hh * LDQ;
+        // K^T operands half a feature tile (two products) ahead of their use
+        Pack8 kf[2][2];
+        auto kread = [&](int u, Pack8 (&dst)[2]) {  // unit u: feature tile u / 2, keys 32 (u % 2) .. + 31
+          const int dt = u >> 1, sb = 2 * (u & 1);
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-          if (dt + 1 < NDT) {
+          for (int s2 = 0; s2 < 2; ++s2) dst[s2] = tr_frag8_at(trK, 16 * (sb + s2) * LDQ + dt * 32, (16 * (sb + s2) + 4) * LDQ + dt * 32);
+        };
+        kread(0, kf[0]);
 #pragma unroll
-            for (int s4 = 0; s4 < 4; ++s4) kf[(dt + 1) & 1][s4] = tr_frag8_at(trK, 16 * s4 * LDQ + (dt + 1) * 32, (16 * s4 + 4) * LDQ + (dt + 1) * 32);
-          }
+        for (int u = 0; u < 2 * NDT; ++u) {
+          if (u + 1 < 2 * NDT) kread(u + 1, kf[(u + 1) & 1]);
 #pragma unroll
-          for (int s4 = 0; s4 < 4; ++s4) acc[dt] = mfma32<T>(kf[dt & 1][s4], df[s4], acc[dt]);  // dQ^T[d][row] += K^T[d][key] dS^T[key][row]
+          for (int s2 = 0; s2 < 2; ++s2) acc[u >> 1] = mfma32<T>(kf[u & 1][s2], dz[2 * (u & 1) + s2], acc[u >> 1]);
           __builtin_amdgcn_sched_barrier(0);
         }
-      }
+      };
+      __syncthreads();  // the positions of the first steps are in LDS
+      static_for<NR - 1>([&](auto e) { fetch(e, decltype(e)::value); });
+      const int nsteps_pad = (nsteps + PADTO - 1) / PADTO * PADTO;
+      for (int step = 0; step < nsteps_pad; step += NR)
+        static_for<NR>([&](auto e) {
+          constexpr int E = decltype(e)::value;
+          __syncthreads();
+          fetch(std::integral_constant<int, (E + NR - 1) % NR>{}, step + E + NR - 1);
+          if (step + E < nsteps) compute(e, step + E);
+        });
       tag_base += nsteps;
     }
     __syncthreads();  // every wave is done with the K tiles: they now hold the output tiles
-
-    // dQ = scale * accumulator, through a per-wave row-major tile
     uint16_t *sOut = reinterpret_cast<uint16_t *>(smem + SM::oK) + (size_t)wave * 32 * LDO;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
@@ -853,7 +859,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a,
             make_uint2(pack2<T>(acc[dt][4 * g] * a.softmax_scale, acc[dt][4 * g + 1] * a.softmax_scale),
                        pack2<T>(acc[dt][4 * g + 2] * a.softmax_scale, acc[dt][4 * g + 3] * a.softmax_scale));
     wave_lds_fence();
-    // rows leave as 16-byte pieces: lane -> (row 4k + lane / 16, features 8 * (lane % 16))
     if ((lane & 15) * 8 < D) {
       uint16_t *op = reinterpret_cast<uint16_t *>(a.dq) + (int64_t)(q0 + m0) * a.dq_row_stride + (int64_t)h * a.dq_head_stride;
 #pragma unroll
