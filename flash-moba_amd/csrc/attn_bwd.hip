@@ -2,7 +2,7 @@
 //
 //   bwd_prep_kernel      : delta[row] = sum_d dO*O (fp32).
 //   attn_bwd_dkdv_kernel : COLUMN-stationary.  One workgroup per (64-key block, head,
-//                          sequence) keeps K and V of the block in LDS and walks the block's
+//                          sequence) keeps K and V of the block in registers and walks the block's
 //                          ascending row list in gathered 32-row tiles:
 //                            S = Q K^T, dP = dO V^T             (A = gathered rows, B = K / V halves)
 //                            P = exp2(S*scale*log2e - LSE*log2e), dS = P o (dP - delta)
@@ -18,10 +18,11 @@
 //   attn_bwd_dq_combine_kernel : dQ from the partials, one wave per (row, head) adds them in ascending
 //                          key-block order and scales.  Work and traffic are proportional to
 //                          the number of visits, whatever the number of chunks per sequence.
-// In the dK/dV kernel half of the waves compute and the other half only move data (global ->
-// registers -> LDS) two rounds ahead of the compute waves.  It runs four waves of 512 registers: a
-// compute wave keeps 32 keys x head_dim of dK^T and dV^T in registers, which does not fit in the 256
-// registers an eight-wave workgroup gets.
+// The dK/dV kernel runs four waves of 512 registers, one per SIMD, and all four compute: two pairs
+// (one wave per 32-key half) that take alternate pairs of tiles and add their sums at the end.  A wave keeps
+// 32 keys x head_dim of dK^T and dV^T plus its K and V operands in registers, which leaves no room for a
+// second wave on the SIMD, so nothing moves data through registers: the gathered Q / dO rows go from global
+// memory straight to LDS (global_load_lds), one round (four tiles) ahead.
 #include "fmoba_common.h"
 
 #include <type_traits>
@@ -29,32 +30,87 @@
 
 namespace fmoba {
 
-constexpr int kListCap = 4096;  // rows of a column list held in LDS at a time
+constexpr int kBwdRoundRows = 128;  // rows of a column list the workgroup takes per round: two 32-row tiles per wave pair
 
 template <int HD>
 struct BwdSmem {
-  // Row stride of the K / V / Q / dO tiles, in elements.  Measured on gfx950 with 16-byte rows-per-lane reads
-  // (lane -> row lane % 32) and the transposing 8-byte reads: HD + 16 runs both at the LDS peak
-  // (8.4 and 4.7 clk per instruction per CU); strides that leave rows 8-byte aligned are 8x slower.
-  static constexpr int LDQ = HD + 16;
-  static constexpr int LDS_ = 32 + 8;  // elements, per-wave dS^T tile [32 keys][32 rows]
-  static constexpr size_t oK = 0;
-  static constexpr size_t oV = oK + (size_t)64 * LDQ * 2;
-  static constexpr size_t oQ = oV + (size_t)64 * LDQ * 2;          // [2 buffers][2 tile slots][32][LDQ]
-  static constexpr size_t odO = oQ + (size_t)4 * 32 * LDQ * 2;
-  static constexpr size_t odS = odO + (size_t)4 * 32 * LDQ * 2;    // [2 tile slots][64 keys][LDS_]: dS^T of both key halves
-  static constexpr int LDH = HD / 2 + 8;                           // elements, per-wave dQ half-row tile [32 rows][LDH]
-  static constexpr size_t odQ = odS + (size_t)2 * 64 * LDS_ * 2;   // [2 waves][32][LDH]
-  static constexpr size_t oSlot = odQ + (size_t)2 * 32 * LDH * 2;  // int[2 buffers][64]
-  static constexpr size_t oRow = oSlot + 4 * 32 * 4;               // int[2 buffers][64]
-  static constexpr size_t oLse = oRow + 4 * 32 * 4;                // LSE * log2(e)
-  static constexpr size_t oDelta = oLse + 4 * 32 * 4;
-  static constexpr size_t oList = oDelta + 4 * 32 * 4;             // int[kListCap]
-  static constexpr size_t mainBytes = oList + (size_t)kListCap * 4;
+  // The gathered Q / dO tiles have rows of exactly HD elements (the loads that fill them write 64 lanes x 16 bytes
+  // to consecutive addresses) and are swizzled instead of padded: the 16-byte piece c of tile row r lies at piece
+  // c ^ bwd_swz<HD>(r).  With that, the 16-byte row reads (lane -> row lane % 32) and the transposing 8-byte
+  // reads both spread over all banks.
+  static constexpr int LDQ = HD + 16;  // elements, K and V while they are read into registers (plain padded rows)
+  static constexpr int LDS_ = 32 + 8;  // elements, dS^T tile rows [key][32 rows]
+  static constexpr size_t tileBytes = (size_t)32 * HD * 2;
+  static constexpr size_t oQ = 0;                                   // [2 buffers][4 tiles][32][HD]
+  static constexpr size_t odO = oQ + 8 * tileBytes;
+  static constexpr size_t odS = odO + 8 * tileBytes;               // partials form: [2 pairs][2 tile slots][64 keys][LDS_]; dS form: [4 waves][32 keys][LDS_]
+  static constexpr int LDH = HD / 2 + 8;                            // elements, per-wave dQ half-row tile [32][LDH]: in a tile that is no longer read
+  static constexpr size_t oRid = odS + (size_t)2 * 2 * 64 * LDS_ * 2;  // int[2 buffers][128]: row ids, one round before the rest
+  static constexpr size_t oRow = oRid + 2 * kBwdRoundRows * 4;     // int[2 buffers][128]
+  static constexpr size_t oSlot = oRow + 2 * kBwdRoundRows * 4;
+  static constexpr size_t oLse = oSlot + 2 * kBwdRoundRows * 4;    // LSE * log2(e)
+  static constexpr size_t oDelta = oLse + 2 * kBwdRoundRows * 4;
+  static constexpr size_t bytes = oDelta + 2 * kBwdRoundRows * 4;
   static constexpr int LDR = HD + 4;  // floats, output transpose buffer [2][64 keys][LDR]
-  static constexpr size_t redBytes = (size_t)2 * 64 * LDR * 4;
-  static constexpr size_t bytes = mainBytes > redBytes ? mainBytes : redBytes;
+  static_assert((size_t)2 * 64 * LDR * 4 <= 16 * tileBytes, "the output buffer reuses the tiles");
+  static_assert((size_t)2 * 64 * LDQ * 2 <= 16 * tileBytes, "K and V pass through the tiles");
+  static_assert((size_t)32 * LDH * 2 <= tileBytes, "a wave's dQ half rows pass through a tile");
+  static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
 };
+
+// piece c of tile row r is stored at piece c ^ bwd_swz<HD>(r)
+template <int HD>
+__device__ __forceinline__ int bwd_swz(int r) {
+  if constexpr (HD > 64)
+    return ((r & 3) << 2) | ((r >> 2) & 3);  // 16 pieces per row, one row per sweep of the banks
+  else
+    return (((r >> 1) & 1) << 2) | ((r >> 2) & 1);  // 8 pieces per row, two rows per sweep
+}
+template <int HD>
+struct BwdSwz {
+  static constexpr int kRow8 = HD > 64 ? 2 : 0;  // bwd_swz(r + 8) ^ bwd_swz(r)
+};
+
+typedef __attribute__((address_space(3))) const Pack8 lds_cpack8;
+__device__ __forceinline__ Pack8 lds_read16(uint32_t byte_addr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return *(lds_cpack8 *)byte_addr;
+#else
+  (void)byte_addr;
+  return Pack8{{0, 0, 0, 0}};
+#endif
+}
+// 8 x 16-bit operand of a transposing read: two 8-byte reads
+__device__ __forceinline__ Pack8 lds_tr8(uint32_t addr_lo, uint32_t addr_hi) {
+  Pack8 r;
+#if defined(__HIP_DEVICE_COMPILE__)
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)addr_lo);
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)addr_hi);
+  __builtin_memcpy(&r.w[0], &lo, 8);
+  __builtin_memcpy(&r.w[2], &hi, 8);
+#else
+  (void)addr_lo, (void)addr_hi;
+  r = Pack8{{0, 0, 0, 0}};
+#endif
+  return r;
+}
+// 64 lanes x 16 bytes from each lane's own global address to LDS bytes [lds_base, lds_base + 1024), lane order;
+// lds_base is the same for the whole wave.  Written as assembly because the compiler makes every later LDS read wait
+// for a load that it knows to write LDS, and these are meant to stay in flight for a whole round: the kernel waits for
+// them itself (wait_all_loads) before the barrier that hands the tiles over.  Nothing else in the kernel uses m0.
+__device__ __forceinline__ void global_to_lds16(const void *g, uint32_t lds_base) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base) : "memory");
+#else
+  (void)g, (void)lds_base;
+#endif
+}
+__device__ __forceinline__ void wait_all_loads() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+}
+__device__ uint4 g_bwd_zero16;  // 16 zero bytes: what the tile loads fetch for absent rows and for features past head_dim
 
 struct BwdWs {
   int32_t *cnt;    // [total_q * heads] visits handed out per (row, head)
@@ -70,17 +126,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   typedef BwdSmem<HD> SM;
   constexpr int KS = HD / 16, LDQ = SM::LDQ, LDS_ = SM::LDS_, NDT = HD / 32, VPR = HD / 8, LDR = SM::LDR, LDH = SM::LDH;
   constexpr int NDH = NDT / 2;  // feature tiles of dQ per compute wave
-  constexpr int NV = 2 * 32 * VPR / 128;  // 16-byte vectors of the two gathered Q (or dO) tiles of a round per loader thread
+  constexpr uint32_t TB = (uint32_t)SM::tileBytes;
+  constexpr int RB = HD * 2;    // bytes of a tile row
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint16_t *sK = reinterpret_cast<uint16_t *>(smem + SM::oK);
-  uint16_t *sV = reinterpret_cast<uint16_t *>(smem + SM::oV);
-  uint16_t *sQ = reinterpret_cast<uint16_t *>(smem + SM::oQ);
-  uint16_t *sdO = reinterpret_cast<uint16_t *>(smem + SM::odO);
+  int *sRid = reinterpret_cast<int *>(smem + SM::oRid);
   int *sRow = reinterpret_cast<int *>(smem + SM::oRow);
   int *sSlot = reinterpret_cast<int *>(smem + SM::oSlot);
   float *sLse = reinterpret_cast<float *>(smem + SM::oLse);
   float *sDelta = reinterpret_cast<float *>(smem + SM::oDelta);
-  int *sList = reinterpret_cast<int *>(smem + SM::oList);
 
   const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + 63) / 64);
   const int nb = item.idx, b = item.pair / a.heads, h = item.pair - b * a.heads;
@@ -92,30 +145,32 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   const int D = a.head_dim;
   const int hk = h / (a.heads / a.heads_k);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
-  const bool is_loader = tid >= 128;
-  const int lt = tid & 127;  // loader thread index
-  const int kh = wave & 1;   // compute wave: key half
+  const int kh = wave & 1;   // key half of this wave
+  const int px = wave >> 1;  // wave pair: takes tiles 2 px and 2 px + 1 of every round
   const bool causal = a.is_causal != 0;
   const float scale_log2 = a.softmax_scale * 1.4426950408889634f;
   constexpr float kLog2e = 1.4426950408889634f;
-  uint16_t *sdS = reinterpret_cast<uint16_t *>(smem + SM::odS);  // + tile slot * 64 * LDS_ + key * LDS_ + row
 
-  // ---- the key block stays in LDS ---------------------------------------------------------
+  // ---- the key block: through LDS into registers.  The loads are issued first and stored after the look-up of
+  // the column list below, so that the two chains of dependent loads wait together (one workgroup per compute
+  // unit: nothing else covers them) ----------------------------------------------
+  constexpr int NKV = 64 * VPR / 256;
+  Pack8 xk[NKV], xv[NKV];
   {
     const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + (int64_t)(k0 + key0) * a.k_row_stride + (int64_t)hk * a.k_head_stride;
     const uint16_t *vp = reinterpret_cast<const uint16_t *>(a.v) + (int64_t)(k0 + key0) * a.v_row_stride + (int64_t)hk * a.v_head_stride;
-    for (int v = tid; v < 64 * VPR; v += 256) {
+#pragma unroll
+    for (int i = 0; i < NKV; ++i) {
+      const int v = tid + 256 * i;
       const int key = v / VPR, e = (v - key * VPR) * 8;
-      Pack8 xk = zero_pack8(), xv = zero_pack8();
+      xk[i] = zero_pack8();
+      xv[i] = zero_pack8();
       if (key0 + key < Lk && e < D) {
-        xk = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
-        xv = ld_global16(vp + (int64_t)key * a.v_row_stride + e);
+        xk[i] = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
+        xv[i] = ld_global16(vp + (int64_t)key * a.v_row_stride + e);
       }
-      *reinterpret_cast<Pack8 *>(sK + key * LDQ + e) = xk;
-      *reinterpret_cast<Pack8 *>(sV + key * LDQ + e) = xv;
     }
   }
-  __syncthreads();
 
   // ---- this block's column list --------------------------------------------------------------
   const int Bn = a.lg_block_n;
@@ -128,414 +183,447 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     nnz = a.col_nnz[bh * a.max_cols + c];
     lbase = a.col_offsets[bh * a.max_cols + c];
     // rows r with r + off < key0 see no key of this block
-    if (causal && nnz > 0) start = lower_bound_i32(a.row_indices + lbase, nnz, key0 - off);
+    if (causal && nnz > 0) start = lower_bound_wave_i32(a.row_indices + lbase, nnz, key0 - off);
   }
-  const int32_t *list = a.row_indices + lbase;
+  const int32_t *list = a.row_indices + lbase + start;
+  const int n = nnz - start;               // rows of the list that the block walks
+  const int nround = (n + kBwdRoundRows - 1) / kBwdRoundRows;
   const int koff = key0 - c * Bn;  // offset of this 64-key block inside its column
+  int rid01[2] = {-1, -1};         // threads 0..127: row ids of rounds 0 and 1
+  if (tid < kBwdRoundRows && n > 0) {
+#pragma unroll
+    for (int sr = 0; sr < 2; ++sr) {
+      const int j = sr * kBwdRoundRows + tid;
+      const int r = list[min(j, n - 1)];
+      rid01[sr] = ((j < n) & (r >= 0) & (r < Lq)) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
+    }
+  }
+
+  {
+    uint16_t *sK = reinterpret_cast<uint16_t *>(smem), *sV = sK + 64 * LDQ;
+#pragma unroll
+    for (int i = 0; i < NKV; ++i) {
+      const int v = tid + 256 * i;
+      const int key = v / VPR, e = (v - key * VPR) * 8;
+      *reinterpret_cast<Pack8 *>(sK + key * LDQ + e) = xk[i];
+      *reinterpret_cast<Pack8 *>(sV + key * LDQ + e) = xv[i];
+    }
+  }
+  __syncthreads();
+  // B operands of S and dP: this lane's key, its half of the head dim; K^T of this wave's half of the features for
+  // the dQ products.  They never change, so they stay in registers.
+  Pack8 kb[KS], vb[KS];
+  Pack8 kt[NDH][4];
+  {
+    const uint16_t *sK = reinterpret_cast<const uint16_t *>(smem), *sV = sK + 64 * LDQ;
+#pragma unroll
+    for (int t = 0; t < KS; ++t) {
+      kb[t] = *reinterpret_cast<const Pack8 *>(sK + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
+      vb[t] = *reinterpret_cast<const Pack8 *>(sV + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
+    }
+    if constexpr (DQP) {
+      lds_cu16 *trK = tr_lane_base(sK, LDQ, lane) + 8 * hh * LDQ;
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+        for (int d2 = 0; d2 < NDH; ++d2) {
+          const int lo = 16 * s4 * LDQ + (kh * NDH + d2) * 32;
+          kt[d2][s4] = tr_frag8_at(trK, lo, lo + 4 * LDQ);
+        }
+    }
+  }
 
   const uint16_t *qg = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)q0 * a.q_row_stride + (int64_t)h * a.q_head_stride;
   const uint16_t *dog = reinterpret_cast<const uint16_t *>(a.dout) + (int64_t)q0 * a.do_row_stride + (int64_t)h * a.do_head_stride;
   const float *lseg = a.softmax_lse + (int64_t)h * a.total_q + q0;
   const float *delg = a.softmax_d + (int64_t)h * ((int64_t)a.total_q + 128 * (int64_t)a.batch) + q0 + 128 * b;
   int32_t *cntg = ws.cnt + (int64_t)q0 * a.heads + h;  // counter of local row r: cntg[r * heads]
-
-  auto fill_list = [&](int seg0, int seg_len) {
-    __syncthreads();
-    for (int i = tid; i < seg_len; i += 256) {
-      int r = list[seg0 + i];
-      sList[i] = (r >= 0 && r < Lq) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
-    }
-    __syncthreads();
-  };
   float *red = reinterpret_cast<float *>(smem);  // [2][64 keys][LDR]: dV^T, dK^T on their way out
 
-  // The two roles run separate code with the same barrier sequence, so that the loaders' rings and the
-  // compute waves' accumulators and operands do not add up in the register allocation.
-  if (is_loader) {
-    // two-deep rings (compile-time parity) of the gathered rows of two rounds.  Loads are unconditional
-    // (indices clamped, the surplus zeroed when stored) so that the compiler counts outstanding loads exactly.
-    typedef std::integral_constant<int, 0> P0;
-    typedef std::integral_constant<int, 1> P1;
-    Pack8 lq[2][NV], ld[2][NV];
-    int lrow[2] = {-1, -1}, lslot[2] = {0, 0};
-    float llse[2] = {INFINITY, INFINITY}, ldel[2] = {0.f, 0.f};
-
-    for (int seg0 = start; seg0 < nnz; seg0 += kListCap) {
-      const int seg_len = min(kListCap, nnz - seg0);
-      fill_list(seg0, seg_len);
-      const int nround = (seg_len + 63) >> 6;
-      auto load_round = [&](auto par, int r) {
-        constexpr int P = decltype(par)::value;
+  f32x16 dv[NDT], dk[NDT];
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-          const int v = lt + 128 * i;
-          const int row = v / VPR, e = min((v - row * VPR) * 8, D - 8);  // row 0..63 over the two tiles of the round
-          const int rid = max(sList[min(r * 64 + row, seg_len - 1)], 0);
-          lq[P][i] = ld_global16(qg + (int64_t)rid * a.q_row_stride + e);
-          ld[P][i] = ld_global16(dog + (int64_t)rid * a.do_row_stride + e);
-        }
-        if (lt < 64) {
-          const int j = r * 64 + lt;
-          const int rid = j < seg_len ? sList[j] : -1;
-          const int rc = max(rid, 0);
-          lrow[P] = rid;
-          llse[P] = lseg[rc];
-          ldel[P] = delg[rc];
-          // every visit of a (row, key block) pair takes one dQ-partial slot of the row (the only conditional
-          // memory operation of the loader)
-          if constexpr (DQP) {
-            if (rid >= 0) lslot[P] = atomicAdd(cntg + (int64_t)rid * a.heads, 1);
-          }
-        }
-      };
-      auto store_round = [&](auto par, int r) {
-        constexpr int P = decltype(par)::value;
+  for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-          const int v = lt + 128 * i;
-          const int row = v / VPR, e = (v - row * VPR) * 8;
-          const int j = r * 64 + row;
-          const bool ok = (e < D) & (j < seg_len) & (sList[min(j, seg_len - 1)] >= 0);
-          Pack8 xq = lq[P][i], xo = ld[P][i];
-#pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            xq.w[w] = ok ? xq.w[w] : 0u;
-            xo.w[w] = ok ? xo.w[w] : 0u;
-          }
-          *reinterpret_cast<Pack8 *>(sQ + (P * 64 + row) * LDQ + e) = xq;
-          *reinterpret_cast<Pack8 *>(sdO + (P * 64 + row) * LDQ + e) = xo;
-        }
-        if (lt < 64) {
-          const bool ok = lrow[P] >= 0;
-          sRow[P * 64 + lt] = lrow[P];
-          sSlot[P * 64 + lt] = lslot[P];
-          sLse[P * 64 + lt] = ok ? llse[P] * kLog2e : INFINITY;  // absent rows: exp2(x - inf) = 0
-          sDelta[P * 64 + lt] = ok ? ldel[P] : 0.f;
-        }
-      };
-
-      // Tiles are double buffered in LDS by round parity, and so are the rings: during round r the loaders
-      // put round r+1 into the other buffer and fetch round r+3 into the registers that this frees.
-      load_round(P0{}, 0);
-      load_round(P1{}, 1);  // past the end: rows clamp to the last one, nothing of it is used
-      store_round(P0{}, 0);
-      load_round(P0{}, 2);
-      auto loader_round = [&](auto par, int r) {  // par: parity of round r + 1
-        // The compute waves exchange dS^T of the round's two tiles through LDS, which takes one more
-        // barrier per round.
-        __syncthreads();  // round r is in LDS; the readers of round r-1 are done with the other buffer
-        if (r + 1 < nround) store_round(par, r + 1);
-        load_round(par, r + 3);
-        if constexpr (DQP) __syncthreads();
-      };
-      const int nround_pad = (nround + 1) & ~1;
-      for (int r = 0; r < nround_pad; r += 2) {
-        loader_round(P1{}, r);
-        loader_round(P0{}, r + 1);
-      }
+    for (int i = 0; i < 16; ++i) {
+      dv[dt][i] = 0.f;
+      dk[dt][i] = 0.f;
     }
-    __syncthreads();
-  } else {
-    f32x16 dv[NDT], dk[NDT];
-  #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
-  #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        dv[dt][i] = 0.f;
-        dk[dt][i] = 0.f;
-      }
 
-    for (int seg0 = start; seg0 < nnz; seg0 += kListCap) {
-      const int seg_len = min(kListCap, nnz - seg0);
-      fill_list(seg0, seg_len);
-      const int ntile = (seg_len + 31) >> 5;
-      const int nround = (ntile + 1) >> 1;
-      // ---- compute-wave stages ---------------------------------------------------------------------
-      // A compute wave is alone on its SIMD, so the MFMA pipe only stays busy if the softmax arithmetic
-      // of one tile runs between the products of the other tile of the round.  Every stage is cut into
-      // four chunks (a quarter of the products + a quarter of the softmax rows); the operands of chunk
-      // g+1 are read from LDS while chunk g computes, and the scheduler is fenced between chunks: left
-      // alone, the compiler sinks every read next to the MFMA that uses it and waits for it there.
-      typedef std::integral_constant<int, 0> C0;
-      typedef std::integral_constant<int, 1> C1;
-      constexpr int KC = KS / 4;       // k-steps of S / dP per chunk
-      constexpr int BC = NDT / 2;      // (d-tile, row-half) operand pairs of dV / dK per chunk
-      lds_cu16 *trQ = tr_lane_base(sQ, LDQ, lane) + 4 * hh * LDQ, *trdO = tr_lane_base(sdO, LDQ, lane) + 4 * hh * LDQ;
-      lds_cu16 *trdS = tr_lane_base(sdS, LDS_, lane) + 8 * hh * LDS_;  // dS^T tile: 8 consecutive keys per read
-      lds_cu16 *trK = tr_lane_base(sK, LDQ, lane) + 8 * hh * LDQ;      // K^T with the same key order
-      uint16_t *sdQ = reinterpret_cast<uint16_t *>(smem + SM::odQ) + (size_t)kh * 32 * LDH;
-      Pack8 qa[2][KC], doa[2][KC];     // A operands of S and dP (this lane's row, its half of the head dim), double-buffered by chunk
-      // B operands of S and dP: this lane's key, its half of the head dim; they never change, so they stay in registers
-      Pack8 kb[KS], vb[KS];
-#pragma unroll
-      for (int t = 0; t < KS; ++t) {
-        kb[t] = *reinterpret_cast<const Pack8 *>(sK + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
-        vb[t] = *reinterpret_cast<const Pack8 *>(sV + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
+  if (nround > 0) {
+    // ---- feeding the tiles --------------------------------------------------------------------------
+    // Nothing passes through registers: every wave fetches one of the four tiles of the NEXT round with loads that
+    // write straight to LDS, issued at the start of a round and awaited at its end.  Threads 0..127 carry the
+    // per-row scalars: the row id of round s+2 (it has to be in LDS one round before the tile loads that use it),
+    // and LSE, delta and the dQ-partial slot of round s+1.
+    const uint32_t ldsQ = (uint32_t)(uintptr_t)(smem + SM::oQ), ldsdO = (uint32_t)(uintptr_t)(smem + SM::odO);
+    int n_rid = -1, m_rid = -1, m_slot = 0;
+    float m_lse = 0.f, m_del = 0.f;
+    int ft = tid;  // thread index for the feeding code, re-made opaque in every round (see below)
+    auto rid_issue = [&](int sr) {
+      if (tid < kBwdRoundRows) {
+        const int j = sr * kBwdRoundRows + ft;
+        const int r = list[min(j, n - 1)];
+        n_rid = ((j < n) & (r >= 0) & (r < Lq)) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
       }
-      Pack8 dot[2][BC], qt[2][BC];     // dO^T / Q^T operands of the dV / dK products, double-buffered by chunk
-      f32x4 lse4[2], del4[2];          // softmax inputs of a chunk's four rows
-      int4 row4[2];
-      Pack8 pf[2][2], dsf[2][2];       // P and dS of both tiles of the round as MFMA operands
-      Pack8 dsx[4];                    // dS^T of all 64 keys as the B operand of the dQ products
-      Pack8 kt[NDH][4];                // K^T of this wave's half of the features: never changes, stays in registers
-      if constexpr (DQP) {
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4)
-#pragma unroll
-          for (int d2 = 0; d2 < NDH; ++d2) {
-            const int lo = 16 * s4 * LDQ + (kh * NDH + d2) * 32;
-            kt[d2][s4] = tr_frag8_at(trK, lo, lo + 4 * LDQ);
-          }
-      }
-      f32x16 dqa[NDH];
-      f32x16 s[2], dp[2];
-      auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
-      auto ld_a = [&](auto pc, auto tsc, auto gc) {
-        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value, G = decltype(gc)::value;
-        const uint16_t *tQ = sQ + TS * 32 * LDQ, *tdO = sdO + TS * 32 * LDQ;
-  #pragma unroll
-        for (int t = 0; t < KC; ++t) {
-          qa[G & 1][t] = *reinterpret_cast<const Pack8 *>(tQ + (lane & 31) * LDQ + (hh * KS + G * KC + t) * 8);
-          doa[G & 1][t] = *reinterpret_cast<const Pack8 *>(tdO + (lane & 31) * LDQ + (hh * KS + G * KC + t) * 8);
-        }
-      };
-      auto mm_a = [&](auto tsc, auto gc) {
-        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
-        if constexpr (G == 0) {
-  #pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            s[TS][i] = 0.f;
-            dp[TS][i] = 0.f;
-          }
-        }
-  #pragma unroll
-        for (int t = 0; t < KC; ++t) {
-          s[TS] = mfma32<T>(qa[G & 1][t], kb[G * KC + t], s[TS]);
-          dp[TS] = mfma32<T>(doa[G & 1][t], vb[G * KC + t], dp[TS]);
-        }
-      };
-      auto ld_b = [&](auto pc, auto tsc, auto gc) {
-        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value, G = decltype(gc)::value;
-  #pragma unroll
-        for (int t = 0; t < BC; ++t) {
-          const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
-          const int lo = (TS * 32 + 16 * s2) * LDQ + dt * 32, hi = lo + 8 * LDQ;
-          dot[G & 1][t] = tr_frag8_at(trdO, lo, hi);
-          qt[G & 1][t] = tr_frag8_at(trQ, lo, hi);
-        }
-      };
-      auto mm_b = [&](auto tsc, auto gc) {
-        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
-        // dV^T[d][key] += dO^T[d][row] P[row][key];  dK^T[d][key] += Q^T[d][row] dS[row][key]
-  #pragma unroll
-        for (int t = 0; t < BC; ++t) {
-          const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
-          dv[dt] = mfma32<T>(dot[G & 1][t], pf[TS][s2], dv[dt]);
-          dk[dt] = mfma32<T>(qt[G & 1][t], dsf[TS][s2], dk[dt]);
-        }
-      };
-      // this lane's key; key j is visible to row r iff r >= row_thr (rows that do not exist are stored as -1)
-      const int j = key0 + kh * 32 + (lane & 31);
-      const int row_thr = j >= Lk ? 0x7fffffff : (causal ? max(0, j - off) : 0);
-      auto ld_s = [&](auto pc, auto tsc, auto gc) {
-        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value, G = decltype(gc)::value;
-        const int base = TS * 32 + 8 * G + 4 * hh;  // accumulator registers 4G..4G+3 hold rows base..base+3
-        lse4[G & 1] = *reinterpret_cast<const f32x4 *>(sLse + base);
-        del4[G & 1] = *reinterpret_cast<const f32x4 *>(sDelta + base);
-        row4[G & 1] = *reinterpret_cast<const int4 *>(sRow + base);
-      };
-      auto smx = [&](auto tsc, auto gc) {
-        constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
-        const int rr[4] = {row4[G & 1].x, row4[G & 1].y, row4[G & 1].z, row4[G & 1].w};
-        float pr[4], ds[4];
-  #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          const int i = 4 * G + jj;
-          const float x = rr[jj] >= row_thr ? fmaf(s[TS][i], scale_log2, -lse4[G & 1][jj]) : -INFINITY;
-          pr[jj] = __builtin_amdgcn_exp2f(x);
-          ds[jj] = pr[jj] * (dp[TS][i] - del4[G & 1][jj]);
-        }
-        // operand register s2 = G/2 holds rows 16*s2 + 8*(w/2) + 4*hh + ..: words 2*(G%2), 2*(G%2)+1
-        pf[TS][G >> 1].w[2 * (G & 1)] = pack2<T>(pr[0], pr[1]);
-        pf[TS][G >> 1].w[2 * (G & 1) + 1] = pack2<T>(pr[2], pr[3]);
-        dsf[TS][G >> 1].w[2 * (G & 1)] = pack2<T>(ds[0], ds[1]);
-        dsf[TS][G >> 1].w[2 * (G & 1) + 1] = pack2<T>(ds[2], ds[3]);
-      };
-      // dQ of the tile: both waves put dS^T of their 32 keys into one LDS tile [64 keys][32 rows]; after a
-      // barrier each wave computes dQ^T = K^T dS^T over all 64 keys for ITS half of the features (K^T and
-      // dS^T through transposing reads, which exchange data between lanes: every lane takes part).  The
-      // half rows (16-bit, unscaled) go to the partial slot that the row handed out for this visit.
-      auto ds_write = [&](auto tsc) {
-        constexpr int TS = decltype(tsc)::value;
-        // DQP: tile slot TS, rows of both key halves; else: this wave's private half of tile slot 0
-        uint16_t *t = sdS + (size_t)((DQP ? TS * 64 : 0) + kh * 32 + (lane & 31)) * LDS_;
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          *reinterpret_cast<uint2 *>(t + 16 * s2 + 4 * hh) = make_uint2(dsf[TS][s2].w[0], dsf[TS][s2].w[1]);
-          *reinterpret_cast<uint2 *>(t + 16 * s2 + 8 + 4 * hh) = make_uint2(dsf[TS][s2].w[2], dsf[TS][s2].w[3]);
-        }
-        if constexpr (!DQP) wave_lds_fence();  // (the partials form waits for both key halves at a workgroup barrier later)
-      };
-      // dS form: the wave's 32 keys of every row go to the dS tile of the row's list entry
-      int dsrow = -1;
-      auto ds_read = [&](auto pc, auto tsc) {
-        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value;
-        dsrow = sRow[TS * 32 + (lane & 31)];
-#pragma unroll
-        for (int s4 = 0; s4 < 2; ++s4) dsx[s4] = tr_frag8_at(trdS, (kh * 32 + 16 * s4) * LDS_, (kh * 32 + 16 * s4 + 4) * LDS_);
-        wave_lds_fence();
-      };
-      auto ds_store = [&](int tile) {
-        if (dsrow >= 0) {
-          uint16_t *wp = ws.ds + (lbase + seg0 + tile * 32 + (lane & 31)) * Bn + koff + kh * 32;
-#pragma unroll
-          for (int s4 = 0; s4 < 2; ++s4) *reinterpret_cast<Pack8 *>(wp + 16 * s4 + 8 * hh) = dsx[s4];
-        }
-      };
-      auto dq_load = [&](auto tsc) {
-        constexpr int TS = decltype(tsc)::value;
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) dsx[s4] = tr_frag8_at(trdS, (TS * 64 + 16 * s4) * LDS_, (TS * 64 + 16 * s4 + 4) * LDS_);
-      };
-      auto dq_mma = [&](auto gc) {  // a quarter of the products per chunk
-        constexpr int G = decltype(gc)::value;
-#pragma unroll
-        for (int d2 = 0; d2 < NDH; ++d2) {
-          if constexpr (G == 0) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) dqa[d2][i] = 0.f;
-          }
-          dqa[d2] = mfma32<T>(kt[d2][G], dsx[G], dqa[d2]);
-        }
-      };
-      const int64_t trash = (int64_t)a.total_q * a.heads * ws.cap;  // spare row: takes the writes of absent rows, no branch
-      auto dq_store = [&](auto pc, auto tsc) {
-        constexpr int TS = decltype(pc)::value * 2 + decltype(tsc)::value;
-        // register i of feature tile d2 <-> feature d2*32 + acc_row(i, hh) of this wave's half, this lane's row
-#pragma unroll
-        for (int d2 = 0; d2 < NDH; ++d2)
-#pragma unroll
-          for (int g = 0; g < 4; ++g)
-            *reinterpret_cast<uint2 *>(sdQ + (lane & 31) * LDH + d2 * 32 + 8 * g + 4 * hh) =
-                make_uint2(pack2<T>(dqa[d2][4 * g], dqa[d2][4 * g + 1]), pack2<T>(dqa[d2][4 * g + 2], dqa[d2][4 * g + 3]));
-        wave_lds_fence();
-        constexpr int LPR = HD / 16;        // lanes per half row (16 bytes each)
-        constexpr int RPP = 64 / LPR;       // rows per pass
-        const int col = (lane % LPR) * 8;
-#pragma unroll
-        for (int k = 0; k < 32 / RPP; ++k) {
-          const int row = k * RPP + lane / LPR;
-          const int r2 = sRow[TS * 32 + row], s2 = sSlot[TS * 32 + row];
-          const Pack8 x = *reinterpret_cast<const Pack8 *>(sdQ + row * LDH + col);
-          const bool ok = (r2 >= 0) & (s2 < ws.cap);
-          const int64_t pidx = ok ? ((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2 : trash;
-          if (kh * (HD / 2) + col < D) *reinterpret_cast<Pack8 *>(ws.part + pidx * D + kh * (HD / 2) + col) = x;
-          if (kh == 0 && col == 0) ws.pid[pidx] = nb;
-        }
-        wave_lds_fence();
-      };
-      // One round = tiles 2r and 2r+1, both already in LDS.  A list with an odd number of tiles ends with a tile
-      // of absent rows (row id -1, zero data): it runs through the same code and adds nothing.
-      auto process_round = [&](auto pc, int r) {  // pc: parity of r = the LDS buffer that holds the round
-        // S, dP of the first tile
-        ld_a(pc, C0{}, C0{});
-        fence();
-        static_for<4>([&](auto gc) {
-          constexpr int G = decltype(gc)::value;
-          if constexpr (G < 3) ld_a(pc, C0{}, std::integral_constant<int, G + 1>{});
-          mm_a(C0{}, gc);
-          fence();
-        });
-        // S, dP of the second tile between the softmax rows of the first
-        ld_a(pc, C1{}, C0{});
-        ld_s(pc, C0{}, C0{});
-        fence();
-        static_for<4>([&](auto gc) {
-          constexpr int G = decltype(gc)::value;
-          if constexpr (G < 3) {
-            ld_a(pc, C1{}, std::integral_constant<int, G + 1>{});
-            ld_s(pc, C0{}, std::integral_constant<int, G + 1>{});
-          }
-          mm_a(C1{}, gc);
-          smx(C0{}, gc);
-          fence();
-        });
-        // dV, dK of the first tile between the softmax rows of the second
-        ds_write(C0{});
-        ld_b(pc, C0{}, C0{});
-        ld_s(pc, C1{}, C0{});
-        if constexpr (!DQP) ds_read(pc, C0{});
-        fence();
-        static_for<4>([&](auto gc) {
-          constexpr int G = decltype(gc)::value;
-          if constexpr (G < 3) {
-            ld_b(pc, C0{}, std::integral_constant<int, G + 1>{});
-            ld_s(pc, C1{}, std::integral_constant<int, G + 1>{});
-          }
-          mm_b(C0{}, gc);
-          smx(C1{}, gc);
-          if constexpr (!DQP && G == 1) ds_store(2 * r);
-          fence();
-        });
-        // dV, dK of the second tile; in the partials form dQ of the first one runs between them: by now both key
-        // halves have put dS^T of both tiles into LDS, so the one barrier the exchange needs hardly ever waits
-        ds_write(C1{});
-        if constexpr (DQP) __syncthreads();
-        ld_b(pc, C1{}, C0{});
-        if constexpr (DQP)
-          dq_load(C0{});
-        else
-          ds_read(pc, C1{});
-        fence();
-        static_for<4>([&](auto gc) {
-          constexpr int G = decltype(gc)::value;
-          if constexpr (G < 3) ld_b(pc, C1{}, std::integral_constant<int, G + 1>{});
-          mm_b(C1{}, gc);
-          if constexpr (DQP) dq_mma(gc);
-          if constexpr (!DQP && G == 1) ds_store(2 * r + 1);
-          fence();
-        });
+    };
+    auto rid_store = [&](int sr) {
+      if (tid < kBwdRoundRows) sRid[(sr & 1) * kBwdRoundRows + ft] = n_rid;
+    };
+    auto meta_issue = [&](int sr) {
+      if (tid < kBwdRoundRows) {
+        m_rid = sRid[(sr & 1) * kBwdRoundRows + ft];
+        const int rc = max(m_rid, 0);
+        m_lse = lseg[rc];
+        m_del = delg[rc];
+        // every visit of a (row, key block) pair takes one dQ-partial slot of the row
         if constexpr (DQP) {
-          dq_store(pc, C0{});
-          // dQ of the second tile
-          dq_load(C1{});
-          fence();
-          static_for<4>([&](auto gc) {
-            dq_mma(gc);
-            fence();
-          });
-          dq_store(pc, C1{});
-        }
-      };
-
-      const int nround_pad = (nround + 1) & ~1;
-      for (int r = 0; r < nround_pad; r += 2) {
-        __syncthreads();  // round r is in LDS
-        process_round(C0{}, r);
-        __syncthreads();
-        if (r + 1 < nround) {
-          process_round(C1{}, r + 1);
-        } else if constexpr (DQP) {  // padding round: only the barrier
-          __syncthreads();
+          if (m_rid >= 0) m_slot = atomicAdd(cntg + (int64_t)m_rid * a.heads, 1);
         }
       }
+    };
+    auto meta_store = [&](int sr) {
+      if (tid < kBwdRoundRows) {
+        const int i = (sr & 1) * kBwdRoundRows + ft;
+        const bool ok = m_rid >= 0;
+        sRow[i] = m_rid;
+        sSlot[i] = m_slot;
+        sLse[i] = ok ? m_lse * kLog2e : INFINITY;  // absent rows: exp2(x - inf) = 0
+        sDelta[i] = ok ? m_del : 0.f;
+      }
+    };
+    auto tile_issue = [&](int sr) {  // tile `wave` of round sr
+      constexpr int RPI = 64 / VPR, NI = 32 / RPI;  // tile rows per instruction, instructions per tile
+      const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
+      const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(((sr & 1) * 4 + wave) * (int)TB);
+      const uint16_t *zero = reinterpret_cast<const uint16_t *>(&g_bwd_zero16);
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int row = i * RPI + rl;
+        const int rid = sRid[(sr & 1) * kBwdRoundRows + wave * 32 + row];
+        const int e = (p ^ bwd_swz<HD>(row)) * 8;
+        const bool ok = (rid >= 0) & (e < D);
+        const uint16_t *gq = ok ? qg + (int64_t)rid * a.q_row_stride + e : zero;
+        const uint16_t *gd = ok ? dog + (int64_t)rid * a.do_row_stride + e : zero;
+        global_to_lds16(gq, ldsQ + dst + (uint32_t)(i * RPI * RB));
+        global_to_lds16(gd, ldsdO + dst + (uint32_t)(i * RPI * RB));
+      }
+    };
+
+    if (tid < kBwdRoundRows) {
+      sRid[tid] = rid01[0];
+      sRid[kBwdRoundRows + tid] = rid01[1];
     }
-    __syncthreads();  // every wave is done with the tiles: the output buffer may overwrite them
+    __syncthreads();  // K, V are in registers; the row ids of rounds 0 and 1 are in LDS
+    meta_issue(0);
+    tile_issue(0);
+    meta_store(0);
+    wait_all_loads();
+    __syncthreads();
+
+    // ---- compute-wave stages ---------------------------------------------------------------------
+    // A wave is alone on its SIMD, so the MFMA pipe only stays busy if the softmax arithmetic
+    // of one tile runs between the products of the other tile of the round.  Every stage is cut into
+    // four chunks (a quarter of the products + a quarter of the softmax rows); the operands of chunk
+    // g+1 are read from LDS while chunk g computes, and the scheduler is fenced between chunks: left
+    // alone, the compiler sinks every read next to the MFMA that uses it and waits for it there.
+    typedef std::integral_constant<int, 0> C0;
+    typedef std::integral_constant<int, 1> C1;
+    constexpr int KC = KS / 4;       // k-steps of S / dP per chunk
+    constexpr int BC = NDT / 2;      // (d-tile, row-half) operand pairs of dV / dK per chunk
+    // byte addresses of this lane's pieces in tile 0 of the pair, buffer 0: row reads (row lane % 32, pieces
+    // hh * KS ..) and transposing reads (row (lane % 16) / 4 + 4 hh, feature tile 0); every other operand is an
+    // exclusive-or on the piece bits plus a constant
+    const uint32_t pairQ = ldsQ + (uint32_t)(px * 2) * TB, pairdO = ldsdO + (uint32_t)(px * 2) * TB;
+    const uint32_t rowoff = (uint32_t)((lane & 31) * RB + (((hh * KS) ^ bwd_swz<HD>(lane & 31)) * 16));
+    const int li = lane & 15, r0t = (li >> 2) + 4 * hh;
+    const uint32_t troff = (uint32_t)(r0t * RB + ((((((lane >> 4) & 1) * 2 + ((li & 3) >> 1))) ^ bwd_swz<HD>(r0t)) * 16) + (li & 1) * 8);
+    // (re-made opaque in every round: the operand addresses derived from them must not be kept in registers
+    // across rounds, there are none to spare)
+    uint32_t aQ = pairQ + rowoff, adO = pairdO + rowoff, tQ = pairQ + troff, tdO = pairdO + troff;
+    uint16_t *sdS = reinterpret_cast<uint16_t *>(smem + SM::odS) + (DQP ? (size_t)px * 2 * 64 * LDS_ : (size_t)wave * 32 * LDS_);
+    lds_cu16 *trdS = tr_lane_base(sdS, LDS_, lane) + 8 * hh * LDS_;  // dS^T tile: 8 consecutive keys per read
+    // the dQ half rows of a tile leave through the first tile of the pair, which nobody reads after the barrier in
+    // the middle of the round: Q's for the first key half, dO's for the second
+    uint16_t *sdQ0 = reinterpret_cast<uint16_t *>(smem + (kh ? SM::odO : SM::oQ) + (size_t)(px * 2) * TB);
+    const int *pRow = sRow + px * 64, *pSlot = sSlot + px * 64;
+    const float *pLse = sLse + px * 64, *pDelta = sDelta + px * 64;
+    Pack8 qa[2][KC], doa[2][KC];     // A operands of S and dP (this lane's row, its half of the head dim), double-buffered by chunk
+    Pack8 dot[2][BC], qt[2][BC];     // dO^T / Q^T operands of the dV / dK products, double-buffered by chunk
+    f32x4 lse4[2], del4[2];          // softmax inputs of a chunk's four rows
+    int4 row4[2];
+    Pack8 pf[2][2], dsf[2][2];       // P and dS of both tiles of the round as MFMA operands
+    Pack8 dsx[4];                    // dS^T of all 64 keys as the B operand of the dQ products
+    f32x16 dqa[NDH];
+    f32x16 s[2], dp[2];
+    auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+    auto ld_a = [&](auto pc, auto tsc, auto gc) {
+      constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(tsc)::value) * TB;
+      constexpr int G = decltype(gc)::value;
+#pragma unroll
+      for (int t = 0; t < KC; ++t) {
+        qa[G & 1][t] = lds_read16((aQ ^ (uint32_t)((G * KC + t) * 16)) + TO);
+        doa[G & 1][t] = lds_read16((adO ^ (uint32_t)((G * KC + t) * 16)) + TO);
+      }
+    };
+    auto mm_a = [&](auto tsc, auto gc) {
+      constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+      if constexpr (G == 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          s[TS][i] = 0.f;
+          dp[TS][i] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < KC; ++t) {
+        s[TS] = mfma32<T>(qa[G & 1][t], kb[G * KC + t], s[TS]);
+        dp[TS] = mfma32<T>(doa[G & 1][t], vb[G * KC + t], dp[TS]);
+      }
+    };
+    auto ld_b = [&](auto pc, auto tsc, auto gc) {
+      constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(tsc)::value) * TB;
+      constexpr int G = decltype(gc)::value;
+#pragma unroll
+      for (int t = 0; t < BC; ++t) {
+        const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
+        // rows 16 s2 + (0..3) + 4 hh and the same + 8, features dt * 32 ..
+        const uint32_t xlo = (uint32_t)(dt * 4 * 16), xhi = (uint32_t)(((dt * 4) ^ BwdSwz<HD>::kRow8) * 16);
+        const uint32_t olo = TO + (uint32_t)(16 * s2 * RB), ohi = olo + (uint32_t)(8 * RB);
+        dot[G & 1][t] = lds_tr8((tdO ^ xlo) + olo, (tdO ^ xhi) + ohi);
+        qt[G & 1][t] = lds_tr8((tQ ^ xlo) + olo, (tQ ^ xhi) + ohi);
+      }
+    };
+    auto mm_b = [&](auto tsc, auto gc) {
+      constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+      // dV^T[d][key] += dO^T[d][row] P[row][key];  dK^T[d][key] += Q^T[d][row] dS[row][key]
+#pragma unroll
+      for (int t = 0; t < BC; ++t) {
+        const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
+        dv[dt] = mfma32<T>(dot[G & 1][t], pf[TS][s2], dv[dt]);
+        dk[dt] = mfma32<T>(qt[G & 1][t], dsf[TS][s2], dk[dt]);
+      }
+    };
+    // this lane's key; key j is visible to row r iff r >= row_thr (rows that do not exist are stored as -1)
+    const int j = key0 + kh * 32 + (lane & 31);
+    const int row_thr = j >= Lk ? 0x7fffffff : (causal ? max(0, j - off) : 0);
+    auto ld_s = [&](auto pc, auto tsc, auto gc) {
+      constexpr int TS = decltype(pc)::value * 4 + decltype(tsc)::value, G = decltype(gc)::value;
+      const int base = TS * 32 + 8 * G + 4 * hh;  // accumulator registers 4G..4G+3 hold rows base..base+3
+      lse4[G & 1] = *reinterpret_cast<const f32x4 *>(pLse + base);
+      del4[G & 1] = *reinterpret_cast<const f32x4 *>(pDelta + base);
+      row4[G & 1] = *reinterpret_cast<const int4 *>(pRow + base);
+    };
+    auto smx = [&](auto tsc, auto gc) {
+      constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
+      const int rr[4] = {row4[G & 1].x, row4[G & 1].y, row4[G & 1].z, row4[G & 1].w};
+      float pr[4], ds[4];
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const int i = 4 * G + jj;
+        const float x = rr[jj] >= row_thr ? fmaf(s[TS][i], scale_log2, -lse4[G & 1][jj]) : -INFINITY;
+        pr[jj] = __builtin_amdgcn_exp2f(x);
+        ds[jj] = pr[jj] * (dp[TS][i] - del4[G & 1][jj]);
+      }
+      // operand register s2 = G/2 holds rows 16*s2 + 8*(w/2) + 4*hh + ..: words 2*(G%2), 2*(G%2)+1
+      pf[TS][G >> 1].w[2 * (G & 1)] = pack2<T>(pr[0], pr[1]);
+      pf[TS][G >> 1].w[2 * (G & 1) + 1] = pack2<T>(pr[2], pr[3]);
+      dsf[TS][G >> 1].w[2 * (G & 1)] = pack2<T>(ds[0], ds[1]);
+      dsf[TS][G >> 1].w[2 * (G & 1) + 1] = pack2<T>(ds[2], ds[3]);
+    };
+    // dQ of the tile: both waves of a pair put dS^T of their 32 keys into one LDS tile [64 keys][32 rows]; after a
+    // barrier each wave computes dQ^T = K^T dS^T over all 64 keys for ITS half of the features.  The
+    // half rows (16-bit, unscaled) go to the partial slot that the row handed out for this visit.
+    auto ds_write = [&](auto tsc) {
+      constexpr int TS = decltype(tsc)::value;
+      // partials form: tile slot TS of the pair, rows of both key halves; else: this wave's private tile
+      uint16_t *t = sdS + (size_t)((DQP ? TS * 64 + kh * 32 : 0) + (lane & 31)) * LDS_;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        *reinterpret_cast<uint2 *>(t + 16 * s2 + 4 * hh) = make_uint2(dsf[TS][s2].w[0], dsf[TS][s2].w[1]);
+        *reinterpret_cast<uint2 *>(t + 16 * s2 + 8 + 4 * hh) = make_uint2(dsf[TS][s2].w[2], dsf[TS][s2].w[3]);
+      }
+      if constexpr (!DQP) wave_lds_fence();  // (the partials form waits for both key halves at a workgroup barrier later)
+    };
+    // dS form: the wave's 32 keys of every row go to the dS tile of the row's list entry
+    int dsrow = -1;
+    auto ds_read = [&](auto pc, auto tsc) {
+      constexpr int TS = decltype(pc)::value * 4 + decltype(tsc)::value;
+      dsrow = pRow[TS * 32 + (lane & 31)];
+#pragma unroll
+      for (int s4 = 0; s4 < 2; ++s4) dsx[s4] = tr_frag8_at(trdS, 16 * s4 * LDS_, (16 * s4 + 4) * LDS_);
+      wave_lds_fence();
+    };
+    auto ds_store = [&](int tile) {
+      if (dsrow >= 0) {
+        uint16_t *wp = ws.ds + (lbase + start + tile * 32 + (lane & 31)) * Bn + koff + kh * 32;
+#pragma unroll
+        for (int s4 = 0; s4 < 2; ++s4) *reinterpret_cast<Pack8 *>(wp + 16 * s4 + 8 * hh) = dsx[s4];
+      }
+    };
+    auto dq_load = [&](auto tsc) {
+      constexpr int TS = decltype(tsc)::value;
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) dsx[s4] = tr_frag8_at(trdS, (TS * 64 + 16 * s4) * LDS_, (TS * 64 + 16 * s4 + 4) * LDS_);
+    };
+    auto dq_mma = [&](auto gc) {  // a quarter of the products per chunk
+      constexpr int G = decltype(gc)::value;
+#pragma unroll
+      for (int d2 = 0; d2 < NDH; ++d2) {
+        if constexpr (G == 0) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) dqa[d2][i] = 0.f;
+        }
+        dqa[d2] = mfma32<T>(kt[d2][G], dsx[G], dqa[d2]);
+      }
+    };
+    const int64_t trash = (int64_t)a.total_q * a.heads * ws.cap;  // spare row: takes the writes of absent rows, no branch
+    auto dq_store = [&](auto pc, auto tsc) {
+      constexpr int TS = decltype(pc)::value * 4 + decltype(tsc)::value;
+      uint16_t *sdQ = sdQ0 + (size_t)decltype(pc)::value * 4 * (TB / 2);
+      // register i of feature tile d2 <-> feature d2*32 + acc_row(i, hh) of this wave's half, this lane's row
+#pragma unroll
+      for (int d2 = 0; d2 < NDH; ++d2)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          *reinterpret_cast<uint2 *>(sdQ + (lane & 31) * LDH + d2 * 32 + 8 * g + 4 * hh) =
+              make_uint2(pack2<T>(dqa[d2][4 * g], dqa[d2][4 * g + 1]), pack2<T>(dqa[d2][4 * g + 2], dqa[d2][4 * g + 3]));
+      wave_lds_fence();
+      constexpr int LPR = HD / 16;        // lanes per half row (16 bytes each)
+      constexpr int RPP = 64 / LPR;       // rows per pass
+      const int col = (lane % LPR) * 8;
+#pragma unroll
+      for (int k = 0; k < 32 / RPP; ++k) {
+        const int row = k * RPP + lane / LPR;
+        const int r2 = pRow[TS * 32 + row], s2 = pSlot[TS * 32 + row];
+        const Pack8 x = *reinterpret_cast<const Pack8 *>(sdQ + row * LDH + col);
+        const bool ok = (r2 >= 0) & (s2 < ws.cap);
+        const int64_t pidx = ok ? ((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2 : trash;
+        if (kh * (HD / 2) + col < D) *reinterpret_cast<Pack8 *>(ws.part + pidx * D + kh * (HD / 2) + col) = x;
+        if (kh == 0 && col == 0) ws.pid[pidx] = nb;
+      }
+      wave_lds_fence();
+    };
+    // One round of a pair = its tiles 2 px and 2 px + 1, both already in LDS.  Tiles past the end of the list hold
+    // absent rows (row id -1, zero data): they run through the same code and add nothing.
+    auto process_round = [&](auto pc, int r) {  // pc: parity of r = the LDS buffer that holds the round
+      // S, dP of the first tile
+      ld_a(pc, C0{}, C0{});
+      fence();
+      static_for<4>([&](auto gc) {
+        constexpr int G = decltype(gc)::value;
+        if constexpr (G < 3) ld_a(pc, C0{}, std::integral_constant<int, G + 1>{});
+        mm_a(C0{}, gc);
+        fence();
+      });
+      // S, dP of the second tile between the softmax rows of the first
+      ld_a(pc, C1{}, C0{});
+      ld_s(pc, C0{}, C0{});
+      fence();
+      static_for<4>([&](auto gc) {
+        constexpr int G = decltype(gc)::value;
+        if constexpr (G < 3) {
+          ld_a(pc, C1{}, std::integral_constant<int, G + 1>{});
+          ld_s(pc, C0{}, std::integral_constant<int, G + 1>{});
+        }
+        mm_a(C1{}, gc);
+        smx(C0{}, gc);
+        fence();
+      });
+      // dV, dK of the first tile between the softmax rows of the second
+      ds_write(C0{});
+      ld_b(pc, C0{}, C0{});
+      ld_s(pc, C1{}, C0{});
+      if constexpr (!DQP) ds_read(pc, C0{});
+      fence();
+      static_for<4>([&](auto gc) {
+        constexpr int G = decltype(gc)::value;
+        if constexpr (G < 3) {
+          ld_b(pc, C0{}, std::integral_constant<int, G + 1>{});
+          ld_s(pc, C1{}, std::integral_constant<int, G + 1>{});
+        }
+        mm_b(C0{}, gc);
+        smx(C1{}, gc);
+        if constexpr (!DQP && G == 1) ds_store(4 * r + 2 * px);
+        fence();
+      });
+      // dV, dK of the second tile; in the partials form dQ of the first one runs between them: by now both key
+      // halves have put dS^T of both tiles into LDS, so the one barrier the exchange needs hardly ever waits
+      ds_write(C1{});
+      if constexpr (DQP) __syncthreads();
+      ld_b(pc, C1{}, C0{});
+      if constexpr (DQP)
+        dq_load(C0{});
+      else
+        ds_read(pc, C1{});
+      fence();
+      static_for<4>([&](auto gc) {
+        constexpr int G = decltype(gc)::value;
+        if constexpr (G < 3) ld_b(pc, C1{}, std::integral_constant<int, G + 1>{});
+        mm_b(C1{}, gc);
+        if constexpr (DQP) dq_mma(gc);
+        if constexpr (!DQP && G == 1) ds_store(4 * r + 2 * px + 1);
+        fence();
+      });
+      if constexpr (DQP) {
+        dq_store(pc, C0{});
+        // dQ of the second tile
+        dq_load(C1{});
+        fence();
+        static_for<4>([&](auto gc) {
+          dq_mma(gc);
+          fence();
+        });
+        dq_store(pc, C1{});
+      }
+    };
+    auto round = [&](auto pc, int r) {
+#if defined(__HIP_DEVICE_COMPILE__)
+      asm volatile("" : "+v"(aQ), "+v"(adO), "+v"(tQ), "+v"(tdO), "+v"(ft));
+#endif
+      rid_issue(r + 2);
+      meta_issue(r + 1);
+      tile_issue(r + 1);
+      process_round(pc, r);
+      meta_store(r + 1);
+      rid_store(r + 2);
+      wait_all_loads();
+      __syncthreads();  // round r + 1 is in LDS; everyone is done with round r
+    };
+    for (int r = 0; r < nround; r += 2) {
+      round(C0{}, r);
+      if (r + 1 < nround) round(C1{}, r + 1);
+    }
+  }
+
+  // ---- dK^T / dV^T: the second pair hands its sums to the first, which adds its own ---------------------------
+  __syncthreads();  // K and V have left LDS (lists without rows come here directly)
+  auto red_io = [&](bool add) {
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        float *rp = red + (size_t)(kh * 32 + (lane & 31)) * LDR + dt * 32 + 8 * g + 4 * hh;
         f32x4 v4, k4;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
           v4[jj] = dv[dt][4 * g + jj];
           k4[jj] = dk[dt][4 * g + jj];
         }
-        float *rp = red + (size_t)(kh * 32 + (lane & 31)) * LDR + dt * 32 + 8 * g + 4 * hh;
+        if (add) {
+          const f32x4 ov = *reinterpret_cast<const f32x4 *>(rp), ok = *reinterpret_cast<const f32x4 *>(rp + 64 * LDR);
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) {
+            v4[jj] += ov[jj];
+            k4[jj] += ok[jj];
+          }
+        }
         *reinterpret_cast<f32x4 *>(rp) = v4;
         *reinterpret_cast<f32x4 *>(rp + 64 * LDR) = k4;
       }
-  }
+  };
+  if (px == 1) red_io(false);
+  __syncthreads();
+  if (px == 0) red_io(true);
   __syncthreads();
 
   // ---- dK^T / dV^T leave as rows, once ----------------------------------------------------------------

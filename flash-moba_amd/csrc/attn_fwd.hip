@@ -111,7 +111,7 @@ __global__ __launch_bounds__((NCW + 2) * 64) void attn_fwd_col_kernel(fmoba_attn
   if (c < a.max_cols) {
     nnz = a.col_nnz[bh * a.max_cols + c];
     lbase = a.col_offsets[bh * a.max_cols + c];
-    if (causal && nnz > 0) start = lower_bound_i32(a.row_indices + lbase, nnz, key0 - off);  // earlier rows see no key of the block
+    if (causal && nnz > 0) start = lower_bound_wave_i32(a.row_indices + lbase, nnz, key0 - off);  // earlier rows see no key of the block
   }
   const int32_t *list = a.row_indices + lbase;
   const uint16_t *qg = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)q0 * a.q_row_stride + (int64_t)h * a.q_head_stride;

@@ -309,6 +309,24 @@ __device__ __forceinline__ int lower_bound_i32(const int32_t *p, int n, int v) {
   return lo;
 }
 
+// The same search by a whole wave (every lane passes the same arguments and gets the same result): 64 probes per
+// step, so a list of a few thousand entries takes two or three dependent loads instead of a dozen.
+__device__ __forceinline__ int lower_bound_wave_i32(const int32_t *p, int n, int v) {
+  const int lane = threadIdx.x & 63;
+  int lo = 0, hi = n;
+  while (lo < hi) {
+    const int step = (hi - lo + 63) >> 6;
+    const int q = lo + lane * step;
+    const bool below = q < hi && p[q] < v;
+    const int cnt = __popcll(__ballot(below));  // the probes are ascending: the first cnt of them are below v
+    if (cnt == 0) break;
+    const int q1 = lo + (cnt - 1) * step;       // last probe below v: the answer lies in (q1, q1 + step]
+    lo = q1 + 1;
+    hi = min(q1 + step, hi);
+  }
+  return lo;
+}
+
 // f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}): a loop whose index is a
 // compile-time constant inside the body (register arrays, template arguments)
 template <typename F, int... I>
