@@ -43,18 +43,16 @@ struct BwdSmem {
   static constexpr size_t tileBytes = (size_t)32 * HD * 2;
   static constexpr size_t oQ = 0;                                   // [2 buffers][4 tiles][32][HD]
   static constexpr size_t odO = oQ + 8 * tileBytes;
-  static constexpr size_t odS = odO + 8 * tileBytes;               // partials form: [2 pairs][2 tile slots][64 keys][LDS_]; dS form: [4 waves][32 keys][LDS_]
-  static constexpr int LDH = HD / 2 + 8;                            // elements, per-wave dQ half-row tile [32][LDH]: in a tile that is no longer read
+  static constexpr size_t odS = odO + 8 * tileBytes;               // partials form: [2 pairs][2 tile slots][64 keys][LDS_] or [2 tile slots][128 keys][LDS_]; dS form: [4 waves][32 keys][LDS_]
   static constexpr size_t oRid = odS + (size_t)2 * 2 * 64 * LDS_ * 2;  // int[2 buffers][128]: row ids, one round before the rest
   static constexpr size_t oRow = oRid + 2 * kBwdRoundRows * 4;     // int[2 buffers][128]
   static constexpr size_t oSlot = oRow + 2 * kBwdRoundRows * 4;
   static constexpr size_t oLse = oSlot + 2 * kBwdRoundRows * 4;    // LSE * log2(e)
   static constexpr size_t oDelta = oLse + 2 * kBwdRoundRows * 4;
   static constexpr size_t bytes = oDelta + 2 * kBwdRoundRows * 4;
-  static constexpr int LDR = HD + 4;  // floats, output transpose buffer [2][64 keys][LDR]
-  static_assert((size_t)2 * 64 * LDR * 4 <= 16 * tileBytes, "the output buffer reuses the tiles");
-  static_assert((size_t)2 * 64 * LDQ * 2 <= 16 * tileBytes, "K and V pass through the tiles");
-  static_assert((size_t)32 * LDH * 2 <= tileBytes, "a wave's dQ half rows pass through a tile");
+  static constexpr int LDR = HD + 4;  // floats, output transpose buffer [2][64 or 128 keys][LDR]
+  static_assert((size_t)2 * 128 * LDR * 4 <= bytes, "the output buffer reuses the tiles");
+  static_assert((size_t)2 * 128 * LDQ * 2 <= 16 * tileBytes, "K and V pass through the tiles");
   static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
 };
 
@@ -78,6 +76,15 @@ __device__ __forceinline__ Pack8 lds_read16(uint32_t byte_addr) {
 #else
   (void)byte_addr;
   return Pack8{{0, 0, 0, 0}};
+#endif
+}
+template <typename V>
+__device__ __forceinline__ V lds_read_vec(uint32_t byte_addr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return *(__attribute__((address_space(3))) const V *)byte_addr;
+#else
+  (void)byte_addr;
+  return V{};
 #endif
 }
 // 8 x 16-bit operand of a transposing read: two 8-byte reads
@@ -120,12 +127,20 @@ struct BwdWs {
   uint16_t *ds;    // [row list entry][lg_block_n] dS tiles (row-stationary dQ form)
 };
 
-// DQP = true: dQ partials per visit (for the combine kernel); false: dS^T tiles to ws.ds (for the row-stationary dQ kernel)
-template <typename T, int HD, bool DQP>
+// DQP = true: dQ partials per visit (for the combine kernel); false: dS^T tiles to ws.ds (for the row-stationary dQ kernel).
+// KB = 1: the workgroup owns 64 keys, wave pair px takes tiles 2 px, 2 px + 1 of a round and wave kq of the pair the
+// key half kq.  KB = 2 (columns of a multiple of 128 keys, whose two 64-key blocks share one row list): it owns 128
+// keys, every wave takes all four tiles for its key quarter kq, so a gathered row serves twice the keys and a visit
+// leaves one dQ partial instead of two.
+template <typename T, int HD, bool DQP, int KB>
 __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args a, BwdWs ws) {
   typedef BwdSmem<HD> SM;
-  constexpr int KS = HD / 16, LDQ = SM::LDQ, LDS_ = SM::LDS_, NDT = HD / 32, VPR = HD / 8, LDR = SM::LDR, LDH = SM::LDH;
-  constexpr int NDH = NDT / 2;  // feature tiles of dQ per compute wave
+  constexpr int KS = HD / 16, LDQ = SM::LDQ, LDS_ = SM::LDS_, NDT = HD / 32, VPR = HD / 8, LDR = SM::LDR;
+  constexpr int NKEY = 64 * KB;         // keys of the workgroup
+  constexpr int NDH = NDT / (2 * KB);   // feature tiles of dQ per wave
+  constexpr int LDH = NDH * 32 + 8;     // elements, per-wave dQ part-row tile [32][LDH]
+  static_assert(NDH >= 1, "128-key workgroups need head_dim 128");
+  static_assert((size_t)KB * 32 * LDH * 2 <= SM::tileBytes, "the dQ part rows of KB waves pass through a tile");
   constexpr uint32_t TB = (uint32_t)SM::tileBytes;
   constexpr int RB = HD * 2;    // bytes of a tile row
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -135,18 +150,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   float *sLse = reinterpret_cast<float *>(smem + SM::oLse);
   float *sDelta = reinterpret_cast<float *>(smem + SM::oDelta);
 
-  const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + 63) / 64);
+  const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + NKEY - 1) / NKEY);
   const int nb = item.idx, b = item.pair / a.heads, h = item.pair - b * a.heads;
   const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
-  const int key0 = nb * 64;
+  const int key0 = nb * NKEY;
   if (key0 >= Lk) return;
   const int q0 = a.cu_seqlens_q[b], Lq = a.cu_seqlens_q[b + 1] - q0;
   const int off = Lk - Lq;
   const int D = a.head_dim;
   const int hk = h / (a.heads / a.heads_k);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
-  const int kh = wave & 1;   // key half of this wave
-  const int px = wave >> 1;  // wave pair: takes tiles 2 px and 2 px + 1 of every round
+  const int kq = KB == 1 ? (wave & 1) : wave;  // this wave's 32 keys of the block, and its share of the dQ features
+  const int px = KB == 1 ? (wave >> 1) : 0;    // KB = 1: wave pair, takes tiles 2 px and 2 px + 1 of every round
   const bool causal = a.is_causal != 0;
   const float scale_log2 = a.softmax_scale * 1.4426950408889634f;
   constexpr float kLog2e = 1.4426950408889634f;
@@ -154,7 +169,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   // ---- the key block: through LDS into registers.  The loads are issued first and stored after the look-up of
   // the column list below, so that the two chains of dependent loads wait together (one workgroup per compute
   // unit: nothing else covers them) ----------------------------------------------
-  constexpr int NKV = 64 * VPR / 256;
+  constexpr int NKV = NKEY * VPR / 256;
   Pack8 xk[NKV], xv[NKV];
   {
     const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + (int64_t)(k0 + key0) * a.k_row_stride + (int64_t)hk * a.k_head_stride;
@@ -200,7 +215,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   }
 
   {
-    uint16_t *sK = reinterpret_cast<uint16_t *>(smem), *sV = sK + 64 * LDQ;
+    uint16_t *sK = reinterpret_cast<uint16_t *>(smem), *sV = sK + NKEY * LDQ;
 #pragma unroll
     for (int i = 0; i < NKV; ++i) {
       const int v = tid + 256 * i;
@@ -213,21 +228,21 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   // B operands of S and dP: this lane's key, its half of the head dim; K^T of this wave's half of the features for
   // the dQ products.  They never change, so they stay in registers.
   Pack8 kb[KS], vb[KS];
-  Pack8 kt[NDH][4];
+  Pack8 kt[NDH][4 * KB];
   {
-    const uint16_t *sK = reinterpret_cast<const uint16_t *>(smem), *sV = sK + 64 * LDQ;
+    const uint16_t *sK = reinterpret_cast<const uint16_t *>(smem), *sV = sK + NKEY * LDQ;
 #pragma unroll
     for (int t = 0; t < KS; ++t) {
-      kb[t] = *reinterpret_cast<const Pack8 *>(sK + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
-      vb[t] = *reinterpret_cast<const Pack8 *>(sV + (kh * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
+      kb[t] = *reinterpret_cast<const Pack8 *>(sK + (kq * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
+      vb[t] = *reinterpret_cast<const Pack8 *>(sV + (kq * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
     }
     if constexpr (DQP) {
       lds_cu16 *trK = tr_lane_base(sK, LDQ, lane) + 8 * hh * LDQ;
 #pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4)
+      for (int s4 = 0; s4 < 4 * KB; ++s4)
 #pragma unroll
         for (int d2 = 0; d2 < NDH; ++d2) {
-          const int lo = 16 * s4 * LDQ + (kh * NDH + d2) * 32;
+          const int lo = 16 * s4 * LDQ + (kq * NDH + d2) * 32;
           kt[d2][s4] = tr_frag8_at(trK, lo, lo + 4 * LDQ);
         }
     }
@@ -238,7 +253,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   const float *lseg = a.softmax_lse + (int64_t)h * a.total_q + q0;
   const float *delg = a.softmax_d + (int64_t)h * ((int64_t)a.total_q + 128 * (int64_t)a.batch) + q0 + 128 * b;
   int32_t *cntg = ws.cnt + (int64_t)q0 * a.heads + h;  // counter of local row r: cntg[r * heads]
-  float *red = reinterpret_cast<float *>(smem);  // [2][64 keys][LDR]: dV^T, dK^T on their way out
+  float *red = reinterpret_cast<float *>(smem);  // [2][NKEY][LDR]: dV^T, dK^T on their way out
 
   f32x16 dv[NDT], dk[NDT];
 #pragma unroll
@@ -337,32 +352,42 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     const uint32_t rowoff = (uint32_t)((lane & 31) * RB + (((hh * KS) ^ bwd_swz<HD>(lane & 31)) * 16));
     const int li = lane & 15, r0t = (li >> 2) + 4 * hh;
     const uint32_t troff = (uint32_t)(r0t * RB + ((((((lane >> 4) & 1) * 2 + ((li & 3) >> 1))) ^ bwd_swz<HD>(r0t)) * 16) + (li & 1) * 8);
-    // (re-made opaque in every round: the operand addresses derived from them must not be kept in registers
-    // across rounds, there are none to spare)
-    uint32_t aQ = pairQ + rowoff, adO = pairdO + rowoff, tQ = pairQ + troff, tdO = pairdO + troff;
-    uint16_t *sdS = reinterpret_cast<uint16_t *>(smem + SM::odS) + (DQP ? (size_t)px * 2 * 64 * LDS_ : (size_t)wave * 32 * LDS_);
+    // (re-made opaque wherever they are used: the operand addresses derived from them must not be kept in
+    // registers from one use to the next, there are none to spare)
+    const uint32_t aQ = pairQ + rowoff, adO = pairdO + rowoff, tQ = pairQ + troff, tdO = pairdO + troff;
+    auto opaque = [](uint32_t &x, uint32_t &y) {
+#if defined(__HIP_DEVICE_COMPILE__)
+      asm volatile("" : "+v"(x), "+v"(y));
+#else
+      (void)x, (void)y;
+#endif
+    };
+    uint16_t *sdS = reinterpret_cast<uint16_t *>(smem + SM::odS) + (DQP ? (size_t)px * 2 * 64 * LDS_ : (size_t)wave * 32 * LDS_);  // (px = 0 with 128 keys)
     lds_cu16 *trdS = tr_lane_base(sdS, LDS_, lane) + 8 * hh * LDS_;  // dS^T tile: 8 consecutive keys per read
-    // the dQ half rows of a tile leave through the first tile of the pair, which nobody reads after the barrier in
-    // the middle of the round: Q's for the first key half, dO's for the second
-    uint16_t *sdQ0 = reinterpret_cast<uint16_t *>(smem + (kh ? SM::odO : SM::oQ) + (size_t)(px * 2) * TB);
-    const int *pRow = sRow + px * 64, *pSlot = sSlot + px * 64;
-    const float *pLse = sLse + px * 64, *pDelta = sDelta + px * 64;
+    // the dQ part rows of a tile leave through the first tile of the pair, which nobody reads after the barrier in
+    // the middle of the round: Q's for even waves, dO's for odd ones, one half of it each with four key quarters
+    uint16_t *sdQ0 = reinterpret_cast<uint16_t *>(smem + ((kq & 1) ? SM::odO : SM::oQ) + (size_t)(px * 2) * TB + (size_t)(kq >> 1) * (TB / 2));
+    const int *pRow = sRow + px * 64;
+    const uint32_t smx0 = (uint32_t)(uintptr_t)(smem + SM::oRow) + (uint32_t)(px * 64 * 4 + hh * 16);  // softmax inputs of this lane's rows
     Pack8 qa[2][KC], doa[2][KC];     // A operands of S and dP (this lane's row, its half of the head dim), double-buffered by chunk
     Pack8 dot[2][BC], qt[2][BC];     // dO^T / Q^T operands of the dV / dK products, double-buffered by chunk
     f32x4 lse4[2], del4[2];          // softmax inputs of a chunk's four rows
     int4 row4[2];
     Pack8 pf[2][2], dsf[2][2];       // P and dS of both tiles of the round as MFMA operands
-    Pack8 dsx[4];                    // dS^T of all 64 keys as the B operand of the dQ products
+    Pack8 dsx[4 * KB];               // dS^T of all keys of the block as the B operand of the dQ products
     f32x16 dqa[NDH];
     f32x16 s[2], dp[2];
     auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
-    auto ld_a = [&](auto pc, auto tsc, auto gc) {
-      constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(tsc)::value) * TB;
+    // pc: buffer of the round; pp: tile pair (always 0 with KB = 1, where the pair is part of the addresses); tsc: tile of the pair
+    auto ld_a = [&](auto pc, auto pp, auto tsc, auto gc) {
+      constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value) * TB;
       constexpr int G = decltype(gc)::value;
+      uint32_t bq = aQ, bo = adO;
+      opaque(bq, bo);
 #pragma unroll
       for (int t = 0; t < KC; ++t) {
-        qa[G & 1][t] = lds_read16((aQ ^ (uint32_t)((G * KC + t) * 16)) + TO);
-        doa[G & 1][t] = lds_read16((adO ^ (uint32_t)((G * KC + t) * 16)) + TO);
+        qa[G & 1][t] = lds_read16((bq ^ (uint32_t)((G * KC + t) * 16)) + TO);
+        doa[G & 1][t] = lds_read16((bo ^ (uint32_t)((G * KC + t) * 16)) + TO);
       }
     };
     auto mm_a = [&](auto tsc, auto gc) {
@@ -380,17 +405,19 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         dp[TS] = mfma32<T>(doa[G & 1][t], vb[G * KC + t], dp[TS]);
       }
     };
-    auto ld_b = [&](auto pc, auto tsc, auto gc) {
-      constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(tsc)::value) * TB;
+    auto ld_b = [&](auto pc, auto pp, auto tsc, auto gc) {
+      constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value) * TB;
       constexpr int G = decltype(gc)::value;
+      uint32_t bq = tQ, bo = tdO;
+      opaque(bq, bo);
 #pragma unroll
       for (int t = 0; t < BC; ++t) {
         const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
         // rows 16 s2 + (0..3) + 4 hh and the same + 8, features dt * 32 ..
         const uint32_t xlo = (uint32_t)(dt * 4 * 16), xhi = (uint32_t)(((dt * 4) ^ BwdSwz<HD>::kRow8) * 16);
         const uint32_t olo = TO + (uint32_t)(16 * s2 * RB), ohi = olo + (uint32_t)(8 * RB);
-        dot[G & 1][t] = lds_tr8((tdO ^ xlo) + olo, (tdO ^ xhi) + ohi);
-        qt[G & 1][t] = lds_tr8((tQ ^ xlo) + olo, (tQ ^ xhi) + ohi);
+        dot[G & 1][t] = lds_tr8((bo ^ xlo) + olo, (bo ^ xhi) + ohi);
+        qt[G & 1][t] = lds_tr8((bq ^ xlo) + olo, (bq ^ xhi) + ohi);
       }
     };
     auto mm_b = [&](auto tsc, auto gc) {
@@ -404,14 +431,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       }
     };
     // this lane's key; key j is visible to row r iff r >= row_thr (rows that do not exist are stored as -1)
-    const int j = key0 + kh * 32 + (lane & 31);
+    const int j = key0 + kq * 32 + (lane & 31);
     const int row_thr = j >= Lk ? 0x7fffffff : (causal ? max(0, j - off) : 0);
-    auto ld_s = [&](auto pc, auto tsc, auto gc) {
-      constexpr int TS = decltype(pc)::value * 4 + decltype(tsc)::value, G = decltype(gc)::value;
-      const int base = TS * 32 + 8 * G + 4 * hh;  // accumulator registers 4G..4G+3 hold rows base..base+3
-      lse4[G & 1] = *reinterpret_cast<const f32x4 *>(pLse + base);
-      del4[G & 1] = *reinterpret_cast<const f32x4 *>(pDelta + base);
-      row4[G & 1] = *reinterpret_cast<const int4 *>(pRow + base);
+    auto ld_s = [&](auto pc, auto pp, auto tsc, auto gc) {
+      constexpr int TS = decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value, G = decltype(gc)::value;
+      // accumulator registers 4G..4G+3 hold rows TS * 32 + 8 G + 4 hh + (0..3); one address register, the rest
+      // are offsets in the instructions
+      constexpr uint32_t O = (uint32_t)(TS * 32 + 8 * G) * 4;
+      uint32_t bs = smx0, unused = 0;
+      opaque(bs, unused);
+      row4[G & 1] = lds_read_vec<int4>(bs + O);
+      lse4[G & 1] = lds_read_vec<f32x4>(bs + O + (uint32_t)(SM::oLse - SM::oRow));
+      del4[G & 1] = lds_read_vec<f32x4>(bs + O + (uint32_t)(SM::oDelta - SM::oRow));
     };
     auto smx = [&](auto tsc, auto gc) {
       constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
@@ -435,8 +466,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     // half rows (16-bit, unscaled) go to the partial slot that the row handed out for this visit.
     auto ds_write = [&](auto tsc) {
       constexpr int TS = decltype(tsc)::value;
-      // partials form: tile slot TS of the pair, rows of both key halves; else: this wave's private tile
-      uint16_t *t = sdS + (size_t)((DQP ? TS * 64 + kh * 32 : 0) + (lane & 31)) * LDS_;
+      // partials form: tile slot TS of the pair, rows of all keys of the block; else: this wave's private tile
+      uint16_t *t = sdS + (size_t)((DQP ? TS * NKEY + kq * 32 : 0) + (lane & 31)) * LDS_;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         *reinterpret_cast<uint2 *>(t + 16 * s2 + 4 * hh) = make_uint2(dsf[TS][s2].w[0], dsf[TS][s2].w[1]);
@@ -446,8 +477,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     };
     // dS form: the wave's 32 keys of every row go to the dS tile of the row's list entry
     int dsrow = -1;
-    auto ds_read = [&](auto pc, auto tsc) {
-      constexpr int TS = decltype(pc)::value * 4 + decltype(tsc)::value;
+    auto ds_read = [&](auto pc, auto pp, auto tsc) {
+      constexpr int TS = decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value;
       dsrow = pRow[TS * 32 + (lane & 31)];
 #pragma unroll
       for (int s4 = 0; s4 < 2; ++s4) dsx[s4] = tr_frag8_at(trdS, 16 * s4 * LDS_, (16 * s4 + 4) * LDS_);
@@ -455,7 +486,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     };
     auto ds_store = [&](int tile) {
       if (dsrow >= 0) {
-        uint16_t *wp = ws.ds + (lbase + start + tile * 32 + (lane & 31)) * Bn + koff + kh * 32;
+        uint16_t *wp = ws.ds + (lbase + start + tile * 32 + (lane & 31)) * Bn + koff + kq * 32;
 #pragma unroll
         for (int s4 = 0; s4 < 2; ++s4) *reinterpret_cast<Pack8 *>(wp + 16 * s4 + 8 * hh) = dsx[s4];
       }
@@ -463,7 +494,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     auto dq_load = [&](auto tsc) {
       constexpr int TS = decltype(tsc)::value;
 #pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) dsx[s4] = tr_frag8_at(trdS, (TS * 64 + 16 * s4) * LDS_, (TS * 64 + 16 * s4 + 4) * LDS_);
+      for (int s4 = 0; s4 < 4 * KB; ++s4) dsx[s4] = tr_frag8_at(trdS, (TS * NKEY + 16 * s4) * LDS_, (TS * NKEY + 16 * s4 + 4) * LDS_);
     };
     auto dq_mma = [&](auto gc) {  // a quarter of the products per chunk
       constexpr int G = decltype(gc)::value;
@@ -473,13 +504,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 #pragma unroll
           for (int i = 0; i < 16; ++i) dqa[d2][i] = 0.f;
         }
-        dqa[d2] = mfma32<T>(kt[d2][G], dsx[G], dqa[d2]);
+#pragma unroll
+        for (int t = 0; t < KB; ++t) dqa[d2] = mfma32<T>(kt[d2][G * KB + t], dsx[G * KB + t], dqa[d2]);
       }
     };
     const int64_t trash = (int64_t)a.total_q * a.heads * ws.cap;  // spare row: takes the writes of absent rows, no branch
-    auto dq_store = [&](auto pc, auto tsc) {
-      constexpr int TS = decltype(pc)::value * 4 + decltype(tsc)::value;
-      uint16_t *sdQ = sdQ0 + (size_t)decltype(pc)::value * 4 * (TB / 2);
+    auto dq_store = [&](auto pc, auto pp, auto tsc) {
+      constexpr int TS = decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value;
+      uint16_t *sdQ = sdQ0 + (size_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2) * (TB / 2);
       // register i of feature tile d2 <-> feature d2*32 + acc_row(i, hh) of this wave's half, this lane's row
 #pragma unroll
       for (int d2 = 0; d2 < NDH; ++d2)
@@ -488,84 +520,90 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           *reinterpret_cast<uint2 *>(sdQ + (lane & 31) * LDH + d2 * 32 + 8 * g + 4 * hh) =
               make_uint2(pack2<T>(dqa[d2][4 * g], dqa[d2][4 * g + 1]), pack2<T>(dqa[d2][4 * g + 2], dqa[d2][4 * g + 3]));
       wave_lds_fence();
-      constexpr int LPR = HD / 16;        // lanes per half row (16 bytes each)
+      constexpr int LPR = NDH * 4;        // lanes per part row (16 bytes each)
       constexpr int RPP = 64 / LPR;       // rows per pass
       const int col = (lane % LPR) * 8;
+      uint32_t bs = (uint32_t)(uintptr_t)(smem + SM::oRow) + (uint32_t)((px * 64 + lane / LPR) * 4), unused = 0;
+      opaque(bs, unused);
 #pragma unroll
       for (int k = 0; k < 32 / RPP; ++k) {
         const int row = k * RPP + lane / LPR;
-        const int r2 = pRow[TS * 32 + row], s2 = pSlot[TS * 32 + row];
+        const int r2 = lds_read_vec<int>(bs + (uint32_t)(TS * 32 + k * RPP) * 4);
+        const int s2 = lds_read_vec<int>(bs + (uint32_t)(TS * 32 + k * RPP) * 4 + (uint32_t)(SM::oSlot - SM::oRow));
         const Pack8 x = *reinterpret_cast<const Pack8 *>(sdQ + row * LDH + col);
         const bool ok = (r2 >= 0) & (s2 < ws.cap);
         const int64_t pidx = ok ? ((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2 : trash;
-        if (kh * (HD / 2) + col < D) *reinterpret_cast<Pack8 *>(ws.part + pidx * D + kh * (HD / 2) + col) = x;
-        if (kh == 0 && col == 0) ws.pid[pidx] = nb;
+        if (kq * (NDH * 32) + col < D) *reinterpret_cast<Pack8 *>(ws.part + pidx * D + kq * (NDH * 32) + col) = x;
+        if (kq == 0 && col == 0) ws.pid[pidx] = nb;
       }
       wave_lds_fence();
     };
     // One round of a pair = its tiles 2 px and 2 px + 1, both already in LDS.  Tiles past the end of the list hold
     // absent rows (row id -1, zero data): they run through the same code and add nothing.
-    auto process_round = [&](auto pc, int r) {  // pc: parity of r = the LDS buffer that holds the round
+    auto process_round = [&](auto pc, auto pp, int r) {  // pc: parity of r = the LDS buffer that holds the round
+      const int tile0 = 4 * r + 2 * (KB == 1 ? px : decltype(pp)::value);  // position of the pair's first tile in the list
       // S, dP of the first tile
-      ld_a(pc, C0{}, C0{});
+      ld_a(pc, pp, C0{}, C0{});
       fence();
       static_for<4>([&](auto gc) {
         constexpr int G = decltype(gc)::value;
-        if constexpr (G < 3) ld_a(pc, C0{}, std::integral_constant<int, G + 1>{});
+        if constexpr (G < 3) ld_a(pc, pp, C0{}, std::integral_constant<int, G + 1>{});
         mm_a(C0{}, gc);
         fence();
       });
       // S, dP of the second tile between the softmax rows of the first
-      ld_a(pc, C1{}, C0{});
-      ld_s(pc, C0{}, C0{});
+      ld_a(pc, pp, C1{}, C0{});
+      ld_s(pc, pp, C0{}, C0{});
       fence();
       static_for<4>([&](auto gc) {
         constexpr int G = decltype(gc)::value;
         if constexpr (G < 3) {
-          ld_a(pc, C1{}, std::integral_constant<int, G + 1>{});
-          ld_s(pc, C0{}, std::integral_constant<int, G + 1>{});
+          ld_a(pc, pp, C1{}, std::integral_constant<int, G + 1>{});
+          ld_s(pc, pp, C0{}, std::integral_constant<int, G + 1>{});
         }
         mm_a(C1{}, gc);
         smx(C0{}, gc);
         fence();
       });
       // dV, dK of the first tile between the softmax rows of the second
+      // (a second pair of the same waves reuses the dS^T tiles of the first: its readers have to be done)
+      if constexpr (DQP && decltype(pp)::value == 1) __syncthreads();
       ds_write(C0{});
-      ld_b(pc, C0{}, C0{});
-      ld_s(pc, C1{}, C0{});
-      if constexpr (!DQP) ds_read(pc, C0{});
+      ld_b(pc, pp, C0{}, C0{});
+      ld_s(pc, pp, C1{}, C0{});
+      if constexpr (!DQP) ds_read(pc, pp, C0{});
       fence();
       static_for<4>([&](auto gc) {
         constexpr int G = decltype(gc)::value;
         if constexpr (G < 3) {
-          ld_b(pc, C0{}, std::integral_constant<int, G + 1>{});
-          ld_s(pc, C1{}, std::integral_constant<int, G + 1>{});
+          ld_b(pc, pp, C0{}, std::integral_constant<int, G + 1>{});
+          ld_s(pc, pp, C1{}, std::integral_constant<int, G + 1>{});
         }
         mm_b(C0{}, gc);
         smx(C1{}, gc);
-        if constexpr (!DQP && G == 1) ds_store(4 * r + 2 * px);
+        if constexpr (!DQP && G == 1) ds_store(tile0);
         fence();
       });
-      // dV, dK of the second tile; in the partials form dQ of the first one runs between them: by now both key
-      // halves have put dS^T of both tiles into LDS, so the one barrier the exchange needs hardly ever waits
+      // dV, dK of the second tile; in the partials form dQ of the first one runs between them: by now all key
+      // groups have put dS^T of both tiles into LDS, so the one barrier the exchange needs hardly ever waits
       ds_write(C1{});
       if constexpr (DQP) __syncthreads();
-      ld_b(pc, C1{}, C0{});
+      ld_b(pc, pp, C1{}, C0{});
       if constexpr (DQP)
         dq_load(C0{});
       else
-        ds_read(pc, C1{});
+        ds_read(pc, pp, C1{});
       fence();
       static_for<4>([&](auto gc) {
         constexpr int G = decltype(gc)::value;
-        if constexpr (G < 3) ld_b(pc, C1{}, std::integral_constant<int, G + 1>{});
+        if constexpr (G < 3) ld_b(pc, pp, C1{}, std::integral_constant<int, G + 1>{});
         mm_b(C1{}, gc);
         if constexpr (DQP) dq_mma(gc);
-        if constexpr (!DQP && G == 1) ds_store(4 * r + 2 * px + 1);
+        if constexpr (!DQP && G == 1) ds_store(tile0 + 1);
         fence();
       });
       if constexpr (DQP) {
-        dq_store(pc, C0{});
+        dq_store(pc, pp, C0{});
         // dQ of the second tile
         dq_load(C1{});
         fence();
@@ -573,17 +611,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           dq_mma(gc);
           fence();
         });
-        dq_store(pc, C1{});
+        dq_store(pc, pp, C1{});
       }
     };
     auto round = [&](auto pc, int r) {
 #if defined(__HIP_DEVICE_COMPILE__)
-      asm volatile("" : "+v"(aQ), "+v"(adO), "+v"(tQ), "+v"(tdO), "+v"(ft));
+      asm volatile("" : "+v"(ft));
 #endif
       rid_issue(r + 2);
       meta_issue(r + 1);
       tile_issue(r + 1);
-      process_round(pc, r);
+      process_round(pc, C0{}, r);
+      if constexpr (KB == 2) process_round(pc, C1{}, r);
       meta_store(r + 1);
       rid_store(r + 2);
       wait_all_loads();
@@ -595,14 +634,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     }
   }
 
-  // ---- dK^T / dV^T: the second pair hands its sums to the first, which adds its own ---------------------------
+  // ---- dK^T / dV^T: with two pairs the second hands its sums to the first, which adds its own ------------------
   __syncthreads();  // K and V have left LDS (lists without rows come here directly)
   auto red_io = [&](bool add) {
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        float *rp = red + (size_t)(kh * 32 + (lane & 31)) * LDR + dt * 32 + 8 * g + 4 * hh;
+        float *rp = red + (size_t)(kq * 32 + (lane & 31)) * LDR + dt * 32 + 8 * g + 4 * hh;
         f32x4 v4, k4;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
@@ -610,7 +649,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           k4[jj] = dk[dt][4 * g + jj];
         }
         if (add) {
-          const f32x4 ov = *reinterpret_cast<const f32x4 *>(rp), ok = *reinterpret_cast<const f32x4 *>(rp + 64 * LDR);
+          const f32x4 ov = *reinterpret_cast<const f32x4 *>(rp), ok = *reinterpret_cast<const f32x4 *>(rp + NKEY * LDR);
 #pragma unroll
           for (int jj = 0; jj < 4; ++jj) {
             v4[jj] += ov[jj];
@@ -618,21 +657,25 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           }
         }
         *reinterpret_cast<f32x4 *>(rp) = v4;
-        *reinterpret_cast<f32x4 *>(rp + 64 * LDR) = k4;
+        *reinterpret_cast<f32x4 *>(rp + NKEY * LDR) = k4;
       }
   };
-  if (px == 1) red_io(false);
-  __syncthreads();
-  if (px == 0) red_io(true);
+  if constexpr (KB == 1) {
+    if (px == 1) red_io(false);
+    __syncthreads();
+    if (px == 0) red_io(true);
+  } else {
+    red_io(false);
+  }
   __syncthreads();
 
   // ---- dK^T / dV^T leave as rows, once ----------------------------------------------------------------
   uint16_t *dkg = reinterpret_cast<uint16_t *>(a.dk) + (int64_t)(k0 + key0) * a.dk_row_stride + (int64_t)h * a.dk_head_stride;
   uint16_t *dvg = reinterpret_cast<uint16_t *>(a.dv) + (int64_t)(k0 + key0) * a.dv_row_stride + (int64_t)h * a.dv_head_stride;
-  for (int v = tid; v < 64 * VPR; v += 256) {
+  for (int v = tid; v < NKEY * VPR; v += 256) {
     const int key = v / VPR, e = (v - key * VPR) * 8;
     if (key0 + key >= Lk || e >= D) continue;
-    const float *s0 = red + (size_t)key * LDR + e, *s1 = s0 + 64 * LDR;
+    const float *s0 = red + (size_t)key * LDR + e, *s1 = s0 + NKEY * LDR;
     Pack8 ov, ok;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
@@ -1059,15 +1102,15 @@ __global__ void zero_f32_kernel(float *p, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.f;
 }
 
-template <typename T, int HD, bool DQP>
+template <typename T, int HD, bool DQP, int KB>
 static int launch_dkdv(const fmoba_attn_bwd_args &a, const BwdWs &ws, hipStream_t s) {
-  auto kern = attn_bwd_dkdv_kernel<T, HD, DQP>;
+  auto kern = attn_bwd_dkdv_kernel<T, HD, DQP, KB>;
   const size_t smem = BwdSmem<HD>::bytes;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("attn_bwd: cannot reserve %zu bytes of LDS", smem);
     return 2;
   }
-  const int64_t items = (int64_t)a.batch * a.heads * ceil_div(a.max_seqlen_k, 64);
+  const int64_t items = (int64_t)a.batch * a.heads * ceil_div(a.max_seqlen_k, 64 * KB);
   if (items >= ((int64_t)1 << 31)) {
     set_error("attn_bwd: too many (sequence, head, key block) work items");
     return 1;
@@ -1116,11 +1159,13 @@ static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hi
   }
   if (phases & FMOBA_BWD_DKDV) {
     int rc;
+    // columns of a multiple of 128 keys: one workgroup per 128 keys (the two 64-key blocks share their row list)
+    const bool wide = a.lg_block_n % 128 == 0;
     if (partials) {
       hipLaunchKernelGGL(zero_i32_kernel, dim3(512), dim3(256), 0, s, ws.cnt, (int64_t)a.total_q * a.heads);
-      rc = a.head_dim <= 64 ? launch_dkdv<T, 64, true>(a, ws, s) : launch_dkdv<T, 128, true>(a, ws, s);
+      rc = a.head_dim <= 64 ? launch_dkdv<T, 64, true, 1>(a, ws, s) : (wide ? launch_dkdv<T, 128, true, 2>(a, ws, s) : launch_dkdv<T, 128, true, 1>(a, ws, s));
     } else {
-      rc = a.head_dim <= 64 ? launch_dkdv<T, 64, false>(a, ws, s) : launch_dkdv<T, 128, false>(a, ws, s);
+      rc = a.head_dim <= 64 ? launch_dkdv<T, 64, false, 1>(a, ws, s) : (wide ? launch_dkdv<T, 128, false, 2>(a, ws, s) : launch_dkdv<T, 128, false, 1>(a, ws, s));
     }
     if (rc) return rc;
   }
