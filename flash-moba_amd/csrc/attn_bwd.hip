@@ -36,7 +36,7 @@ template <int HD>
 struct BwdSmem {
   // The gathered Q / dO tiles have rows of exactly HD elements (the loads that fill them write 64 lanes x 16 bytes
   // to consecutive addresses) and are swizzled instead of padded: the 16-byte piece c of tile row r lies at piece
-  // c ^ bwd_swz<HD>(r).  With that, the 16-byte row reads (lane -> row lane % 32) and the transposing 8-byte
+  // c ^ tile_swz<HD>(r).  With that, the 16-byte row reads (lane -> row lane % 32) and the transposing 8-byte
   // reads both spread over all banks.
   static constexpr int LDQ = HD + 16;  // elements, K and V while they are read into registers (plain padded rows)
   static constexpr int LDS_ = 32 + 8;  // elements, dS^T tile rows [key][32 rows]
@@ -55,69 +55,6 @@ struct BwdSmem {
   static_assert((size_t)2 * 128 * LDQ * 2 <= 16 * tileBytes, "K and V pass through the tiles");
   static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
 };
-
-// piece c of tile row r is stored at piece c ^ bwd_swz<HD>(r)
-template <int HD>
-__device__ __forceinline__ int bwd_swz(int r) {
-  if constexpr (HD > 64)
-    return ((r & 3) << 2) | ((r >> 2) & 3);  // 16 pieces per row, one row per sweep of the banks
-  else
-    return (((r >> 1) & 1) << 2) | ((r >> 2) & 1);  // 8 pieces per row, two rows per sweep
-}
-template <int HD>
-struct BwdSwz {
-  static constexpr int kRow8 = HD > 64 ? 2 : 0;  // bwd_swz(r + 8) ^ bwd_swz(r)
-};
-
-typedef __attribute__((address_space(3))) const Pack8 lds_cpack8;
-__device__ __forceinline__ Pack8 lds_read16(uint32_t byte_addr) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  return *(lds_cpack8 *)byte_addr;
-#else
-  (void)byte_addr;
-  return Pack8{{0, 0, 0, 0}};
-#endif
-}
-template <typename V>
-__device__ __forceinline__ V lds_read_vec(uint32_t byte_addr) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  return *(__attribute__((address_space(3))) const V *)byte_addr;
-#else
-  (void)byte_addr;
-  return V{};
-#endif
-}
-// 8 x 16-bit operand of a transposing read: two 8-byte reads
-__device__ __forceinline__ Pack8 lds_tr8(uint32_t addr_lo, uint32_t addr_hi) {
-  Pack8 r;
-#if defined(__HIP_DEVICE_COMPILE__)
-  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)addr_lo);
-  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)addr_hi);
-  __builtin_memcpy(&r.w[0], &lo, 8);
-  __builtin_memcpy(&r.w[2], &hi, 8);
-#else
-  (void)addr_lo, (void)addr_hi;
-  r = Pack8{{0, 0, 0, 0}};
-#endif
-  return r;
-}
-// 64 lanes x 16 bytes from each lane's own global address to LDS bytes [lds_base, lds_base + 1024), lane order;
-// lds_base is the same for the whole wave.  Written as assembly because the compiler makes every later LDS read wait
-// for a load that it knows to write LDS, and these are meant to stay in flight for a whole round: the kernel waits for
-// them itself (wait_all_loads) before the barrier that hands the tiles over.  Nothing else in the kernel uses m0.
-__device__ __forceinline__ void global_to_lds16(const void *g, uint32_t lds_base) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base) : "memory");
-#else
-  (void)g, (void)lds_base;
-#endif
-}
-__device__ __forceinline__ void wait_all_loads() {
-#if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
-}
-__device__ uint4 g_bwd_zero16;  // 16 zero bytes: what the tile loads fetch for absent rows and for features past head_dim
 
 struct BwdWs {
   int32_t *cnt;    // [total_q * heads] visits handed out per (row, head)
@@ -310,12 +247,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       constexpr int RPI = 64 / VPR, NI = 32 / RPI;  // tile rows per instruction, instructions per tile
       const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
       const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(((sr & 1) * 4 + wave) * (int)TB);
-      const uint16_t *zero = reinterpret_cast<const uint16_t *>(&g_bwd_zero16);
+      const uint16_t *zero = reinterpret_cast<const uint16_t *>(&g_zero16);
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int row = i * RPI + rl;
         const int rid = sRid[(sr & 1) * kBwdRoundRows + wave * 32 + row];
-        const int e = (p ^ bwd_swz<HD>(row)) * 8;
+        const int e = (p ^ tile_swz<HD>(row)) * 8;
         const bool ok = (rid >= 0) & (e < D);
         const uint16_t *gq = ok ? qg + (int64_t)rid * a.q_row_stride + e : zero;
         const uint16_t *gd = ok ? dog + (int64_t)rid * a.do_row_stride + e : zero;
@@ -349,9 +286,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     // hh * KS ..) and transposing reads (row (lane % 16) / 4 + 4 hh, feature tile 0); every other operand is an
     // exclusive-or on the piece bits plus a constant
     const uint32_t pairQ = ldsQ + (uint32_t)(px * 2) * TB, pairdO = ldsdO + (uint32_t)(px * 2) * TB;
-    const uint32_t rowoff = (uint32_t)((lane & 31) * RB + (((hh * KS) ^ bwd_swz<HD>(lane & 31)) * 16));
+    const uint32_t rowoff = (uint32_t)((lane & 31) * RB + (((hh * KS) ^ tile_swz<HD>(lane & 31)) * 16));
     const int li = lane & 15, r0t = (li >> 2) + 4 * hh;
-    const uint32_t troff = (uint32_t)(r0t * RB + ((((((lane >> 4) & 1) * 2 + ((li & 3) >> 1))) ^ bwd_swz<HD>(r0t)) * 16) + (li & 1) * 8);
+    const uint32_t troff = (uint32_t)(r0t * RB + ((((((lane >> 4) & 1) * 2 + ((li & 3) >> 1))) ^ tile_swz<HD>(r0t)) * 16) + (li & 1) * 8);
     // (re-made opaque wherever they are used: the operand addresses derived from them must not be kept in
     // registers from one use to the next, there are none to spare)
     const uint32_t aQ = pairQ + rowoff, adO = pairdO + rowoff, tQ = pairQ + troff, tdO = pairdO + troff;
@@ -414,7 +351,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       for (int t = 0; t < BC; ++t) {
         const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
         // rows 16 s2 + (0..3) + 4 hh and the same + 8, features dt * 32 ..
-        const uint32_t xlo = (uint32_t)(dt * 4 * 16), xhi = (uint32_t)(((dt * 4) ^ BwdSwz<HD>::kRow8) * 16);
+        const uint32_t xlo = (uint32_t)(dt * 4 * 16), xhi = (uint32_t)(((dt * 4) ^ TileSwz<HD>::kRow8) * 16);
         const uint32_t olo = TO + (uint32_t)(16 * s2 * RB), ohi = olo + (uint32_t)(8 * RB);
         dot[G & 1][t] = lds_tr8((bo ^ xlo) + olo, (bo ^ xhi) + ohi);
         qt[G & 1][t] = lds_tr8((bq ^ xlo) + olo, (bq ^ xhi) + ohi);

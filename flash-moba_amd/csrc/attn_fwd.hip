@@ -18,8 +18,9 @@
 // Work and traffic are proportional to the number of (row, key block) visits whatever the number of
 // chunks per sequence; a row-stationary formulation degenerates when every 128-row block touches
 // thousands of chunks with one or two rows each.
-// In the first kernel two or four waves compute (one tile each per round) and two more only move data
-// (global -> registers -> LDS), two rounds ahead.
+// In the first kernel all four waves compute (one tile each per round, one wave per SIMD: K of the block and
+// the operands of a tile take most of its registers); the gathered Q rows go from global memory straight to
+// LDS (global_load_lds), one round ahead.
 #include "fmoba_common.h"
 
 #include <algorithm>
@@ -28,23 +29,24 @@
 
 namespace fmoba {
 
-constexpr int kFwdListCap = 4096;  // rows of a column list held in LDS at a time
 constexpr int kFwdRowsDensity = 6;  // row-block form when a row selects at least 1/6 of the chunks it may see
 
-// NCW compute waves (one 32-row tile each per round) + 2 loader waves
-template <int HD, int KB, int NCW>
+constexpr int kFwdRoundRows = 128;  // rows of a column list per round: one 32-row tile per wave
+
+template <int HD, int KB>
 struct FwdColSmem {
-  static constexpr int RR = 32 * NCW;  // rows per round
-  static constexpr int LDQ = HD + 16;  // elements, K / V / Q tiles (conflict-free for the 16-byte row reads and the transposing reads)
+  static constexpr int LDQ = HD + 16;  // elements, K / V rows (conflict-free for the 16-byte row reads and the transposing reads)
   static constexpr int LDO = HD + 8;   // elements, per-wave output tile [32 rows][LDO]
-  static constexpr size_t oK = 0;
-  static constexpr size_t oV = oK + (size_t)KB * LDQ * 2;
-  static constexpr size_t oQ = oV + (size_t)KB * LDQ * 2;            // [2 buffers][RR rows][LDQ]
-  static constexpr size_t oOut = oQ + (size_t)2 * RR * LDQ * 2;      // [NCW waves][32][LDO]
-  static constexpr size_t oRow = oOut + (size_t)NCW * 32 * LDO * 2;  // int[2][RR]
-  static constexpr size_t oSlot = oRow + 2 * RR * 4;                 // int[2][RR]
-  static constexpr size_t oList = oSlot + 2 * RR * 4;                // int[kFwdListCap]
-  static constexpr size_t bytes = oList + (size_t)kFwdListCap * 4;
+  static constexpr size_t tileBytes = (size_t)32 * HD * 2;  // a gathered Q tile: rows of exactly HD elements, swizzled
+  static constexpr size_t oV = 0;
+  static constexpr size_t oQ = oV + (size_t)KB * LDQ * 2;           // [2 buffers][4 tiles][32][HD]; K passes through it on its way to registers
+  static constexpr size_t oOut = oQ + 8 * tileBytes;                 // [4 waves][32][LDO]
+  static constexpr size_t oRid = oOut + (size_t)4 * 32 * LDO * 2;    // int[2][128]: row ids, one round before the rest
+  static constexpr size_t oRow = oRid + 2 * kFwdRoundRows * 4;       // int[2][128]
+  static constexpr size_t oSlot = oRow + 2 * kFwdRoundRows * 4;      // int[2][128]
+  static constexpr size_t bytes = oSlot + 2 * kFwdRoundRows * 4;
+  static_assert((size_t)KB * LDQ * 2 <= 8 * tileBytes + (size_t)4 * 32 * LDO * 2, "K passes through the Q tiles and the output tiles");
+  static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
 };
 
 struct FwdWs {
@@ -54,20 +56,19 @@ struct FwdWs {
   int32_t cap;
 };
 
-template <typename T, int HD, int KB, int NCW>
-__global__ __launch_bounds__((NCW + 2) * 64) void attn_fwd_col_kernel(fmoba_attn_fwd_args a, FwdWs ws) {
-  typedef FwdColSmem<HD, KB, NCW> SM;
-  constexpr int NTHR = (NCW + 2) * 64, RR = SM::RR;
+template <typename T, int HD, int KB>
+__global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a, FwdWs ws) {
+  typedef FwdColSmem<HD, KB> SM;
+  constexpr int NTHR = 256;
   constexpr int KS = HD / 16, LDQ = SM::LDQ, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
   constexpr int KT = KB / 32;                 // 32-key tiles of the block
-  constexpr int NV = RR * VPR / 128;          // 16-byte vectors of a round's gathered Q rows per loader thread
+  constexpr uint32_t TB = (uint32_t)SM::tileBytes;
+  constexpr int RB = HD * 2;                  // bytes of a tile row
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint16_t *sK = reinterpret_cast<uint16_t *>(smem + SM::oK);
   uint16_t *sV = reinterpret_cast<uint16_t *>(smem + SM::oV);
-  uint16_t *sQ = reinterpret_cast<uint16_t *>(smem + SM::oQ);
+  int *sRid = reinterpret_cast<int *>(smem + SM::oRid);
   int *sRow = reinterpret_cast<int *>(smem + SM::oRow);
   int *sSlot = reinterpret_cast<int *>(smem + SM::oSlot);
-  int *sList = reinterpret_cast<int *>(smem + SM::oList);
 
   const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + KB - 1) / KB);
   const int nb = item.idx, b = item.pair / a.heads, h = item.pair - b * a.heads;
@@ -79,27 +80,28 @@ __global__ __launch_bounds__((NCW + 2) * 64) void attn_fwd_col_kernel(fmoba_attn
   const int D = a.head_dim;
   const int hk = h / (a.heads / a.heads_k);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
-  const bool is_loader = wave >= NCW;
-  const int lt = tid - NCW * 64;
   const bool causal = a.is_causal != 0;
   const float scale_log2 = a.softmax_scale * 1.4426950408889634f;
 
-  // ---- K and V of the block ------------------------------------------------------------------
+  // ---- K and V of the block: the loads are issued first and stored after the look-up of the column list, so
+  // that the two chains of dependent loads wait together (one workgroup per compute unit: nothing else covers them)
+  constexpr int NKV = KB * VPR / NTHR;
+  Pack8 xk[NKV], xv[NKV];
   {
     const uint16_t *kp = reinterpret_cast<const uint16_t *>(a.k) + (int64_t)(k0 + key0) * a.k_row_stride + (int64_t)hk * a.k_head_stride;
     const uint16_t *vp = reinterpret_cast<const uint16_t *>(a.v) + (int64_t)(k0 + key0) * a.v_row_stride + (int64_t)hk * a.v_head_stride;
-    for (int v = tid; v < KB * VPR; v += NTHR) {
+#pragma unroll
+    for (int i = 0; i < NKV; ++i) {
+      const int v = tid + NTHR * i;
       const int key = v / VPR, e = (v - key * VPR) * 8;
-      Pack8 xk = zero_pack8(), xv = zero_pack8();
+      xk[i] = zero_pack8();
+      xv[i] = zero_pack8();
       if (key0 + key < Lk && e < D) {
-        xk = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
-        xv = ld_global16(vp + (int64_t)key * a.v_row_stride + e);
+        xk[i] = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
+        xv[i] = ld_global16(vp + (int64_t)key * a.v_row_stride + e);
       }
-      *reinterpret_cast<Pack8 *>(sK + key * LDQ + e) = xk;
-      *reinterpret_cast<Pack8 *>(sV + key * LDQ + e) = xv;
     }
   }
-  __syncthreads();
 
   // ---- the block's column list --------------------------------------------------------------------
   const int Bn = a.lg_block_n;
@@ -113,227 +115,242 @@ __global__ __launch_bounds__((NCW + 2) * 64) void attn_fwd_col_kernel(fmoba_attn
     lbase = a.col_offsets[bh * a.max_cols + c];
     if (causal && nnz > 0) start = lower_bound_wave_i32(a.row_indices + lbase, nnz, key0 - off);  // earlier rows see no key of the block
   }
-  const int32_t *list = a.row_indices + lbase;
+  const int32_t *list = a.row_indices + lbase + start;
+  const int n = nnz - start;  // rows of the list that the block walks
+  const int nround = (n + kFwdRoundRows - 1) / kFwdRoundRows;
+  const int ntile = (n + 31) >> 5;
   const uint16_t *qg = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)q0 * a.q_row_stride + (int64_t)h * a.q_head_stride;
   int32_t *cntg = ws.cnt + (int64_t)q0 * a.heads + h;       // counter of local row r: cntg[r * heads]
-
-  auto fill_list = [&](int seg0, int seg_len) {
-    __syncthreads();
-    for (int i = tid; i < seg_len; i += NTHR) {
-      const int r = list[seg0 + i];
-      sList[i] = (r >= 0 && r < Lq) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
+  if (nround == 0) return;
+  int rid01[2] = {-1, -1};  // threads 0..127: row ids of rounds 0 and 1
+  if (tid < kFwdRoundRows) {
+#pragma unroll
+    for (int sr = 0; sr < 2; ++sr) {
+      const int j = sr * kFwdRoundRows + tid;
+      const int r = list[min(j, n - 1)];
+      rid01[sr] = ((j < n) & (r >= 0) & (r < Lq)) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
     }
-    __syncthreads();
-  };
-  typedef std::integral_constant<int, 0> C0;
-  typedef std::integral_constant<int, 1> C1;
-
-  // The two roles run separate code with the same barrier sequence (register allocation, exact load counting).
-  if (is_loader) {
-    // two-deep rings of the gathered rows of two rounds; loads are unconditional (indices clamped, the
-    // surplus zeroed when stored) so that the compiler counts outstanding loads exactly
-    Pack8 lq[2][NV];
-    int lrow[2] = {-1, -1}, lslot[2] = {0, 0};
-    for (int seg0 = start; seg0 < nnz; seg0 += kFwdListCap) {
-      const int seg_len = min(kFwdListCap, nnz - seg0);
-      fill_list(seg0, seg_len);
-      const int nround = (seg_len + RR - 1) / RR;
-      auto load_round = [&](auto par, int r) {
-        constexpr int P = decltype(par)::value;
+  }
+  {
+    uint16_t *sK = reinterpret_cast<uint16_t *>(smem + SM::oQ);
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-          const int v = lt + 128 * i;
-          const int row = v / VPR, e = min((v - row * VPR) * 8, D - 8);
-          const int j = min(r * RR + row, seg_len - 1);
-          const int rid = max(sList[j], 0);
-          lq[P][i] = ld_global16(qg + (int64_t)rid * a.q_row_stride + e);
-        }
-        if (lt < RR) {
-          const int j = r * RR + lt;
-          const int rid = j < seg_len ? sList[j] : -1;
-          lrow[P] = rid;
-          // every visit of a (row, key block) pair takes one slot of the row (the only conditional memory
-          // operation of the loader: a shared dummy counter would serialise the whole grid on one address)
-          if (rid >= 0) lslot[P] = atomicAdd(cntg + (int64_t)rid * a.heads, 1);
-        }
-      };
-      auto store_round = [&](auto par, int r) {
-        constexpr int P = decltype(par)::value;
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-          const int v = lt + 128 * i;
-          const int row = v / VPR, e = (v - row * VPR) * 8;
-          const int j = r * RR + row;
-          const bool ok = (e < D) & (j < seg_len) & (sList[min(j, seg_len - 1)] >= 0);
-          Pack8 x = lq[P][i];
-#pragma unroll
-          for (int w = 0; w < 4; ++w) x.w[w] = ok ? x.w[w] : 0u;
-          *reinterpret_cast<Pack8 *>(sQ + (P * RR + row) * LDQ + e) = x;
-        }
-        if (lt < RR) {
-          sRow[P * RR + lt] = lrow[P];
-          sSlot[P * RR + lt] = lslot[P];
-        }
-      };
-      load_round(C0{}, 0);
-      load_round(C1{}, 1);  // past the end: rows clamp to the last one, nothing of it is used
-      store_round(C0{}, 0);
-      load_round(C0{}, 2);
-      auto loader_round = [&](auto par, int r) {  // par: parity of round r + 1
-        __syncthreads();  // round r is in LDS; the readers of round r-1 are done with the other buffer
-        if (r + 1 < nround) store_round(par, r + 1);
-        load_round(par, r + 3);
-      };
-      const int nround_pad = (nround + 1) & ~1;
-      for (int r = 0; r < nround_pad; r += 2) {
-        loader_round(C1{}, r);
-        loader_round(C0{}, r + 1);
-      }
+    for (int i = 0; i < NKV; ++i) {
+      const int v = tid + NTHR * i;
+      const int key = v / VPR, e = (v - key * VPR) * 8;
+      *reinterpret_cast<Pack8 *>(sK + key * LDQ + e) = xk[i];
+      *reinterpret_cast<Pack8 *>(sV + key * LDQ + e) = xv[i];
     }
-  } else {
-    // K of this block as the A operand of S^T = K Q^T: lane -> key (lane % 32) of each 32-key tile
-    Pack8 kfr[KT][KS];
+  }
+  __syncthreads();
+  // K of this block as the A operand of S^T = K Q^T: lane -> key (lane % 32) of each 32-key tile
+  Pack8 kfr[KT][KS];
+  {
+    const uint16_t *sK = reinterpret_cast<const uint16_t *>(smem + SM::oQ);
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
         kfr[kt][ks] = *reinterpret_cast<const Pack8 *>(sK + (kt * 32 + (lane & 31)) * LDQ + (hh * KS + ks) * 8);
-    lds_cu16 *trV = tr_lane_base(sV, LDQ, lane) + 4 * hh * LDQ;
-    uint16_t *sOut = reinterpret_cast<uint16_t *>(smem + SM::oOut) + (size_t)wave * 32 * LDO;
+  }
+  if (tid < kFwdRoundRows) {
+    sRid[tid] = rid01[0];
+    sRid[kFwdRoundRows + tid] = rid01[1];
+  }
+  __syncthreads();  // K is in registers; the row ids of rounds 0 and 1 are in LDS
 
-    for (int seg0 = start; seg0 < nnz; seg0 += kFwdListCap) {
-      const int seg_len = min(kFwdListCap, nnz - seg0);
-      fill_list(seg0, seg_len);
-      const int ntile = (seg_len + 31) >> 5;
-      const int nround = (seg_len + RR - 1) / RR;
-      const int nround_pad = (nround + 1) & ~1;
+  // ---- feeding the tiles: all four waves compute, nothing passes through registers.  Every wave fetches the tile
+  // it will work on in the NEXT round with loads that write straight to LDS, issued at the start of a round and
+  // awaited at its end.  Threads 0..127 carry the per-row scalars: the row id of round s+2 (it has to be in LDS one
+  // round before the tile loads that use it) and the partial slot of round s+1.
+  typedef std::integral_constant<int, 0> C0;
+  typedef std::integral_constant<int, 1> C1;
+  const uint32_t ldsQ = (uint32_t)(uintptr_t)(smem + SM::oQ);
+  int n_rid = -1, m_rid = -1, m_slot = 0;
+  int ft = tid;  // thread index for the feeding code, re-made opaque in every round: what is derived from it must not be kept in registers across rounds
+  auto rid_issue = [&](int sr) {
+    if (tid < kFwdRoundRows) {
+      const int j = sr * kFwdRoundRows + ft;
+      const int r = list[min(j, n - 1)];
+      n_rid = ((j < n) & (r >= 0) & (r < Lq)) ? r : -1;
+    }
+  };
+  auto rid_store = [&](int sr) {
+    if (tid < kFwdRoundRows) sRid[(sr & 1) * kFwdRoundRows + ft] = n_rid;
+  };
+  auto meta_issue = [&](int sr) {
+    if (tid < kFwdRoundRows) {
+      m_rid = sRid[(sr & 1) * kFwdRoundRows + ft];
+      // every visit of a (row, key block) pair takes one slot of the row (a shared dummy counter for absent
+      // rows would serialise the whole grid on one address)
+      if (m_rid >= 0) m_slot = atomicAdd(cntg + (int64_t)m_rid * a.heads, 1);
+    }
+  };
+  auto meta_store = [&](int sr) {
+    if (tid < kFwdRoundRows) {
+      sRow[(sr & 1) * kFwdRoundRows + ft] = m_rid;
+      sSlot[(sr & 1) * kFwdRoundRows + ft] = m_slot;
+    }
+  };
+  auto tile_issue = [&](int sr) {  // tile `wave` of round sr
+    constexpr int RPI = 64 / VPR, NI = 32 / RPI;  // tile rows per instruction, instructions per tile
+    const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
+    const uint32_t dst = ldsQ + (uint32_t)__builtin_amdgcn_readfirstlane(((sr & 1) * 4 + wave) * (int)TB);
+    const uint16_t *zero = reinterpret_cast<const uint16_t *>(&g_zero16);
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int row = i * RPI + rl;
+      const int rid = sRid[(sr & 1) * kFwdRoundRows + wave * 32 + row];
+      const int e = (p ^ tile_swz<HD>(row)) * 8;
+      const bool ok = (rid >= 0) & (e < D);
+      global_to_lds16(ok ? qg + (int64_t)rid * a.q_row_stride + e : zero, dst + (uint32_t)(i * RPI * RB));
+    }
+  };
+  meta_issue(0);
+  tile_issue(0);
+  meta_store(0);
+  wait_all_loads();
+  __syncthreads();
 
-      auto process_tile = [&](auto pc, int tile) {
-        constexpr int PB = decltype(pc)::value;
-        const int sidx = PB * RR + wave * 32 + (lane & 31);
-        const int rid = sRow[sidx];
-        // this lane's query row as the B operand
-        Pack8 qb[KS];
+  lds_cu16 *trV = tr_lane_base(sV, LDQ, lane) + 4 * hh * LDQ;
+  uint16_t *sOut = reinterpret_cast<uint16_t *>(smem + SM::oOut) + (size_t)wave * 32 * LDO;
+  // byte address of this lane's row (lane % 32 of the wave's tile, buffer 0), piece hh * KS; the other pieces
+  // are an exclusive-or on the piece bits
+  const uint32_t qrow = ldsQ + (uint32_t)wave * TB + (uint32_t)((lane & 31) * RB + (((hh * KS) ^ tile_swz<HD>(lane & 31)) * 16));
+
+  auto process_tile = [&](auto pc) {
+    constexpr int PB = decltype(pc)::value;
+    const int sidx = PB * kFwdRoundRows + wave * 32 + (lane & 31);
+    const int rid = sRow[sidx];
+    // this lane's query row as the B operand
+    Pack8 qb[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qb[ks] = *reinterpret_cast<const Pack8 *>(sQ + (size_t)sidx * LDQ + (hh * KS + ks) * 8);
-        __builtin_amdgcn_sched_barrier(0);
-        f32x16 st[KT];  // S^T: register i of tile kt <-> key kt*32 + acc_row(i, hh), this lane's row
+    for (int ks = 0; ks < KS; ++ks) qb[ks] = lds_read16((qrow ^ (uint32_t)(ks * 16)) + (uint32_t)(PB * 4) * TB);
+    __builtin_amdgcn_sched_barrier(0);
+    f32x16 st[KT];  // S^T: register i of tile kt <-> key kt*32 + acc_row(i, hh), this lane's row
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
+    for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) st[kt][i] = 0.f;
+      for (int i = 0; i < 16; ++i) st[kt][i] = 0.f;
 #pragma unroll
-          for (int ks = 0; ks < KS; ++ks) st[kt] = mfma32<T>(kfr[kt][ks], qb[ks], st[kt]);
+      for (int ks = 0; ks < KS; ++ks) st[kt] = mfma32<T>(kfr[kt][ks], qb[ks], st[kt]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // V^T operands of the first half of the feature tiles: their LDS latency runs under the softmax arithmetic
+    Pack8 vt[NDT][KT][2];
+#pragma unroll
+    for (int dt = 0; dt < NDT / 2; ++dt)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const int lo = (kt * 32 + 16 * s2) * LDQ + dt * 32;
+          vt[dt][kt][s2] = tr_frag8_at(trV, lo, lo + 8 * LDQ);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        // V^T operands of the first half of the feature tiles: their LDS latency runs under the softmax arithmetic
-        Pack8 vt[NDT][KT][2];
+    __builtin_amdgcn_sched_barrier(0);
+    // block-local softmax of the row, log2 domain; keys beyond lim are masked
+    const int lim = rid < 0 ? -1 : min(causal ? rid + off : 0x7fffffff, Lk - 1) - key0;  // last visible key, relative
+    float m = -INFINITY;
+    if (__all(lim >= KB - 1)) {
 #pragma unroll
-        for (int dt = 0; dt < NDT / 2; ++dt)
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          st[kt][i] *= scale_log2;
+          m = fmaxf(m, st[kt][i]);
+        }
+    } else {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int jrel = kt * 32 + 8 * (i >> 2) + (i & 3) + 4 * hh;
+          st[kt][i] = jrel <= lim ? st[kt][i] * scale_log2 : -INFINITY;
+          m = fmaxf(m, st[kt][i]);
+        }
+    }
+    m = max_xor32_f(m);
+    const float m_use = m == -INFINITY ? 0.f : m;
+    float l = 0.f;
+    Pack8 pf[KT][2];  // P^T as the B operand of O^T = V^T P^T, straight from the accumulators
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const float p0 = __builtin_amdgcn_exp2f(st[kt][8 * s2 + 2 * w] - m_use);
+          const float p1 = __builtin_amdgcn_exp2f(st[kt][8 * s2 + 2 * w + 1] - m_use);
+          l += p0 + p1;
+          pf[kt][s2].w[w] = pack2<T>(p0, p1);
+        }
+    l = sum_xor32_f(l);
+    __builtin_amdgcn_sched_barrier(0);
+    // O^T[d][row] = sum_key V^T[d][key] P^T[key][row]; register i of d-tile dt <-> d = dt*32 + acc_row(i, hh)
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      if (dt == 0) {  // second half of the V^T operands, under the first products
+#pragma unroll
+        for (int d2 = NDT / 2; d2 < NDT; ++d2)
 #pragma unroll
           for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
-              const int lo = (kt * 32 + 16 * s2) * LDQ + dt * 32;
-              vt[dt][kt][s2] = tr_frag8_at(trV, lo, lo + 8 * LDQ);
+              const int lo = (kt * 32 + 16 * s2) * LDQ + d2 * 32;
+              vt[d2][kt][s2] = tr_frag8_at(trV, lo, lo + 8 * LDQ);
             }
         __builtin_amdgcn_sched_barrier(0);
-        // block-local softmax of the row, log2 domain; keys beyond lim are masked
-        const int lim = rid < 0 ? -1 : min(causal ? rid + off : 0x7fffffff, Lk - 1) - key0;  // last visible key, relative
-        float m = -INFINITY;
-        if (__all(lim >= KB - 1)) {
+      }
+      f32x16 o;
 #pragma unroll
-          for (int kt = 0; kt < KT; ++kt)
+      for (int i = 0; i < 16; ++i) o[i] = 0.f;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              st[kt][i] *= scale_log2;
-              m = fmaxf(m, st[kt][i]);
-            }
-        } else {
+      for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-          for (int kt = 0; kt < KT; ++kt)
+        for (int s2 = 0; s2 < 2; ++s2) o = mfma32<T>(vt[dt][kt][s2], pf[kt][s2], o);
+      // to the wave's row-major output tile, four features (8 bytes) at a time
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int jrel = kt * 32 + 8 * (i >> 2) + (i & 3) + 4 * hh;
-              st[kt][i] = jrel <= lim ? st[kt][i] * scale_log2 : -INFINITY;
-              m = fmaxf(m, st[kt][i]);
-            }
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<uint2 *>(sOut + (lane & 31) * LDO + dt * 32 + 8 * g + 4 * hh) =
+            make_uint2(pack2<T>(o[4 * g], o[4 * g + 1]), pack2<T>(o[4 * g + 2], o[4 * g + 3]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // header of the partial
+    const int slot = sSlot[sidx];
+    const bool keep = rid >= 0 && slot < ws.cap;
+    const int64_t pidx = ((int64_t)(q0 + max(rid, 0)) * a.heads + h) * ws.cap + slot;
+    if (keep && hh == 0) ws.hdr[pidx] = make_float4(m, l, __int_as_float(nb), 0.f);
+    wave_lds_fence();
+    // rows leave as 16-byte pieces: lane -> (row 4k + lane / 16, features 8 * (lane % 16))
+    if ((lane & 15) * 8 < D) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int row = 4 * k + (lane >> 4);
+        const int r2 = sRow[PB * kFwdRoundRows + wave * 32 + row], s2 = sSlot[PB * kFwdRoundRows + wave * 32 + row];
+        if (r2 >= 0 && s2 < ws.cap) {
+          const Pack8 x = *reinterpret_cast<const Pack8 *>(sOut + row * LDO + (lane & 15) * 8);
+          *reinterpret_cast<Pack8 *>(ws.part + (((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2) * D + (lane & 15) * 8) = x;
         }
-        m = max_xor32_f(m);
-        const float m_use = m == -INFINITY ? 0.f : m;
-        float l = 0.f;
-        Pack8 pf[KT][2];  // P^T as the B operand of O^T = V^T P^T, straight from the accumulators
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-              const float p0 = __builtin_amdgcn_exp2f(st[kt][8 * s2 + 2 * w] - m_use);
-              const float p1 = __builtin_amdgcn_exp2f(st[kt][8 * s2 + 2 * w + 1] - m_use);
-              l += p0 + p1;
-              pf[kt][s2].w[w] = pack2<T>(p0, p1);
-            }
-        l = sum_xor32_f(l);
-        __builtin_amdgcn_sched_barrier(0);
-        // O^T[d][row] = sum_key V^T[d][key] P^T[key][row]; register i of d-tile dt <-> d = dt*32 + acc_row(i, hh)
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-          if (dt == 0) {  // second half of the V^T operands, under the first products
-#pragma unroll
-            for (int d2 = NDT / 2; d2 < NDT; ++d2)
-#pragma unroll
-              for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                for (int s2 = 0; s2 < 2; ++s2) {
-                  const int lo = (kt * 32 + 16 * s2) * LDQ + d2 * 32;
-                  vt[d2][kt][s2] = tr_frag8_at(trV, lo, lo + 8 * LDQ);
-                }
-            __builtin_amdgcn_sched_barrier(0);
-          }
-          f32x16 o;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[i] = 0.f;
-#pragma unroll
-          for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2) o = mfma32<T>(vt[dt][kt][s2], pf[kt][s2], o);
-          // to the wave's row-major output tile, four features (8 bytes) at a time
-#pragma unroll
-          for (int g = 0; g < 4; ++g)
-            *reinterpret_cast<uint2 *>(sOut + (lane & 31) * LDO + dt * 32 + 8 * g + 4 * hh) =
-                make_uint2(pack2<T>(o[4 * g], o[4 * g + 1]), pack2<T>(o[4 * g + 2], o[4 * g + 3]));
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        // header of the partial
-        const int slot = sSlot[sidx];
-        const bool keep = rid >= 0 && slot < ws.cap;
-        const int64_t pidx = ((int64_t)(q0 + max(rid, 0)) * a.heads + h) * ws.cap + slot;
-        if (keep && hh == 0) ws.hdr[pidx] = make_float4(m, l, __int_as_float(nb), 0.f);
-        wave_lds_fence();
-        // rows leave as 16-byte pieces: lane -> (row 4k + lane / 16, features 8 * (lane % 16))
-        if ((lane & 15) * 8 < D) {
-#pragma unroll
-          for (int k = 0; k < 8; ++k) {
-            const int row = 4 * k + (lane >> 4);
-            const int r2 = sRow[PB * RR + wave * 32 + row], s2 = sSlot[PB * RR + wave * 32 + row];
-            if (r2 >= 0 && s2 < ws.cap) {
-              const Pack8 x = *reinterpret_cast<const Pack8 *>(sOut + row * LDO + (lane & 15) * 8);
-              *reinterpret_cast<Pack8 *>(ws.part + (((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2) * D + (lane & 15) * 8) = x;
-            }
-          }
-        }
-        wave_lds_fence();
-        (void)tile;
-      };
-
-      for (int r = 0; r < nround_pad; r += 2) {
-        __syncthreads();  // round r is in LDS
-        if (NCW * r + wave < ntile) process_tile(C0{}, NCW * r + wave);
-        __syncthreads();
-        if (NCW * (r + 1) + wave < ntile) process_tile(C1{}, NCW * (r + 1) + wave);
       }
     }
+    wave_lds_fence();
+  };
+
+  auto round = [&](auto pc, int r) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" : "+v"(ft));
+#endif
+    rid_issue(r + 2);
+    meta_issue(r + 1);
+    tile_issue(r + 1);
+    if (4 * r + wave < ntile) process_tile(pc);
+    meta_store(r + 1);
+    rid_store(r + 2);
+    wait_all_loads();
+    __syncthreads();  // round r + 1 is in LDS; everyone is done with round r
+  };
+  for (int r = 0; r < nround; r += 2) {
+    round(C0{}, r);
+    if (r + 1 < nround) round(C1{}, r + 1);
   }
 }
 
@@ -480,10 +497,8 @@ static bool fwd_use_rows(const fmoba_attn_fwd_args &a) {
 
 template <typename T, int HD, int KB>
 static int launch_fwd_col(const fmoba_attn_fwd_args &a, const FwdWs &ws, hipStream_t s) {
-  // 64-key blocks leave room (registers, LDS) for four compute waves; 128-key blocks for two
-  constexpr int NCW = KB == 64 ? 4 : 2;
-  auto kern = attn_fwd_col_kernel<T, HD, KB, NCW>;
-  const size_t smem = FwdColSmem<HD, KB, NCW>::bytes;
+  auto kern = attn_fwd_col_kernel<T, HD, KB>;
+  const size_t smem = FwdColSmem<HD, KB>::bytes;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("attn_fwd: cannot reserve %zu bytes of LDS", smem);
     return 2;
@@ -493,7 +508,7 @@ static int launch_fwd_col(const fmoba_attn_fwd_args &a, const FwdWs &ws, hipStre
     set_error("attn_fwd: too many (sequence, head, key block) work items");
     return 1;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)items), dim3((NCW + 2) * 64), smem, s, a, ws);
+  hipLaunchKernelGGL(kern, dim3((unsigned)items), dim3(256), smem, s, a, ws);
   return 0;
 }
 template <typename T>

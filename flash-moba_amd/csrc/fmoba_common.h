@@ -368,4 +368,72 @@ __device__ __forceinline__ Pack8 zero_pack8() {
   return r;
 }
 
+// ------------------------------------------------------------------------------------
+// gathered tiles that global loads write straight into LDS: rows of exactly HD elements (one load
+// instruction writes 64 lanes x 16 bytes to consecutive addresses), swizzled instead of padded
+// ------------------------------------------------------------------------------------
+// piece c of tile row r is stored at piece c ^ tile_swz<HD>(r)
+template <int HD>
+__device__ __forceinline__ int tile_swz(int r) {
+  if constexpr (HD > 64)
+    return ((r & 3) << 2) | ((r >> 2) & 3);  // 16 pieces per row, one row per sweep of the banks
+  else
+    return (((r >> 1) & 1) << 2) | ((r >> 2) & 1);  // 8 pieces per row, two rows per sweep
+}
+template <int HD>
+struct TileSwz {
+  static constexpr int kRow8 = HD > 64 ? 2 : 0;  // tile_swz(r + 8) ^ tile_swz(r)
+};
+
+typedef __attribute__((address_space(3))) const Pack8 lds_cpack8;
+__device__ __forceinline__ Pack8 lds_read16(uint32_t byte_addr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return *(lds_cpack8 *)byte_addr;
+#else
+  (void)byte_addr;
+  return Pack8{{0, 0, 0, 0}};
+#endif
+}
+template <typename V>
+__device__ __forceinline__ V lds_read_vec(uint32_t byte_addr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return *(__attribute__((address_space(3))) const V *)byte_addr;
+#else
+  (void)byte_addr;
+  return V{};
+#endif
+}
+// 8 x 16-bit operand of a transposing read: two 8-byte reads
+__device__ __forceinline__ Pack8 lds_tr8(uint32_t addr_lo, uint32_t addr_hi) {
+  Pack8 r;
+#if defined(__HIP_DEVICE_COMPILE__)
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)addr_lo);
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)addr_hi);
+  __builtin_memcpy(&r.w[0], &lo, 8);
+  __builtin_memcpy(&r.w[2], &hi, 8);
+#else
+  (void)addr_lo, (void)addr_hi;
+  r = Pack8{{0, 0, 0, 0}};
+#endif
+  return r;
+}
+// 64 lanes x 16 bytes from each lane's own global address to LDS bytes [lds_base, lds_base + 1024), lane order;
+// lds_base is the same for the whole wave.  Written as assembly because the compiler makes every later LDS read wait
+// for a load that it knows to write LDS, and these are meant to stay in flight for a whole round: the kernel waits for
+// them itself (wait_all_loads) before the barrier that hands the tiles over.  Nothing else in the kernel uses m0.
+__device__ __forceinline__ void global_to_lds16(const void *g, uint32_t lds_base) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base) : "memory");
+#else
+  (void)g, (void)lds_base;
+#endif
+}
+__device__ __forceinline__ void wait_all_loads() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+}
+static __device__ uint4 g_zero16;  // 16 zero bytes: what the tile loads fetch for absent rows and for features past head_dim
+
+
 }  // namespace fmoba
