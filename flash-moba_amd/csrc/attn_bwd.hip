@@ -15,7 +15,7 @@
 //                          slot that the row hands out from a counter.
 //   attn_bwd_dq_kernel   : dQ from the dS tiles, one workgroup per 128 query rows, dQ in registers
 //                          (patterns in which a 128-row block meets a dozen rows or more per step).
-//   attn_bwd_dq_combine_kernel : dQ from the partials, one wave per (row, head) adds them in ascending
+//   attn_bwd_dq_combine_kernel : dQ from the partials, sixteen lanes per (row, head) add them in ascending
 //                          key-block order and scales.  Work and traffic are proportional to
 //                          the number of visits, whatever the number of chunks per sequence.
 // The dK/dV kernel runs four waves of 512 registers, one per SIMD, and all four compute: two pairs
@@ -941,56 +941,70 @@ __global__ __launch_bounds__(512, 4) void attn_bwd_dq_kernel(fmoba_attn_bwd_args
 }
 
 // ------------------------------------------------------------------------------------
-// dQ, second form: one wave per (row, head) adds the row's partials in ascending key-block order (sorted by
-// block id: the slot a visit got is arbitrary, the sum must not depend on it) and scales.
+// dQ, second form: the row's partials are added in ascending key-block order (sorted by block id: the slot a visit
+// got is arbitrary, the sum must not depend on it) and scaled.  One 16-lane group per (row, head), four per wave,
+// sixteen per block of 256: a row's chain of dependent steps (count, ids, order, rows) is mostly waiting, so a wave
+// runs four of them side by side.  Lane li of a group owns the 16-byte piece li of the row.
 // ------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void attn_bwd_dq_combine_kernel(fmoba_attn_bwd_args a, BwdWs ws) {
-  __shared__ int sOrd[4][64];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int64_t rh = (int64_t)blockIdx.x * 4 + wv;  // (global row) * heads + head
-  if (rh >= (int64_t)a.total_q * a.heads) return;
+  __shared__ int sOrd[16][16];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, grp = lane >> 4, li = lane & 15;
+  const int sg = wv * 4 + grp;  // group of the block
+  const int64_t total = (int64_t)a.total_q * a.heads;
+  const int64_t rh_raw = (int64_t)blockIdx.x * 16 + sg;  // (global row) * heads + head
+  const bool valid = rh_raw < total;
+  const int64_t rh = valid ? rh_raw : total - 1;
   const int64_t row = rh / a.heads;
   const int h = (int)(rh - row * a.heads);
   const int D = a.head_dim;
-  const int n = min(ws.cnt[rh], ws.cap);
-  const bool mine = 2 * lane < D;
+  const int n = valid ? min(ws.cnt[rh], ws.cap) : 0;
+  int nmax = max(n, __shfl_xor(n, 16, 64));
+  nmax = max(nmax, __shfl_xor(nmax, 32, 64));  // the wave walks the longest of its four rows
+  const int c8 = li * 8;
+  const bool mine = c8 < D;
   const int32_t *pid = ws.pid + rh * ws.cap;
   const uint16_t *part = ws.part + rh * ws.cap * D;
-  float acc0 = 0.f, acc1 = 0.f;
-  for (int base = 0; base < n; base += 64) {
-    const int cntb = min(64, n - base);
-    const int cj = lane < cntb ? pid[base + lane] : 0x7fffffff;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  for (int base = 0; base < nmax; base += 16) {
+    const int cntb = min(16, max(n - base, 0));
+    const int cj = li < cntb ? pid[base + li] : 0x7fffffff;
     int rank = 0;
-    for (int i = 0; i < cntb; ++i) {
-      const int ci = __shfl(cj, i, 64);
-      rank += (ci < cj || (ci == cj && i < lane)) ? 1 : 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int ci = __shfl(cj, (lane & 48) | i, 64);
+      rank += (ci < cj || (ci == cj && i < li)) ? 1 : 0;
     }
     wave_lds_fence();
-    if (lane < cntb) sOrd[wv][rank] = lane;
+    if (li < cntb) sOrd[sg][rank] = li;
     wave_lds_fence();
     if (mine) {
-      int t = 0;
-      for (; t + 4 <= cntb; t += 4) {
-        uint32_t x[4];
+      auto add = [&](const Pack8 &x) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const uint32_t *>(part + (int64_t)(base + sOrd[wv][t + u]) * D + 2 * lane);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          acc0 += elem_to_float<T>((uint16_t)(x[u] & 0xffffu));
-          acc1 += elem_to_float<T>((uint16_t)(x[u] >> 16));
+        for (int k = 0; k < 4; ++k) {
+          acc[2 * k] += elem_to_float<T>((uint16_t)(x.w[k] & 0xffffu));
+          acc[2 * k + 1] += elem_to_float<T>((uint16_t)(x.w[k] >> 16));
         }
+      };
+      int t = 0;
+      for (; t + 4 <= cntb; t += 4) {  // independent loads, four in flight
+        Pack8 x[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) x[u] = ld_global16(part + (int64_t)(base + sOrd[sg][t + u]) * D + c8);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) add(x[u]);
       }
-      for (; t < cntb; ++t) {
-        const uint32_t x = *reinterpret_cast<const uint32_t *>(part + (int64_t)(base + sOrd[wv][t]) * D + 2 * lane);
-        acc0 += elem_to_float<T>((uint16_t)(x & 0xffffu));
-        acc1 += elem_to_float<T>((uint16_t)(x >> 16));
-      }
+      for (; t < cntb; ++t) add(ld_global16(part + (int64_t)(base + sOrd[sg][t]) * D + c8));
     }
   }
-  if (mine)
-    *reinterpret_cast<uint32_t *>(reinterpret_cast<uint16_t *>(a.dq) + row * a.dq_row_stride + (int64_t)h * a.dq_head_stride + 2 * lane) =
-        pack2<T>(acc0 * a.softmax_scale, acc1 * a.softmax_scale);
+  if (valid && mine) {
+    Pack8 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o.w[k] = pack2<T>(acc[2 * k] * a.softmax_scale, acc[2 * k + 1] * a.softmax_scale);
+    *reinterpret_cast<Pack8 *>(reinterpret_cast<uint16_t *>(a.dq) + row * a.dq_row_stride + (int64_t)h * a.dq_head_stride + c8) = o;
+  }
 }
 
 // grid (ceil(max_seqlen_q / rows_per_block), heads, batch), block 256.
@@ -1109,7 +1123,7 @@ static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hi
   if (phases & FMOBA_BWD_DQ) {
     if (partials) {
       const int64_t rows = (int64_t)a.total_q * a.heads;
-      hipLaunchKernelGGL(attn_bwd_dq_combine_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, a, ws);
+      hipLaunchKernelGGL(attn_bwd_dq_combine_kernel<T>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a, ws);
     } else {
       int rc = a.head_dim <= 64 ? launch_dq<T, 64>(a, ws.ds, s) : launch_dq<T, 128>(a, ws.ds, s);
       if (rc) return rc;

@@ -11,7 +11,7 @@
 //                             a (row, key block) pair leaves a PARTIAL result: the block-local
 //                             maximum m, the sum l of exp2(s - m) and the unnormalised output row
 //                             (16-bit), in a slot that the row hands out from a counter.
-//   attn_fwd_combine_kernel : one wave per (row, head) merges the row's partials in ascending
+//   attn_fwd_combine_kernel : sixteen lanes per (row, head) merge the row's partials in ascending
 //                             key-block order (sorted by block id, so the result does not depend
 //                             on which slot a visit happened to get): out, log-sum-exp.
 //
@@ -354,89 +354,104 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
   }
 }
 
-// one wave per (row, head); block 256 = 4 rows
+// One 16-lane group per (row, head), four per wave, sixteen per block of 256: a row's chain of dependent steps (count,
+// headers, order, rows) is mostly waiting, so a wave runs four of them side by side.  Lane li of a group owns the
+// 16-byte piece li of the row.
 template <typename T>
 __global__ __launch_bounds__(256) void attn_fwd_combine_kernel(fmoba_attn_fwd_args a, FwdWs ws) {
-  __shared__ int sOrd[4][64];
-  __shared__ float sWgt[4][64];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int64_t rh = (int64_t)blockIdx.x * 4 + wv;  // (global row) * heads + head
-  if (rh >= (int64_t)a.total_q * a.heads) return;
+  __shared__ int sOrd[16][16];
+  __shared__ float sWgt[16][16], sWl[16][16];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, grp = lane >> 4, li = lane & 15;
+  const int sg = wv * 4 + grp;  // group of the block
+  const int64_t total = (int64_t)a.total_q * a.heads;
+  const int64_t rh_raw = (int64_t)blockIdx.x * 16 + sg;  // (global row) * heads + head
+  const bool valid = rh_raw < total;
+  const int64_t rh = valid ? rh_raw : total - 1;
   const int64_t row = rh / a.heads;
   const int h = (int)(rh - row * a.heads);
   const int D = a.head_dim;
-  const int n = min(ws.cnt[rh], ws.cap);
-  uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + row * a.o_row_stride + (int64_t)h * a.o_head_stride;
-  float *lsep = a.softmax_lse + (int64_t)h * a.total_q + row;
-  float acc0 = 0.f, acc1 = 0.f, L = 0.f, M = -INFINITY;
+  const int n = valid ? min(ws.cnt[rh], ws.cap) : 0;
+  int nmax = max(n, __shfl_xor(n, 16, 64));
+  nmax = max(nmax, __shfl_xor(nmax, 32, 64));  // the wave walks the longest of its four rows
+  const int c8 = li * 8;
+  const bool mine = c8 < D;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  float L = 0.f, M = -INFINITY;
   const float4 *hdr = ws.hdr + rh * ws.cap;
   const uint16_t *part = ws.part + rh * ws.cap * D;
-  const bool mine = 2 * lane < D;
-  // partials are merged in ascending key-block order (the slot a visit got is arbitrary), 64 at a time
-  for (int base = 0; base < n; base += 64) {
-    const int cntb = min(64, n - base);
+  // partials are merged in ascending key-block order (the slot a visit got is arbitrary), 16 at a time
+  for (int base = 0; base < nmax; base += 16) {
+    const int cntb = min(16, max(n - base, 0));
     float mj = -INFINITY, lj = 0.f;
     int cj = 0x7fffffff;
-    if (lane < cntb) {
-      const float4 x = hdr[base + lane];
+    if (li < cntb) {
+      const float4 x = hdr[base + li];
       mj = x.x;
       lj = x.y;
       cj = __float_as_int(x.z);
     }
     // rank of this lane's partial in the batch; equal ids (malformed pattern) are ordered by slot
     int rank = 0;
-    for (int i = 0; i < cntb; ++i) {
-      const int ci = __shfl(cj, i, 64);
-      rank += (ci < cj || (ci == cj && i < lane)) ? 1 : 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int ci = __shfl(cj, (lane & 48) | i, 64);
+      rank += (ci < cj || (ci == cj && i < li)) ? 1 : 0;
     }
     float mb = mj;
-    for (int o = 32; o >= 1; o >>= 1) mb = fmaxf(mb, __shfl_xor(mb, o, 64));
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) mb = fmaxf(mb, __shfl_xor(mb, o, 64));
     const float Mn = fmaxf(M, mb);
     const float Mu = Mn == -INFINITY ? 0.f : Mn;
     const float resc = __builtin_amdgcn_exp2f(M - Mu);  // M = -inf: nothing accumulated yet, factor 0 on zeros
-    acc0 *= resc;
-    acc1 *= resc;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] *= resc;
     L *= resc;
     M = Mn;
-    const float wj = (lane < cntb) ? __builtin_amdgcn_exp2f(mj - Mu) : 0.f;
-    // sum of the weighted l in rank order: every lane adds the same sequence, so L is the same everywhere
+    const float wj = (li < cntb) ? __builtin_amdgcn_exp2f(mj - Mu) : 0.f;
     wave_lds_fence();
-    if (lane < cntb) {
-      sOrd[wv][rank] = lane;
-      sWgt[wv][rank] = wj;
+    if (li < cntb) {
+      sOrd[sg][rank] = li;
+      sWgt[sg][rank] = wj;
+      sWl[sg][rank] = wj * lj;
     }
-    float wl = wj * lj;
     wave_lds_fence();
-    for (int t = 0; t < cntb; ++t) L += __shfl(wl, sOrd[wv][t], 64);
-    // the rows themselves: independent loads, four in flight
+    // sums in rank order: every lane of the group adds the same sequence
+    for (int t = 0; t < cntb; ++t) L += sWl[sg][t];
     if (mine) {
+      auto add = [&](const Pack8 &x, float w) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          acc[2 * k] = fmaf(w, elem_to_float<T>((uint16_t)(x.w[k] & 0xffffu)), acc[2 * k]);
+          acc[2 * k + 1] = fmaf(w, elem_to_float<T>((uint16_t)(x.w[k] >> 16)), acc[2 * k + 1]);
+        }
+      };
       int t = 0;
-      for (; t + 4 <= cntb; t += 4) {
-        uint32_t x[4];
+      for (; t + 4 <= cntb; t += 4) {  // independent loads, four in flight
+        Pack8 x[4];
         float w[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          x[u] = *reinterpret_cast<const uint32_t *>(part + (int64_t)(base + sOrd[wv][t + u]) * D + 2 * lane);
-          w[u] = sWgt[wv][t + u];
+          x[u] = ld_global16(part + (int64_t)(base + sOrd[sg][t + u]) * D + c8);
+          w[u] = sWgt[sg][t + u];
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          acc0 = fmaf(w[u], elem_to_float<T>((uint16_t)(x[u] & 0xffffu)), acc0);
-          acc1 = fmaf(w[u], elem_to_float<T>((uint16_t)(x[u] >> 16)), acc1);
-        }
+        for (int u = 0; u < 4; ++u) add(x[u], w[u]);
       }
-      for (; t < cntb; ++t) {
-        const uint32_t x = *reinterpret_cast<const uint32_t *>(part + (int64_t)(base + sOrd[wv][t]) * D + 2 * lane);
-        const float w = sWgt[wv][t];
-        acc0 = fmaf(w, elem_to_float<T>((uint16_t)(x & 0xffffu)), acc0);
-        acc1 = fmaf(w, elem_to_float<T>((uint16_t)(x >> 16)), acc1);
-      }
+      for (; t < cntb; ++t) add(ld_global16(part + (int64_t)(base + sOrd[sg][t]) * D + c8), sWgt[sg][t]);
     }
   }
+  if (!valid) return;
   const bool empty = !(L > 0.f);
   const float inv = empty ? 0.f : 1.f / L;
-  if (mine) *reinterpret_cast<uint32_t *>(op + 2 * lane) = pack2<T>(acc0 * inv, acc1 * inv);
-  if (lane == 0) *lsep = empty ? INFINITY : (M + __builtin_amdgcn_logf(L)) * 0.6931471805599453f;
+  if (mine) {
+    Pack8 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o.w[k] = pack2<T>(acc[2 * k] * inv, acc[2 * k + 1] * inv);
+    *reinterpret_cast<Pack8 *>(reinterpret_cast<uint16_t *>(a.out) + row * a.o_row_stride + (int64_t)h * a.o_head_stride + c8) = o;
+  }
+  if (li == 0) a.softmax_lse[(int64_t)h * a.total_q + row] = empty ? INFINITY : (M + __builtin_amdgcn_logf(L)) * 0.6931471805599453f;
 }
 
 __global__ void fwd_empty_kernel(void *out, float *lse, int64_t n_out_words, int64_t n_lse) {
@@ -525,7 +540,7 @@ static int run_fwd(const fmoba_attn_fwd_args &a, const FwdWs &ws, int phases, hi
     if (rc) return rc;
   }
   if (phases & FMOBA_FWD_COMBINE)
-    hipLaunchKernelGGL(attn_fwd_combine_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, a, ws);
+    hipLaunchKernelGGL(attn_fwd_combine_kernel<T>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a, ws);
   return 0;
 }
 
