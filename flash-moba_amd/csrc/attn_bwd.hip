@@ -1099,6 +1099,15 @@ static int bwd_dq_partials(const fmoba_attn_bwd_args &a) {
   return 128.0 * chunks_per_row < 12.0 * chunks_per_seq;
 }
 
+// columns of a multiple of 128 keys: one workgroup (and one dQ partial per visit) per 128 keys
+static inline bool bwd_wide_blocks(const fmoba_attn_bwd_args &a) { return a.head_dim > 64 && a.lg_block_n % 128 == 0; }
+// partial slots per (row, head): max_visits_per_row counts 64-key blocks; with 128-key blocks a row has half as many
+// visits (only the last column of a sequence can have an odd number of 64-key blocks)
+static inline int32_t bwd_partial_cap(const fmoba_attn_bwd_args &a) {
+  const int32_t mv = a.max_visits_per_row > 0 ? a.max_visits_per_row : 1;
+  return bwd_wide_blocks(a) ? (mv + 1) / 2 : mv;
+}
+
 template <typename T>
 static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hipStream_t s) {
   const bool partials = bwd_dq_partials(a);
@@ -1111,7 +1120,7 @@ static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hi
   if (phases & FMOBA_BWD_DKDV) {
     int rc;
     // columns of a multiple of 128 keys: one workgroup per 128 keys (the two 64-key blocks share their row list)
-    const bool wide = a.lg_block_n % 128 == 0;
+    const bool wide = bwd_wide_blocks(a);
     if (partials) {
       hipLaunchKernelGGL(zero_i32_kernel, dim3(512), dim3(256), 0, s, ws.cnt, (int64_t)a.total_q * a.heads);
       rc = a.head_dim <= 64 ? launch_dkdv<T, 64, true, 1>(a, ws, s) : (wide ? launch_dkdv<T, 128, true, 2>(a, ws, s) : launch_dkdv<T, 128, true, 1>(a, ws, s));
@@ -1145,7 +1154,7 @@ extern "C" size_t fmoba_attn_bwd_workspace_bytes(const fmoba_attn_bwd_args *a) {
   using namespace fmoba;
   if (a == nullptr || a->total_q <= 0 || a->heads <= 0 || a->head_dim <= 0 || a->batch <= 0 || a->lg_block_n <= 0) return 256;
   if (!bwd_dq_partials(*a)) return (size_t)(a->num_row_indices > 0 ? a->num_row_indices : 0) * a->lg_block_n * 2 + 256;
-  const size_t rows = (size_t)a->total_q * a->heads, cap = (size_t)(a->max_visits_per_row > 0 ? a->max_visits_per_row : 1);
+  const size_t rows = (size_t)a->total_q * a->heads, cap = (size_t)bwd_partial_cap(*a);
   // one spare partial row / block id at the end takes the writes of absent rows
   return bwd_align256(rows * 4) + bwd_align256((rows * cap + 1) * 4) + bwd_align256((rows * cap + 1) * a->head_dim * 2) + 256;
 }
@@ -1207,7 +1216,7 @@ extern "C" int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phase
   const size_t rows = (size_t)a->total_q * a->heads;
   uintptr_t wp = ((uintptr_t)a->workspace + 255) & ~(uintptr_t)255;
   BwdWs ws;
-  ws.cap = a->max_visits_per_row;
+  ws.cap = bwd_partial_cap(*a);
   ws.ds = reinterpret_cast<uint16_t *>(wp);
   ws.cnt = reinterpret_cast<int32_t *>(wp);
   wp += bwd_align256(rows * 4);

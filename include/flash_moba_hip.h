@@ -175,8 +175,9 @@ int fmoba_attn_fwd_phases(const fmoba_attn_fwd_args *a, int32_t phases, void *st
  *       row_indices) in the workspace and a row-stationary pass (128 query rows per workgroup,
  *       accumulators in LDS) multiplies them with K;
  *     partials: the dK/dV pass leaves one dQ partial row (16-bit) per visit of a (query row,
- *       64-key block) pair, a second launch adds the partials of each row in key order.  This is
- *       the form that scales when sequences have thousands of chunks.
+ *       key block) pair, a second launch adds the partials of each row in key order.  This is
+ *       the form that scales when sequences have thousands of chunks.  (Key blocks have 128 keys
+ *       when lg_block_n is a multiple of 128 and head_dim > 64, else 64.)
  *   workspace: fmoba_attn_bwd_workspace_bytes(args) bytes (only the sizes, dq_mode,
  *   num_row_indices and max_visits_per_row of args are read), contents undefined on entry and on
  *   return.  num_row_indices = number of int32 entries of row_indices (every col_offsets[i] +
