@@ -428,7 +428,9 @@ def test_row_block_forms_over_many_columns(fm):
 
 
 @pytest.mark.parametrize("dq_mode", [1, 2])
-@pytest.mark.parametrize("d,chunk", [(128, 64), (64, 128), (96, 64)])
+# (128, 128), (96, 128), (128, 256): columns of a multiple of 128 keys with head_dim > 64, where the dK/dV pass works
+# on 128-key blocks (one or two per column; 96: a wave without features of its own in the dQ products)
+@pytest.mark.parametrize("d,chunk", [(128, 64), (64, 128), (96, 64), (128, 128), (96, 128), (128, 256)])
 def test_backward_both_dq_forms(fm, dq_mode, d, chunk):
     # the library picks the dQ form by shape; both are checked here whatever it would pick
     lens = [300, 0, 77, 650]
