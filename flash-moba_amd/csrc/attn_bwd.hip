@@ -208,22 +208,24 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     // per-row scalars: the row id of round s+2 (it has to be in LDS one round before the tile loads that use it),
     // and LSE, delta and the dQ-partial slot of round s+1.
     const uint32_t ldsQ = (uint32_t)(uintptr_t)(smem + SM::oQ), ldsdO = (uint32_t)(uintptr_t)(smem + SM::odO);
-    int n_rid = -1, m_rid = -1, m_slot = 0;
+    int n_rid = -1, v_rid = rid01[1], m_rid = -1, m_slot = 0;  // v_rid: the checked row id that was stored last = the one of the next round
     float m_lse = 0.f, m_del = 0.f;
     int ft = tid;  // thread index for the feeding code, re-made opaque in every round (see below)
     auto rid_issue = [&](int sr) {
       if (tid < kBwdRoundRows) {
-        const int j = sr * kBwdRoundRows + ft;
-        const int r = list[min(j, n - 1)];
-        n_rid = ((j < n) & (r >= 0) & (r < Lq)) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
+        n_rid = list[min(sr * kBwdRoundRows + ft, n - 1)];  // used (and checked) only when it is stored: no wait for it here
       }
     };
     auto rid_store = [&](int sr) {
-      if (tid < kBwdRoundRows) sRid[(sr & 1) * kBwdRoundRows + ft] = n_rid;
-    };
-    auto meta_issue = [&](int sr) {
       if (tid < kBwdRoundRows) {
-        m_rid = sRid[(sr & 1) * kBwdRoundRows + ft];
+        const int j = sr * kBwdRoundRows + ft;
+        v_rid = ((j < n) & (n_rid >= 0) & (n_rid < Lq)) ? n_rid : -1;  // rows outside the sequence (malformed pattern) are ignored
+        sRid[(sr & 1) * kBwdRoundRows + ft] = v_rid;
+      }
+    };
+    auto meta_issue = [&](int rid) {  // rid: this thread's row of the round after the current one
+      if (tid < kBwdRoundRows) {
+        m_rid = rid;
         const int rc = max(m_rid, 0);
         m_lse = lseg[rc];
         m_del = delg[rc];
@@ -266,7 +268,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       sRid[kBwdRoundRows + tid] = rid01[1];
     }
     __syncthreads();  // K, V are in registers; the row ids of rounds 0 and 1 are in LDS
-    meta_issue(0);
+    meta_issue(rid01[0]);
     tile_issue(0);
     meta_store(0);
     wait_all_loads();
@@ -556,7 +558,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       asm volatile("" : "+v"(ft));
 #endif
       rid_issue(r + 2);
-      meta_issue(r + 1);
+      meta_issue(v_rid);
       tile_issue(r + 1);
       process_round(pc, C0{}, r);
       if constexpr (KB == 2) process_round(pc, C1{}, r);

@@ -165,21 +165,23 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
   typedef std::integral_constant<int, 0> C0;
   typedef std::integral_constant<int, 1> C1;
   const uint32_t ldsQ = (uint32_t)(uintptr_t)(smem + SM::oQ);
-  int n_rid = -1, m_rid = -1, m_slot = 0;
+  int n_rid = -1, v_rid = rid01[1], m_rid = -1, m_slot = 0;  // v_rid: the checked row id that was stored last = the one of the next round
   int ft = tid;  // thread index for the feeding code, re-made opaque in every round: what is derived from it must not be kept in registers across rounds
   auto rid_issue = [&](int sr) {
     if (tid < kFwdRoundRows) {
-      const int j = sr * kFwdRoundRows + ft;
-      const int r = list[min(j, n - 1)];
-      n_rid = ((j < n) & (r >= 0) & (r < Lq)) ? r : -1;
+      n_rid = list[min(sr * kFwdRoundRows + ft, n - 1)];  // used (and checked) only when it is stored: no wait for it here
     }
   };
   auto rid_store = [&](int sr) {
-    if (tid < kFwdRoundRows) sRid[(sr & 1) * kFwdRoundRows + ft] = n_rid;
-  };
-  auto meta_issue = [&](int sr) {
     if (tid < kFwdRoundRows) {
-      m_rid = sRid[(sr & 1) * kFwdRoundRows + ft];
+      const int j = sr * kFwdRoundRows + ft;
+      v_rid = ((j < n) & (n_rid >= 0) & (n_rid < Lq)) ? n_rid : -1;  // rows outside the sequence (malformed pattern) are ignored
+      sRid[(sr & 1) * kFwdRoundRows + ft] = v_rid;
+    }
+  };
+  auto meta_issue = [&](int rid) {  // rid: this thread's row of the round after the current one
+    if (tid < kFwdRoundRows) {
+      m_rid = rid;
       // every visit of a (row, key block) pair takes one slot of the row (a shared dummy counter for absent
       // rows would serialise the whole grid on one address)
       if (m_rid >= 0) m_slot = atomicAdd(cntg + (int64_t)m_rid * a.heads, 1);
@@ -205,7 +207,7 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
       global_to_lds16(ok ? qg + (int64_t)rid * a.q_row_stride + e : zero, dst + (uint32_t)(i * RPI * RB));
     }
   };
-  meta_issue(0);
+  meta_issue(rid01[0]);
   tile_issue(0);
   meta_store(0);
   wait_all_loads();
@@ -340,7 +342,7 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
     asm volatile("" : "+v"(ft));
 #endif
     rid_issue(r + 2);
-    meta_issue(r + 1);
+    meta_issue(v_rid);
     tile_issue(r + 1);
     if (4 * r + wave < ntile) process_tile(pc);
     meta_store(r + 1);
