@@ -520,7 +520,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         }
         mm_b(C0{}, gc);
         smx(C1{}, gc);
-        if constexpr (!DQP && G == 1) ds_store(tile0);
+        if constexpr (!DQP && G == 0) ds_store(tile0);
         fence();
       });
       // dV, dK of the second tile; in the partials form dQ of the first one runs between them: by now all key
@@ -538,7 +538,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         if constexpr (G < 3) ld_b(pc, pp, C1{}, std::integral_constant<int, G + 1>{});
         mm_b(C1{}, gc);
         if constexpr (DQP) dq_mma(gc);
-        if constexpr (!DQP && G == 1) ds_store(tile0 + 1);
+        if constexpr (!DQP && G == 0) ds_store(tile0 + 1);
         fence();
       });
       if constexpr (DQP) {
