@@ -194,7 +194,12 @@ __device__ __forceinline__ Pack8 tr_frag8(const uint16_t *X, int ld, int rows4_l
 // address register (the generic-pointer form above needs one register per read).
 typedef __attribute__((address_space(3))) const uint16_t lds_cu16;
 __device__ __forceinline__ lds_cu16 *to_lds(const void *lds_generic_ptr) {
+#if defined(__HIP_DEVICE_COMPILE__)
   return (lds_cu16 *)(uint32_t)(uintptr_t)lds_generic_ptr;
+#else
+  (void)lds_generic_ptr;
+  return nullptr;
+#endif
 }
 __device__ __forceinline__ lds_cu16 *tr_lane_base(const uint16_t *X, int ld, int lane) {
   const int i = lane & 15;
