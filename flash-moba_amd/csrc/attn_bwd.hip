@@ -250,14 +250,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
       const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(((sr & 1) * 4 + wave) * (int)TB);
       const uint16_t *zero = reinterpret_cast<const uint16_t *>(&g_zero16);
+      const int qs = (int)a.q_row_stride, dos = (int)a.do_row_stride;  // (32 x 32 -> 64-bit products: one instruction each)
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int row = i * RPI + rl;
         const int rid = sRid[(sr & 1) * kBwdRoundRows + wave * 32 + row];
         const int e = (p ^ tile_swz<HD>(row)) * 8;
         const bool ok = (rid >= 0) & (e < D);
-        const uint16_t *gq = ok ? qg + (int64_t)rid * a.q_row_stride + e : zero;
-        const uint16_t *gd = ok ? dog + (int64_t)rid * a.do_row_stride + e : zero;
+        const uint16_t *gq = ok ? qg + ((int64_t)rid * qs + e) : zero;
+        const uint16_t *gd = ok ? dog + ((int64_t)rid * dos + e) : zero;
         global_to_lds16(gq, ldsQ + dst + (uint32_t)(i * RPI * RB));
         global_to_lds16(gd, ldsdO + dst + (uint32_t)(i * RPI * RB));
       }
@@ -1186,6 +1187,7 @@ extern "C" int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phase
                         a->dk_row_stride, a->dk_head_stride, a->dv_row_stride, a->dv_head_stride};
   for (int64_t x : st) FMOBA_REQUIRE(x % 8 == 0, "attn_bwd: strides must be multiples of 8 elements");
   FMOBA_REQUIRE(a->k_row_stride < ((int64_t)1 << 24), "attn_bwd: k_row_stride must be below 2^24 elements");
+  FMOBA_REQUIRE(a->q_row_stride < ((int64_t)1 << 31) && a->do_row_stride < ((int64_t)1 << 31), "attn_bwd: q / dout row strides must be below 2^31 elements");
   const void *ptrs[] = {a->dout, a->q, a->k, a->v, a->out, a->dq, a->dk, a->dv};
   for (const void *p : ptrs) FMOBA_REQUIRE(((uintptr_t)p % 16) == 0, "attn_bwd: tensors must be 16-byte aligned");
 

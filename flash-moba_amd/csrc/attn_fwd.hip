@@ -198,13 +198,14 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
     const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
     const uint32_t dst = ldsQ + (uint32_t)__builtin_amdgcn_readfirstlane(((sr & 1) * 4 + wave) * (int)TB);
     const uint16_t *zero = reinterpret_cast<const uint16_t *>(&g_zero16);
+    const int qs = (int)a.q_row_stride;  // (32 x 32 -> 64-bit product: one instruction)
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int row = i * RPI + rl;
       const int rid = sRid[(sr & 1) * kFwdRoundRows + wave * 32 + row];
       const int e = (p ^ tile_swz<HD>(row)) * 8;
       const bool ok = (rid >= 0) & (e < D);
-      global_to_lds16(ok ? qg + (int64_t)rid * a.q_row_stride + e : zero, dst + (uint32_t)(i * RPI * RB));
+      global_to_lds16(ok ? qg + ((int64_t)rid * qs + e) : zero, dst + (uint32_t)(i * RPI * RB));
     }
   };
   meta_issue(rid01[0]);
@@ -627,6 +628,7 @@ extern "C" int fmoba_attn_fwd_phases(const fmoba_attn_fwd_args *a, int32_t phase
   const int64_t st[] = {a->q_row_stride, a->q_head_stride, a->k_row_stride, a->k_head_stride,
                         a->v_row_stride, a->v_head_stride, a->o_row_stride, a->o_head_stride};
   for (int64_t x : st) FMOBA_REQUIRE(x % 8 == 0, "attn_fwd: strides must be multiples of 8 elements");
+  FMOBA_REQUIRE(a->q_row_stride < ((int64_t)1 << 31), "attn_fwd: q_row_stride must be below 2^31 elements");
   FMOBA_REQUIRE(((uintptr_t)a->q % 16) == 0 && ((uintptr_t)a->k % 16) == 0 && ((uintptr_t)a->v % 16) == 0 && ((uintptr_t)a->out % 16) == 0,
                 "attn_fwd: q, k, v and out must be 16-byte aligned");
   FMOBA_REQUIRE(a->max_visits_per_row > 0, "attn_fwd: max_visits_per_row must be positive");
