@@ -24,7 +24,7 @@ struct TopkParams {
 };
 
 template <typename T, int HD, int NT>
-__global__ __launch_bounds__(256) void topk_gate_kernel(TopkParams p) {
+__global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_kernel(TopkParams p) {
   constexpr int KS = HD / 16;
   constexpr int LD = HD + 16;  // LDS row stride (elements)
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
