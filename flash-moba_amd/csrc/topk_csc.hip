@@ -271,18 +271,20 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
 // ------------------------------------------------------------------------------------
 constexpr int kBigCap = 32;  // running winners per row (K' = scored chunks kept)
 
-template <typename T, int HD, int NT>
-__global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
+// CAP: entries of a row's list of running winners (16 or CAP).  With 16 and groups of 128 chunks the kernel needs
+// half the LDS and fewer registers, and two workgroups share a compute unit.
+template <typename T, int HD, int NT, int CAP>
+__global__ __launch_bounds__(256, CAP < CAP ? 2 : 1) void topk_gate_big_kernel(TopkParams p) {
   constexpr int KS = HD / 16;
   constexpr int LD = HD + 16;
   constexpr int GC = NT * 32;        // chunks per group
-  constexpr int PL = kBigCap / 2;    // previous winners held per lane (two lanes per row)
+  constexpr int PL = CAP / 2;    // previous winners held per lane (two lanes per row)
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint16_t *sKm = reinterpret_cast<uint16_t *>(smem);
   uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [W][128], reuses the chunk-mean tile after the last group
-  float *sVal = reinterpret_cast<float *>(smem + (size_t)GC * LD * 2);   // [2][128][kBigCap]
-  int *sIdx = reinterpret_cast<int *>(sVal + 2 * kGateRows * kBigCap);   // [2][128][kBigCap]
-  int *sCnt = sIdx + 2 * kGateRows * kBigCap;                            // [2][128]
+  float *sVal = reinterpret_cast<float *>(smem + (size_t)GC * LD * 2);   // [2][128][CAP]
+  int *sIdx = reinterpret_cast<int *>(sVal + 2 * kGateRows * CAP);   // [2][128][CAP]
+  int *sCnt = sIdx + 2 * kGateRows * CAP;                            // [2][128]
   int *sHist = sCnt + 2 * kGateRows;                                     // [max_cols]
   int *sTrash = sHist + p.max_cols;                                      // [256]: takes the stores of lanes that have nothing to store
 
@@ -362,8 +364,8 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
     for (int j = 0; j < PL; ++j) {
       const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
       const bool ok = e < m_prev;
-      pv[j] = ok ? sVal[(cur * kGateRows + rs) * kBigCap + e] : -INFINITY;
-      pi[j] = ok ? sIdx[(cur * kGateRows + rs) * kBigCap + e] : -1;
+      pv[j] = ok ? sVal[(cur * kGateRows + rs) * CAP + e] : -INFINITY;
+      pi[j] = ok ? sIdx[(cur * kGateRows + rs) * CAP + e] : -1;
       vmin = fminf(vmin, ok ? pv[j] : INFINITY);
       vmax = fmaxf(vmax, pv[j]);
     }
@@ -416,9 +418,9 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
       wave_lds_fence();
       const int ne_row = sCnt[nxt * kGateRows + rs];
       wave_lds_fence();
-      if (__all(ne_row <= kBigCap)) {
-        float *ev = sVal + (size_t)(nxt * kGateRows + rs) * kBigCap;
-        int *ei = sIdx + (size_t)(nxt * kGateRows + rs) * kBigCap;
+      if (__all(ne_row <= CAP)) {
+        float *ev = sVal + (size_t)(nxt * kGateRows + rs) * CAP;
+        int *ei = sIdx + (size_t)(nxt * kGateRows + rs) * CAP;
         // (no branches: a lane without an entrant at this position stores to its trash word)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
@@ -473,8 +475,8 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
         for (int j = 0; j < PL; ++j) {
           const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
           if (e < m_prev) {
-            sVal[(cur * kGateRows + rs) * kBigCap + e] = pv[j];
-            sIdx[(cur * kGateRows + rs) * kBigCap + e] = pi[j];
+            sVal[(cur * kGateRows + rs) * CAP + e] = pv[j];
+            sIdx[(cur * kGateRows + rs) * CAP + e] = pi[j];
           }
         }
         continue;
@@ -589,8 +591,8 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
     }
     int slot = 0;
     if (nwin > 0) slot = atomicAdd(&sCnt[nxt * kGateRows + rs], nwin);
-    float *ov = sVal + (size_t)(nxt * kGateRows + rs) * kBigCap;
-    int *oi = sIdx + (size_t)(nxt * kGateRows + rs) * kBigCap;
+    float *ov = sVal + (size_t)(nxt * kGateRows + rs) * CAP;
+    int *oi = sIdx + (size_t)(nxt * kGateRows + rs) * CAP;
     if (__any(nwin > 0)) {  // (no branches inside: a lane without a winner at a position stores to its trash word)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
@@ -599,7 +601,7 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
           for (int i = 0; i < 16; ++i) {
             const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
             const float x = sc[t][i];
-            const bool w = (kp > 0) & ((x > tau) | ((x == tau_eq) & (c >= iota))) & (slot < kBigCap);
+            const bool w = (kp > 0) & ((x > tau) | ((x == tau_eq) & (c >= iota))) & (slot < CAP);
             *(w ? ov + slot : reinterpret_cast<float *>(sTrash + tid)) = x;
             *(w ? oi + slot : sTrash + tid) = (int)c;
             slot += w ? 1 : 0;
@@ -607,7 +609,7 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
         }
 #pragma unroll
       for (int j = 0; j < PL; ++j) {
-        const bool w = (kp > 0) & (pi[j] >= 0) & ((pv[j] > tau) | ((pv[j] == tau_eq) & ((uint32_t)pi[j] >= iota))) & (slot < kBigCap);
+        const bool w = (kp > 0) & (pi[j] >= 0) & ((pv[j] > tau) | ((pv[j] == tau_eq) & ((uint32_t)pi[j] >= iota))) & (slot < CAP);
         *(w ? ov + slot : reinterpret_cast<float *>(sTrash + tid)) = pv[j];
         *(w ? oi + slot : sTrash + tid) = pi[j];
         slot += w ? 1 : 0;
@@ -622,12 +624,12 @@ __global__ __launch_bounds__(256) void topk_gate_big_kernel(TopkParams p) {
   for (int c = tid; c < p.max_cols; c += 256) sHist[c] = 0;
   __syncthreads();
   if (valid) {
-    const int m = min(sCnt[cur * kGateRows + rs], kBigCap);
+    const int m = min(sCnt[cur * kGateRows + rs], CAP);
 #pragma unroll
     for (int j = 0; j < PL; ++j) {
       const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
       if (e < m) {
-        const int c = sIdx[(cur * kGateRows + rs) * kBigCap + e];
+        const int c = sIdx[(cur * kGateRows + rs) * CAP + e];
         atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
         atomicAdd(&sHist[c], 1);
       }
@@ -854,15 +856,20 @@ static int launch_gate_nt(const TopkParams &p, dim3 grid, hipStream_t s) {
   if (p.W <= 4) return launch_gate<T, HD, 4>(p, grid, s);
   return launch_gate<T, HD, 8>(p, grid, s);
 }
-template <typename T, int HD, int NT>
-static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
+template <int HD, int NT, int CAP>
+static size_t gate_big_smem(const TopkParams &p) {
   const size_t tile = (size_t)NT * 32 * (HD + 16) * 2;
-  const size_t smem = tile + (size_t)2 * kGateRows * kBigCap * 8 + (size_t)2 * kGateRows * 4 + (size_t)p.max_cols * 4 + 256 * 4;
-  if ((size_t)p.W * kGateRows * 4 > tile || smem > 160 * 1024) {
+  if ((size_t)p.W * kGateRows * 4 > tile) return (size_t)1 << 30;  // the selection words reuse the tile
+  return tile + (size_t)2 * kGateRows * CAP * 8 + (size_t)2 * kGateRows * 4 + (size_t)p.max_cols * 4 + 256 * 4;
+}
+template <typename T, int HD, int NT, int CAP>
+static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
+  const size_t smem = gate_big_smem<HD, NT, CAP>(p);
+  if (smem > 160 * 1024) {
     set_error("fused_topk: %d key chunks per sequence exceed what the LDS of this build holds", p.max_cols);
     return 1;
   }
-  auto kern = topk_gate_big_kernel<T, HD, NT>;
+  auto kern = topk_gate_big_kernel<T, HD, NT, CAP>;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("fused_topk: cannot reserve %zu bytes of LDS", smem);
     return 2;
@@ -872,9 +879,17 @@ static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
 }
 template <typename T>
 static int launch_gate_big_hd(const TopkParams &p, dim3 grid, hipStream_t s) {
-  if (p.a.head_dim <= 64) return launch_gate_big<T, 64, 8>(p, grid, s);
-  if (p.a.head_dim <= 128) return launch_gate_big<T, 128, 8>(p, grid, s);
-  return launch_gate_big<T, 256, 4>(p, grid, s);
+  // up to 16 running winners per row: short lists and groups of 128 chunks, if that lets two workgroups share a compute unit
+  const int kp = p.a.is_causal ? p.a.topk - 1 : p.a.topk;
+  if (p.a.head_dim <= 64) {
+    if (kp <= 16 && gate_big_smem<64, 4, 16>(p) <= 80 * 1024) return launch_gate_big<T, 64, 4, 16>(p, grid, s);
+    return launch_gate_big<T, 64, 8, kBigCap>(p, grid, s);
+  }
+  if (p.a.head_dim <= 128) {
+    if (kp <= 16 && gate_big_smem<128, 4, 16>(p) <= 80 * 1024) return launch_gate_big<T, 128, 4, 16>(p, grid, s);
+    return launch_gate_big<T, 128, 8, kBigCap>(p, grid, s);
+  }
+  return launch_gate_big<T, 256, 4, kBigCap>(p, grid, s);
 }
 template <typename T>
 static int launch_gate_hd(const TopkParams &p, dim3 grid, hipStream_t s) {
