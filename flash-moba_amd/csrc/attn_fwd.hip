@@ -220,14 +220,26 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
   // are an exclusive-or on the piece bits
   const uint32_t qrow = ldsQ + (uint32_t)wave * TB + (uint32_t)((lane & 31) * RB + (((hh * KS) ^ tile_swz<HD>(lane & 31)) * 16));
 
+  // LDS addresses are one register (made opaque to the compiler where it is used) plus an offset in the instruction:
+  // left alone, the compiler computes every address of a tile outside the loop and parks them in spare registers
+  auto opaque = [](uint32_t &x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" : "+v"(x));
+#else
+    (void)x;
+#endif
+  };
+  const uint32_t ldsOut = (uint32_t)(uintptr_t)sOut, ldsRow = (uint32_t)(uintptr_t)(smem + SM::oRow) + (uint32_t)(wave * 32 * 4);
   auto process_tile = [&](auto pc) {
     constexpr int PB = decltype(pc)::value;
     const int sidx = PB * kFwdRoundRows + wave * 32 + (lane & 31);
     const int rid = sRow[sidx];
     // this lane's query row as the B operand
     Pack8 qb[KS];
+    uint32_t bq = qrow;
+    opaque(bq);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qb[ks] = lds_read16((qrow ^ (uint32_t)(ks * 16)) + (uint32_t)(PB * 4) * TB);
+    for (int ks = 0; ks < KS; ++ks) qb[ks] = lds_read16((bq ^ (uint32_t)(ks * 16)) + (uint32_t)(PB * 4) * TB);
     __builtin_amdgcn_sched_barrier(0);
     f32x16 st[KT];  // S^T: register i of tile kt <-> key kt*32 + acc_row(i, hh), this lane's row
 #pragma unroll
@@ -311,10 +323,11 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) o = mfma32<T>(vt[dt][kt][s2], pf[kt][s2], o);
       // to the wave's row-major output tile, four features (8 bytes) at a time
+      uint32_t bo = ldsOut + (uint32_t)(((lane & 31) * LDO + 4 * hh) * 2);
+      opaque(bo);
 #pragma unroll
       for (int g = 0; g < 4; ++g)
-        *reinterpret_cast<uint2 *>(sOut + (lane & 31) * LDO + dt * 32 + 8 * g + 4 * hh) =
-            make_uint2(pack2<T>(o[4 * g], o[4 * g + 1]), pack2<T>(o[4 * g + 2], o[4 * g + 3]));
+        lds_write_vec<uint2>(bo + (uint32_t)((dt * 32 + 8 * g) * 2), make_uint2(pack2<T>(o[4 * g], o[4 * g + 1]), pack2<T>(o[4 * g + 2], o[4 * g + 3])));
       __builtin_amdgcn_sched_barrier(0);
     }
     // header of the partial
@@ -325,12 +338,16 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
     wave_lds_fence();
     // rows leave as 16-byte pieces: lane -> (row 4k + lane / 16, features 8 * (lane % 16))
     if ((lane & 15) * 8 < D) {
+      uint32_t br = ldsRow + (uint32_t)((lane >> 4) * 4), bx = ldsOut + (uint32_t)(((lane >> 4) * LDO + (lane & 15) * 8) * 2);
+      opaque(br);
+      opaque(bx);
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         const int row = 4 * k + (lane >> 4);
-        const int r2 = sRow[PB * kFwdRoundRows + wave * 32 + row], s2 = sSlot[PB * kFwdRoundRows + wave * 32 + row];
+        const int r2 = lds_read_vec<int>(br + (uint32_t)((PB * kFwdRoundRows + 4 * k) * 4));
+        const int s2 = lds_read_vec<int>(br + (uint32_t)((PB * kFwdRoundRows + 4 * k) * 4) + (uint32_t)(SM::oSlot - SM::oRow));
         if (r2 >= 0 && s2 < ws.cap) {
-          const Pack8 x = *reinterpret_cast<const Pack8 *>(sOut + row * LDO + (lane & 15) * 8);
+          const Pack8 x = lds_read16(bx + (uint32_t)(4 * k * LDO * 2));
           *reinterpret_cast<Pack8 *>(ws.part + (((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2) * D + (lane & 15) * 8) = x;
         }
       }

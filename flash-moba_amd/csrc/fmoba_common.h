@@ -408,6 +408,14 @@ __device__ __forceinline__ V lds_read_vec(uint32_t byte_addr) {
   return V{};
 #endif
 }
+template <typename V>
+__device__ __forceinline__ void lds_write_vec(uint32_t byte_addr, const V &v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  *(__attribute__((address_space(3))) V *)byte_addr = v;
+#else
+  (void)byte_addr, (void)v;
+#endif
+}
 // 8 x 16-bit operand of a transposing read: two 8-byte reads
 __device__ __forceinline__ Pack8 lds_tr8(uint32_t addr_lo, uint32_t addr_hi) {
   Pack8 r;
