@@ -451,26 +451,28 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     const int64_t trash = (int64_t)a.total_q * a.heads * ws.cap;  // spare row: takes the writes of absent rows, no branch
     auto dq_store = [&](auto pc, auto pp, auto tsc) {
       constexpr int TS = decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value;
-      uint16_t *sdQ = sdQ0 + (size_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2) * (TB / 2);
+      constexpr uint32_t SO = (uint32_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2) * TB;  // the tile that serves as staging
       // register i of feature tile d2 <-> feature d2*32 + acc_row(i, hh) of this wave's half, this lane's row
+      uint32_t bw = (uint32_t)(uintptr_t)sdQ0 + (uint32_t)(((lane & 31) * LDH + 4 * hh) * 2), unused_w = 0;
+      opaque(bw, unused_w);
 #pragma unroll
       for (int d2 = 0; d2 < NDH; ++d2)
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          *reinterpret_cast<uint2 *>(sdQ + (lane & 31) * LDH + d2 * 32 + 8 * g + 4 * hh) =
-              make_uint2(pack2<T>(dqa[d2][4 * g], dqa[d2][4 * g + 1]), pack2<T>(dqa[d2][4 * g + 2], dqa[d2][4 * g + 3]));
+          lds_write_vec<uint2>(bw + SO + (uint32_t)((d2 * 32 + 8 * g) * 2),
+                               make_uint2(pack2<T>(dqa[d2][4 * g], dqa[d2][4 * g + 1]), pack2<T>(dqa[d2][4 * g + 2], dqa[d2][4 * g + 3])));
       wave_lds_fence();
       constexpr int LPR = NDH * 4;        // lanes per part row (16 bytes each)
       constexpr int RPP = 64 / LPR;       // rows per pass
       const int col = (lane % LPR) * 8;
-      uint32_t bs = (uint32_t)(uintptr_t)(smem + SM::oRow) + (uint32_t)((px * 64 + lane / LPR) * 4), unused = 0;
-      opaque(bs, unused);
+      uint32_t bs = (uint32_t)(uintptr_t)(smem + SM::oRow) + (uint32_t)((px * 64 + lane / LPR) * 4);
+      uint32_t bx = (uint32_t)(uintptr_t)sdQ0 + (uint32_t)(((lane / LPR) * LDH + col) * 2);
+      opaque(bs, bx);
 #pragma unroll
       for (int k = 0; k < 32 / RPP; ++k) {
-        const int row = k * RPP + lane / LPR;
         const int r2 = lds_read_vec<int>(bs + (uint32_t)(TS * 32 + k * RPP) * 4);
         const int s2 = lds_read_vec<int>(bs + (uint32_t)(TS * 32 + k * RPP) * 4 + (uint32_t)(SM::oSlot - SM::oRow));
-        const Pack8 x = *reinterpret_cast<const Pack8 *>(sdQ + row * LDH + col);
+        const Pack8 x = lds_read16(bx + SO + (uint32_t)(k * RPP * LDH * 2));
         const bool ok = (r2 >= 0) & (s2 < ws.cap);
         const int64_t pidx = ok ? ((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2 : trash;
         if (kq * (NDH * 32) + col < D) *reinterpret_cast<Pack8 *>(ws.part + pidx * D + kq * (NDH * 32) + col) = x;
