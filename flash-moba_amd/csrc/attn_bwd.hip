@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     for (int sr = 0; sr < 2; ++sr) {
       const int j = sr * kBwdRoundRows + tid;
       const int r = list[min(j, n - 1)];
-      rid01[sr] = ((j < n) & (r >= 0) & (r < Lq)) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
+      rid01[sr] = tile_row_code(r, j < n, Lq);
     }
   }
 
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     auto rid_store = [&](int sr) {
       if (tid < kBwdRoundRows) {
         const int j = sr * kBwdRoundRows + ft;
-        v_rid = ((j < n) & (n_rid >= 0) & (n_rid < Lq)) ? n_rid : -1;  // rows outside the sequence (malformed pattern) are ignored
+        v_rid = tile_row_code(n_rid, j < n, Lq);
         sRid[(sr & 1) * kBwdRoundRows + ft] = v_rid;
       }
     };
@@ -249,18 +249,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       constexpr int RPI = 64 / VPR, NI = 32 / RPI;  // tile rows per instruction, instructions per tile
       const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
       const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(((sr & 1) * 4 + wave) * (int)TB);
-      const uint16_t *zero = reinterpret_cast<const uint16_t *>(&g_zero16);
-      const int qs = (int)a.q_row_stride, dos = (int)a.do_row_stride;  // (32 x 32 -> 64-bit products: one instruction each)
+      const uint32_t qs = (uint32_t)a.q_row_stride, dos = (uint32_t)a.do_row_stride;  // (32 x 32 -> 64-bit products: one instruction each)
+      // Absent rows and features past head_dim are fetched from a row and a piece that exist (tile_row_code): every
+      // load is unconditional, and what such data meets is an exact zero (probabilities of absent rows, K / V features
+      // past head_dim) or is never written out.
+      int src[NI];
+#pragma unroll
+      for (int i = 0; i < NI; ++i) src[i] = sRid[(sr & 1) * kBwdRoundRows + wave * 32 + i * RPI + rl] & 0x7fffffff;
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
-        const int row = i * RPI + rl;
-        const int rid = sRid[(sr & 1) * kBwdRoundRows + wave * 32 + row];
-        const int e = (p ^ tile_swz<HD>(row)) * 8;
-        const bool ok = (rid >= 0) & (e < D);
-        const uint16_t *gq = ok ? qg + ((int64_t)rid * qs + e) : zero;
-        const uint16_t *gd = ok ? dog + ((int64_t)rid * dos + e) : zero;
-        global_to_lds16(gq, ldsQ + dst + (uint32_t)(i * RPI * RB));
-        global_to_lds16(gd, ldsdO + dst + (uint32_t)(i * RPI * RB));
+        const uint32_t e = (uint32_t)min((p ^ tile_swz<HD>(i * RPI + rl)) * 8, D - 8);
+        global_to_lds16(qg + ((uint64_t)(uint32_t)src[i] * qs + e), ldsQ + dst + (uint32_t)(i * RPI * RB));
+        global_to_lds16(dog + ((uint64_t)(uint32_t)src[i] * dos + e), ldsdO + dst + (uint32_t)(i * RPI * RB));
       }
     };
 

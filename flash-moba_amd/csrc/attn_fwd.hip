@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
     for (int sr = 0; sr < 2; ++sr) {
       const int j = sr * kFwdRoundRows + tid;
       const int r = list[min(j, n - 1)];
-      rid01[sr] = ((j < n) & (r >= 0) & (r < Lq)) ? r : -1;  // rows outside the sequence (malformed pattern) are ignored
+      rid01[sr] = tile_row_code(r, j < n, Lq);
     }
   }
   {
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
   auto rid_store = [&](int sr) {
     if (tid < kFwdRoundRows) {
       const int j = sr * kFwdRoundRows + ft;
-      v_rid = ((j < n) & (n_rid >= 0) & (n_rid < Lq)) ? n_rid : -1;  // rows outside the sequence (malformed pattern) are ignored
+      v_rid = tile_row_code(n_rid, j < n, Lq);
       sRid[(sr & 1) * kFwdRoundRows + ft] = v_rid;
     }
   };
@@ -197,15 +197,16 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
     constexpr int RPI = 64 / VPR, NI = 32 / RPI;  // tile rows per instruction, instructions per tile
     const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
     const uint32_t dst = ldsQ + (uint32_t)__builtin_amdgcn_readfirstlane(((sr & 1) * 4 + wave) * (int)TB);
-    const uint16_t *zero = reinterpret_cast<const uint16_t *>(&g_zero16);
-    const int qs = (int)a.q_row_stride;  // (32 x 32 -> 64-bit product: one instruction)
+    const uint32_t qs = (uint32_t)a.q_row_stride;  // (32 x 32 -> 64-bit product: one instruction)
+    // Absent rows and features past head_dim are fetched from a row and a piece that exist (tile_row_code): every load
+    // is unconditional; the scores of absent rows are masked, and K is zero in the features past head_dim.
+    int src[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) src[i] = sRid[(sr & 1) * kFwdRoundRows + wave * 32 + i * RPI + rl] & 0x7fffffff;
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int row = i * RPI + rl;
-      const int rid = sRid[(sr & 1) * kFwdRoundRows + wave * 32 + row];
-      const int e = (p ^ tile_swz<HD>(row)) * 8;
-      const bool ok = (rid >= 0) & (e < D);
-      global_to_lds16(ok ? qg + ((int64_t)rid * qs + e) : zero, dst + (uint32_t)(i * RPI * RB));
+      const uint32_t e = (uint32_t)min((p ^ tile_swz<HD>(i * RPI + rl)) * 8, D - 8);
+      global_to_lds16(qg + ((uint64_t)(uint32_t)src[i] * qs + e), dst + (uint32_t)(i * RPI * RB));
     }
   };
   meta_issue(rid01[0]);

@@ -446,7 +446,15 @@ __device__ __forceinline__ void wait_all_loads() {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #endif
 }
-static __device__ uint4 g_zero16;  // 16 zero bytes: what the tile loads fetch for absent rows and for features past head_dim
+// Row id of a gathered tile row as it is kept in LDS: r itself if the entry is present and the row exists, else
+// negative with a row that exists in the low 31 bits (the entry's own if it exists: past the end of a list that is the
+// list's last row, whose data the column meets anyway; else row 0).  The tile loads fetch that row unconditionally, the
+// arithmetic treats every negative id as absent.
+__device__ __forceinline__ int tile_row_code(int r, bool present, int rows) {
+  const bool exists = (r >= 0) & (r < rows);
+  const int src = exists ? r : 0;
+  return (present & exists) ? src : (int)((uint32_t)src | 0x80000000u);
+}
 
 
 }  // namespace fmoba
