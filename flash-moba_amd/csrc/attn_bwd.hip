@@ -294,12 +294,19 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     const uint32_t troff = (uint32_t)(r0t * RB + ((((((lane >> 4) & 1) * 2 + ((li & 3) >> 1))) ^ tile_swz<HD>(r0t)) * 16) + (li & 1) * 8);
     // (re-made opaque wherever they are used: the operand addresses derived from them must not be kept in
     // registers from one use to the next, there are none to spare)
-    const uint32_t aQ = pairQ + rowoff, adO = pairdO + rowoff, tQ = pairQ + troff, tdO = pairdO + troff;
+    uint32_t aQ = pairQ + rowoff, adO = pairdO + rowoff, tQ = pairQ + troff, tdO = pairdO + troff;  // (never change; not const so that they can be made opaque in place)
     auto opaque = [](uint32_t &x, uint32_t &y) {
 #if defined(__HIP_DEVICE_COMPILE__)
       asm volatile("" : "+v"(x), "+v"(y));
 #else
       (void)x, (void)y;
+#endif
+    };
+    auto opaque1 = [](uint32_t &x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+      asm volatile("" : "+v"(x));
+#else
+      (void)x;
 #endif
     };
     uint16_t *sdS = reinterpret_cast<uint16_t *>(smem + SM::odS) + (DQP ? (size_t)px * 2 * 64 * LDS_ : (size_t)wave * 32 * LDS_);  // (px = 0 with 128 keys)
@@ -308,7 +315,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     // the middle of the round: Q's for even waves, dO's for odd ones, one half of it each with four key quarters
     uint16_t *sdQ0 = reinterpret_cast<uint16_t *>(smem + ((kq & 1) ? SM::odO : SM::oQ) + (size_t)(px * 2) * TB + (size_t)(kq >> 1) * (TB / 2));
     const int *pRow = sRow + px * 64;
-    const uint32_t smx0 = (uint32_t)(uintptr_t)(smem + SM::oRow) + (uint32_t)(px * 64 * 4 + hh * 16);  // softmax inputs of this lane's rows
+    uint32_t smx0 = (uint32_t)(uintptr_t)(smem + SM::oRow) + (uint32_t)(px * 64 * 4 + hh * 16);  // softmax inputs of this lane's rows
     Pack8 qa[2][KC], doa[2][KC];     // A operands of S and dP (this lane's row, its half of the head dim), double-buffered by chunk
     Pack8 dot[2][BC], qt[2][BC];     // dO^T / Q^T operands of the dV / dK products, double-buffered by chunk
     f32x4 lse4[2], del4[2];          // softmax inputs of a chunk's four rows
@@ -322,12 +329,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     auto ld_a = [&](auto pc, auto pp, auto tsc, auto gc) {
       constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value) * TB;
       constexpr int G = decltype(gc)::value;
-      uint32_t bq = aQ, bo = adO;
-      opaque(bq, bo);
+      opaque(aQ, adO);
 #pragma unroll
       for (int t = 0; t < KC; ++t) {
-        qa[G & 1][t] = lds_read16((bq ^ (uint32_t)((G * KC + t) * 16)) + TO);
-        doa[G & 1][t] = lds_read16((bo ^ (uint32_t)((G * KC + t) * 16)) + TO);
+        qa[G & 1][t] = lds_read16((aQ ^ (uint32_t)((G * KC + t) * 16)) + TO);
+        doa[G & 1][t] = lds_read16((adO ^ (uint32_t)((G * KC + t) * 16)) + TO);
       }
     };
     auto mm_a = [&](auto tsc, auto gc) {
@@ -348,16 +354,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     auto ld_b = [&](auto pc, auto pp, auto tsc, auto gc) {
       constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value) * TB;
       constexpr int G = decltype(gc)::value;
-      uint32_t bq = tQ, bo = tdO;
-      opaque(bq, bo);
+      opaque(tQ, tdO);
 #pragma unroll
       for (int t = 0; t < BC; ++t) {
         const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
         // rows 16 s2 + (0..3) + 4 hh and the same + 8, features dt * 32 ..
         const uint32_t xlo = (uint32_t)(dt * 4 * 16), xhi = (uint32_t)(((dt * 4) ^ TileSwz<HD>::kRow8) * 16);
         const uint32_t olo = TO + (uint32_t)(16 * s2 * RB), ohi = olo + (uint32_t)(8 * RB);
-        dot[G & 1][t] = lds_tr8((bo ^ xlo) + olo, (bo ^ xhi) + ohi);
-        qt[G & 1][t] = lds_tr8((bq ^ xlo) + olo, (bq ^ xhi) + ohi);
+        dot[G & 1][t] = lds_tr8((tdO ^ xlo) + olo, (tdO ^ xhi) + ohi);
+        qt[G & 1][t] = lds_tr8((tQ ^ xlo) + olo, (tQ ^ xhi) + ohi);
       }
     };
     auto mm_b = [&](auto tsc, auto gc) {
@@ -378,11 +383,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       // accumulator registers 4G..4G+3 hold rows TS * 32 + 8 G + 4 hh + (0..3); one address register, the rest
       // are offsets in the instructions
       constexpr uint32_t O = (uint32_t)(TS * 32 + 8 * G) * 4;
-      uint32_t bs = smx0, unused = 0;
-      opaque(bs, unused);
-      row4[G & 1] = lds_read_vec<int4>(bs + O);
-      lse4[G & 1] = lds_read_vec<f32x4>(bs + O + (uint32_t)(SM::oLse - SM::oRow));
-      del4[G & 1] = lds_read_vec<f32x4>(bs + O + (uint32_t)(SM::oDelta - SM::oRow));
+      opaque1(smx0);
+      row4[G & 1] = lds_read_vec<int4>(smx0 + O);
+      lse4[G & 1] = lds_read_vec<f32x4>(smx0 + O + (uint32_t)(SM::oLse - SM::oRow));
+      del4[G & 1] = lds_read_vec<f32x4>(smx0 + O + (uint32_t)(SM::oDelta - SM::oRow));
     };
     auto smx = [&](auto tsc, auto gc) {
       constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
