@@ -51,7 +51,6 @@ struct BwdSmem {
   static constexpr size_t oDelta = oLse + 2 * kBwdRoundRows * 4;
   static constexpr size_t bytes = oDelta + 2 * kBwdRoundRows * 4;
   static constexpr int LDR = HD + 4;  // floats, output transpose buffer [2][64 or 128 keys][LDR]
-  static_assert((size_t)2 * 128 * LDR * 4 <= bytes, "the output buffer reuses the tiles");
   static_assert((size_t)2 * 128 * LDQ * 2 <= 16 * tileBytes, "K and V pass through the tiles");
   static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
 };
@@ -580,38 +579,27 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     }
   }
 
-  // ---- dK^T / dV^T: with two pairs the second hands its sums to the first, which adds its own ------------------
+  // ---- dK^T / dV^T: every wave puts its sums into LDS (one copy per pair); with two pairs the rows add them on their way out
   __syncthreads();  // K and V have left LDS (lists without rows come here directly)
-  auto red_io = [&](bool add) {
+  constexpr int NCOPY = KB == 1 ? 2 : 1;
+  constexpr size_t kCopy = (size_t)2 * NKEY * LDR;  // floats of one copy: dV^T then dK^T
+  static_assert(NCOPY * kCopy * 4 <= SM::bytes, "the output buffers reuse the tiles");
+  {
+    float *mine = red + (size_t)px * kCopy;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        float *rp = red + (size_t)(kq * 32 + (lane & 31)) * LDR + dt * 32 + 8 * g + 4 * hh;
+        float *rp = mine + (size_t)(kq * 32 + (lane & 31)) * LDR + dt * 32 + 8 * g + 4 * hh;
         f32x4 v4, k4;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
           v4[jj] = dv[dt][4 * g + jj];
           k4[jj] = dk[dt][4 * g + jj];
         }
-        if (add) {
-          const f32x4 ov = *reinterpret_cast<const f32x4 *>(rp), ok = *reinterpret_cast<const f32x4 *>(rp + NKEY * LDR);
-#pragma unroll
-          for (int jj = 0; jj < 4; ++jj) {
-            v4[jj] += ov[jj];
-            k4[jj] += ok[jj];
-          }
-        }
         *reinterpret_cast<f32x4 *>(rp) = v4;
         *reinterpret_cast<f32x4 *>(rp + NKEY * LDR) = k4;
       }
-  };
-  if constexpr (KB == 1) {
-    if (px == 1) red_io(false);
-    __syncthreads();
-    if (px == 0) red_io(true);
-  } else {
-    red_io(false);
   }
   __syncthreads();
 
@@ -622,11 +610,21 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     const int key = v / VPR, e = (v - key * VPR) * 8;
     if (key0 + key >= Lk || e >= D) continue;
     const float *s0 = red + (size_t)key * LDR + e, *s1 = s0 + NKEY * LDR;
+    float fv[8], fk[8];
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      fv[w] = s0[w];
+      fk[w] = s1[w];
+      if constexpr (NCOPY == 2) {
+        fv[w] += s0[kCopy + w];
+        fk[w] += s1[kCopy + w];
+      }
+    }
     Pack8 ov, ok;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      ov.w[w] = pack2<T>(s0[2 * w], s0[2 * w + 1]);
-      ok.w[w] = pack2<T>(s1[2 * w] * a.softmax_scale, s1[2 * w + 1] * a.softmax_scale);
+      ov.w[w] = pack2<T>(fv[2 * w], fv[2 * w + 1]);
+      ok.w[w] = pack2<T>(fk[2 * w] * a.softmax_scale, fk[2 * w + 1] * a.softmax_scale);
     }
     *reinterpret_cast<Pack8 *>(dvg + (int64_t)key * a.dv_row_stride + e) = ov;
     *reinterpret_cast<Pack8 *>(dkg + (int64_t)key * a.dk_row_stride + e) = ok;
