@@ -271,10 +271,10 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
 // ------------------------------------------------------------------------------------
 constexpr int kBigCap = 32;  // running winners per row (K' = scored chunks kept)
 
-// CAP: entries of a row's list of running winners (16 or CAP).  With 16 and groups of 128 chunks the kernel needs
+// CAP: entries of a row's list of running winners (16 or kBigCap).  With 16 and groups of 128 chunks the kernel needs
 // half the LDS and fewer registers, and two workgroups share a compute unit.
 template <typename T, int HD, int NT, int CAP>
-__global__ __launch_bounds__(256, CAP < CAP ? 2 : 1) void topk_gate_big_kernel(TopkParams p) {
+__global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kernel(TopkParams p) {
   constexpr int KS = HD / 16;
   constexpr int LD = HD + 16;
   constexpr int GC = NT * 32;        // chunks per group

@@ -249,6 +249,24 @@ def test_varlen_sort_extremes_gaps_and_small_ranges(fm):
     assert (out == 0).all()
 
 
+def test_varlen_sort_size_classes(fm):
+    # segment lengths on both sides of every size class of the kernel (2048, 8192, 16384 keys), mixed in one call,
+    # with gaps, keys of both signs and a segment of equal keys
+    lens = [2048, 1, 2049, 0, 8192, 63, 8193, 64, 16384, 65, 16385, 2047, 300, 40000]
+    g = torch.Generator().manual_seed(21)
+    starts, ends, pos = [], [], 3
+    for n in lens:
+        starts.append(pos)
+        ends.append(pos + n)
+        pos += n + 5
+    src = torch.randint(-2 ** 31, 2 ** 31 - 1, (pos,), generator=g, dtype=torch.int64).to(torch.int32)
+    src[starts[12]:ends[12]] = -7
+    src[starts[4]:ends[4]] = torch.randint(0, 70000, (8192,), generator=g, dtype=torch.int64).to(torch.int32)
+    starts, ends = torch.tensor(starts, dtype=torch.int64), torch.tensor(ends, dtype=torch.int64)
+    out = fm.hip.varlen_sort(starts.cuda(), ends.cuda(), src.cuda())
+    assert torch.equal(out.cpu(), O.varlen_sort(starts, ends, src))
+
+
 def test_varlen_sort_restores_a_shuffled_csc(fm):
     # the op as the reference pipeline uses it: shuffle each column list, sort it back
     q, k, cuq, cuk = _gate_case(fm, 3, [700, 300], [700, 300], 4, 4, 64, 32, 6, True)
