@@ -1095,19 +1095,22 @@ static int launch_dq(const fmoba_attn_bwd_args &a, const uint16_t *ws, hipStream
   return 0;
 }
 
+// columns of a multiple of 128 keys: one workgroup (and one dQ partial per visit) per 128 keys
+static inline bool bwd_wide_blocks(const fmoba_attn_bwd_args &a) { return a.head_dim > 64 && a.lg_block_n % 128 == 0; }
+
 // Which form of the dQ computation a call uses.  The row-stationary form works on (128-row block, key block) steps
-// and is the faster one while a step has a dozen rows or more; with many chunks per sequence a step has one or
-// two rows and only the per-visit partials scale.  rows per step ~ 128 * (chunks a row selects) / (chunks per sequence).
+// and is the faster one while a step has enough rows; with many chunks per sequence a step has one or two rows and
+// only the per-visit partials scale.  Measured break-even points (16 heads of 128, 8K and 16K tokens per sequence,
+// top-k 8 to 32): a row selects a tenth of the chunks it may see (64-key blocks), three eighths with 128-key blocks,
+// where a visit leaves one partial per 128 keys.
 static int bwd_dq_partials(const fmoba_attn_bwd_args &a) {
   if (a.dq_mode == 1) return 0;
   if (a.dq_mode == 2) return 1;
   const double chunks_per_seq = (double)a.total_k / a.batch / a.lg_block_n;
   const double chunks_per_row = (double)a.max_visits_per_row * 64.0 / a.lg_block_n;
-  return 128.0 * chunks_per_row < 12.0 * chunks_per_seq;
+  const double seen = a.is_causal ? 0.5 * chunks_per_seq : chunks_per_seq;
+  return chunks_per_row < (bwd_wide_blocks(a) ? 0.37 : 0.10) * seen;
 }
-
-// columns of a multiple of 128 keys: one workgroup (and one dQ partial per visit) per 128 keys
-static inline bool bwd_wide_blocks(const fmoba_attn_bwd_args &a) { return a.head_dim > 64 && a.lg_block_n % 128 == 0; }
 // partial slots per (row, head): max_visits_per_row counts 64-key blocks; with 128-key blocks a row has half as many
 // visits (only the last column of a sequence can have an odd number of 64-key blocks)
 static inline int32_t bwd_partial_cap(const fmoba_attn_bwd_args &a) {

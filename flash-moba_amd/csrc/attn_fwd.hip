@@ -29,7 +29,9 @@
 
 namespace fmoba {
 
-constexpr int kFwdRowsDensity = 6;  // row-block form when a row selects at least 1/6 of the chunks it may see
+// row-block form when a row selects at least 10/50 (64-key blocks) resp. 10/27 (128-key blocks) of the chunks it may see:
+// measured break-even points (16 heads of 128, 8K and 16K tokens per sequence, top-k 8 to 32)
+constexpr int kFwdRowsDensity64 = 50, kFwdRowsDensity128 = 27;
 
 constexpr int kFwdRoundRows = 128;  // rows of a column list per round: one 32-row tile per wave
 
@@ -520,7 +522,8 @@ int run_fwd_rows(const fmoba_attn_fwd_args &a, int phases, hipStream_t s);
 
 // Which form runs.  The row-block form multiplies every row of a 128-row block with every chunk that
 // any of its rows selected, the column form only the selected pairs but pays a partial result per
-// visit: the first wins while a row selects more than about a sixth of the chunks it may see.
+// visit: the first wins while a row selects more than about a fifth of the chunks it may see (64-key blocks) or
+// more than about three eighths of them (128-key blocks, whose visits cost the column form less per key).
 static bool fwd_use_rows(const fmoba_attn_fwd_args &a) {
   if (a.fwd_mode == 1) return false;
   if (!fwd_rows_feasible(a)) return false;
@@ -528,7 +531,7 @@ static bool fwd_use_rows(const fmoba_attn_fwd_args &a) {
   const int64_t chunks_per_seq = std::max<int64_t>(1, ceil_div64(ceil_div64(std::max(a.total_k, 1), a.batch), a.lg_block_n));
   const int64_t chunks_per_row = std::max<int64_t>(1, (int64_t)a.max_visits_per_row * fwd_key_block(a.lg_block_n) / a.lg_block_n);
   const int64_t seen = a.is_causal ? (chunks_per_seq + 1) / 2 : chunks_per_seq;
-  return chunks_per_row * kFwdRowsDensity >= seen;
+  return chunks_per_row * (fwd_key_block(a.lg_block_n) == 128 ? kFwdRowsDensity128 : kFwdRowsDensity64) >= seen * 10;
 }
 
 template <typename T, int HD, int KB>
