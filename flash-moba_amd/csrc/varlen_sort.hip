@@ -15,7 +15,7 @@
 //
 // The LDS a workgroup reserves decides how many of them share a compute unit, so segments are
 // sorted by size class, one launch per class (2048, 8192, 16384 keys per buffer: seven workgroups of four
-// waves, two of eight, one of sixteen per compute unit), and a last launch for the segments that go through HBM.  Every
+// waves, two of eight, one of sixteen per compute unit; the last class also takes the segments that go through HBM).  Every
 // launch looks at all segments, 64 at a time with one coalesced load, and takes those of its class.
 #include "fmoba_common.h"
 
@@ -114,12 +114,13 @@ __device__ __forceinline__ int radix_passes(uint32_t mn, uint32_t mx, uint32_t *
   return diff == 0u ? 0 : (32 - __clz(diff) + 7) / 8;
 }
 
-// CAP > 0: segments of n_lo < n <= CAP keys, through LDS.  CAP == 0: segments of more than n_lo keys, through HBM.
+// Segments of n_lo < n <= n_hi keys: through LDS those of up to CAP keys, through HBM the longer ones (which only the
+// last class takes).
 // grid: batches of 64 segments x `split` workgroups that share a batch (8 for the smallest class ... 64, i.e. a segment each)
 template <int CAP, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void varlen_sort_kernel(const int64_t *starts, const int64_t *ends, int64_t nseg,
                                                                    const int32_t *src, int32_t *dst, int32_t *tmp, int64_t total,
-                                                                   int64_t n_lo, int split) {
+                                                                   int64_t n_lo, int64_t n_hi, int split) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint32_t *bufA = reinterpret_cast<uint32_t *>(smem);
   uint32_t *bufB = bufA + CAP;
@@ -143,7 +144,7 @@ __global__ __launch_bounds__(WAVES * 64) void varlen_sort_kernel(const int64_t *
       e_l = ends[sg];
     }
     const int64_t n_l = e_l - s_l;
-    const bool mine = sg < nseg && n_l > n_lo && (CAP == 0 || n_l <= CAP) && s_l >= 0 && e_l <= total &&
+    const bool mine = sg < nseg && n_l > n_lo && n_l <= n_hi && s_l >= 0 && e_l <= total &&
                       (lane % split) == part;
     unsigned long long todo = __ballot(mine);
     while (todo) {
@@ -154,7 +155,7 @@ __global__ __launch_bounds__(WAVES * 64) void varlen_sort_kernel(const int64_t *
       const uint32_t *in0 = reinterpret_cast<const uint32_t *>(src + s);
       uint32_t *out0 = reinterpret_cast<uint32_t *>(dst + s);
       uint32_t mn = 0xffffffffu, mx = 0u;
-      if (CAP > 0) {
+      if (n <= CAP) {
         for (int i = tid; i < (int)n; i += kThreads) {
           const uint32_t k = in0[i] ^ 0x80000000u;
           bufA[i] = k;
@@ -214,7 +215,7 @@ __global__ void fill_zero_i32_kernel(int32_t *p, int64_t n) {
 
 template <int CAP, int WAVES>
 static int launch_sort_class(const int64_t *seg_starts, const int64_t *seg_ends, int64_t num_segments, const int32_t *src, int32_t *dst,
-                             int32_t *tmp, int64_t total, int64_t n_lo, int split, hipStream_t s) {
+                             int32_t *tmp, int64_t total, int64_t n_lo, int64_t n_hi, int split, hipStream_t s) {
   const size_t smem = (size_t)2 * CAP * 4 + (size_t)WAVES * 256 * 4 + 4 * 4 + 2 * WAVES * 4;
   auto kern = varlen_sort_kernel<CAP, WAVES>;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
@@ -225,7 +226,7 @@ static int launch_sort_class(const int64_t *seg_starts, const int64_t *seg_ends,
   const int64_t items = nbatch * split;
   const int64_t grid = items < 4096 ? items : 4096;  // a workgroup takes every 4096th item: few dispatches, and runs of long segments spread out
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WAVES * 64), smem, s, seg_starts, seg_ends, num_segments, src, dst, tmp, total, n_lo,
-                     split);
+                     n_hi, split);
   FMOBA_LAUNCH_CHECK("varlen_sort");
   return 0;
 }
@@ -249,12 +250,10 @@ extern "C" int fmoba_varlen_sort(const int64_t *seg_starts, const int64_t *seg_e
   FMOBA_LAUNCH_CHECK("varlen_sort(zero)");
   if (num_segments == 0) return 0;
   int32_t *tmp = reinterpret_cast<int32_t *>(workspace);
-  if (int rc = launch_sort_class<2048, 4>(seg_starts, seg_ends, num_segments, src, dst, tmp, total, 0, 8, s)) return rc;
+  if (int rc = launch_sort_class<2048, 4>(seg_starts, seg_ends, num_segments, src, dst, tmp, total, 0, 2048, 8, s)) return rc;
   if (total > 2048)
-    if (int rc = launch_sort_class<8192, 8>(seg_starts, seg_ends, num_segments, src, dst, tmp, total, 2048, 32, s)) return rc;
+    if (int rc = launch_sort_class<8192, 8>(seg_starts, seg_ends, num_segments, src, dst, tmp, total, 2048, 8192, 32, s)) return rc;
   if (total > 8192)
-    if (int rc = launch_sort_class<kLdsCapMax, 16>(seg_starts, seg_ends, num_segments, src, dst, tmp, total, 8192, 64, s)) return rc;
-  if (total > kLdsCapMax)
-    if (int rc = launch_sort_class<0, 16>(seg_starts, seg_ends, num_segments, src, dst, tmp, total, kLdsCapMax, 64, s)) return rc;
+    if (int rc = launch_sort_class<kLdsCapMax, 16>(seg_starts, seg_ends, num_segments, src, dst, tmp, total, 8192, INT64_MAX, 64, s)) return rc;
   return 0;
 }
