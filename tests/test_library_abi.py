@@ -66,6 +66,35 @@ def test_workspace_queries_are_pure_host_functions():
     assert lib.fmoba_attn_fwd_key_block(64) == 64 and lib.fmoba_attn_fwd_key_block(128) == 128 and lib.fmoba_attn_fwd_key_block(192) == 64
 
 
+@pytest.mark.parametrize("lens,chunk,topk,fwd_rows,dq_partials", [
+    ([8192], 128, 8, 0, 1),           # a row selects 8 of 32 visible 128-key chunks: columns, partials
+    ([4096, 4096], 128, 8, 1, 0),     # 8 of 16: row blocks in both passes
+    ([32768], 128, 16, 0, 1),         # 16 of 128
+    ([8192] * 8, 64, 32, 1, 0),       # the headline density, 32 of 64 visible 64-key chunks: row blocks
+    ([8192, 8192], 64, 16, 1, 0),     # 16 of 64: still row blocks with 64-key blocks
+    ([8192, 8192], 64, 8, 0, 0),      # 8 of 64: column forward, but the row-block dQ until a tenth
+    ([262144], 128, 16, 0, 1),
+])
+def test_form_choice_follows_the_measured_break_even_points(lens, chunk, topk, fwd_rows, dq_partials):
+    lib = H.load_library()
+    T, L = sum(lens), max(lens)
+    f = H.AttnFwdArgs()
+    f.total_q = f.total_k = T
+    f.heads = f.heads_k = 16
+    f.head_dim, f.batch, f.lg_block_n, f.is_causal = 128, len(lens), chunk, 1
+    f.max_seqlen_q = f.max_seqlen_k = L
+    f.max_cols = (L + chunk - 1) // chunk
+    f.max_visits_per_row = topk * (chunk // lib.fmoba_attn_fwd_key_block(chunk))
+    assert lib.fmoba_attn_fwd_uses_row_blocks(ctypes.byref(f)) == fwd_rows
+    a = H.AttnBwdArgs()
+    a.total_q = a.total_k = T
+    a.heads = a.heads_k = 16
+    a.head_dim, a.batch, a.lg_block_n, a.is_causal = 128, len(lens), chunk, 1
+    a.max_seqlen_q = a.max_seqlen_k = L
+    a.max_visits_per_row = topk * (chunk // 64)
+    assert lib.fmoba_attn_bwd_uses_partials(ctypes.byref(a)) == dq_partials
+
+
 def test_struct_sizes_match_the_header_layout():
     # pointers and int64 are 8 bytes, int32/float 4; sizes follow from the field lists
     assert ctypes.sizeof(H.MeanPoolArgs) == 4 * 8 + 6 * 4 + 4 * 8
