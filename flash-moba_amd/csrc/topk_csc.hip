@@ -672,10 +672,17 @@ __global__ __launch_bounds__(256) void csc_scan_kernel(TopkParams p) {
     const int c = c0 + tid;
     int nnz = 0;
     if (c < p.max_cols) {
-      for (int s = 0; s < nseg_b; ++s) {
-        const int v = segc[(int64_t)s * p.max_cols + c];
-        segc[(int64_t)s * p.max_cols + c] = nnz;
-        nnz += v;
+      // eight counts in flight at a time (a long sequence has over a hundred segments, and a load that waits for
+      // the store before it costs a round trip each)
+      for (int s0 = 0; s0 < nseg_b; s0 += 8) {
+        int v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = s0 + i < nseg_b ? segc[(int64_t)(s0 + i) * p.max_cols + c] : 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (s0 + i < nseg_b) segc[(int64_t)(s0 + i) * p.max_cols + c] = nnz;
+          nnz += v[i];
+        }
       }
     }
     sscan[tid] = nnz;
