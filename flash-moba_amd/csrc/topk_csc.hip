@@ -14,14 +14,25 @@
 namespace fmoba {
 
 constexpr int kGateRows = 128;   // query rows per workgroup (4 waves x 32)
-constexpr int kSegRows = 2048;   // rows per counting segment
+constexpr int kSegRows = 2048;   // rows per counting segment (fewer for small problems, see csc_seg_rows)
 
 struct TopkParams {
   fmoba_fused_topk_args a;
   uint32_t *sel;      // [heads][W][total_q] selection bits, word w covers chunks 32w..32w+31
   int32_t *segcnt;    // [batch][heads][nseg][max_cols]
-  int32_t W, nseg, max_cols;
+  int32_t W, nseg, max_cols, seg_rows;
 };
+
+// Rows per counting segment.  A wave of the fill kernel walks one segment of one 32-chunk word column, 64 rows at a
+// time, one after the other: segments of 2048 rows keep the counts small, but a short batch (one sequence of 8192
+// tokens: 128 waves) would leave most of the GPU idle for the 32 steps of a segment, so segments shrink (down to 256
+// rows, a multiple of the gate's 128-row blocks) until there are a few thousand waves.
+static inline int csc_seg_rows(int64_t batch, int64_t heads, int64_t max_seqlen_q, int64_t W) {
+  int seg_rows = kSegRows;
+  const int64_t lq = max_seqlen_q > 0 ? max_seqlen_q : 1;
+  while (seg_rows > 256 && batch * heads * W * ((lq + seg_rows - 1) / seg_rows) < 2048) seg_rows >>= 1;
+  return seg_rows;
+}
 
 template <typename T, int HD, int NT>
 __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_kernel(TopkParams p) {
@@ -219,7 +230,7 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
   // selection words (32 chunks each), own chunk forced in causal mode
   const bool has_self = a.is_causal && valid && rp >= 0;
   const int pself = has_self ? rp / B : -1;
-  const int seg = m0 / kSegRows;
+  const int seg = m0 / p.seg_rows;
   uint32_t *selp = p.sel + (int64_t)h * p.W * a.total_q + q0 + r;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
@@ -647,7 +658,7 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
     const int t = v / kGateRows, slot_r = v - t * kGateRows;
     if (m0 + slot_r < Lq) p.sel[((int64_t)h * p.W + t) * a.total_q + q0 + m0 + slot_r] = sSel[v];
   }
-  const int seg = m0 / kSegRows;
+  const int seg = m0 / p.seg_rows;
   for (int c = tid; c < p.max_cols; c += 256) {
     const int v = sHist[c];
     if (v) atomicAdd(&p.segcnt[(((int64_t)b * a.heads + h) * p.nseg + seg) * p.max_cols + c], v);
@@ -660,7 +671,7 @@ __global__ __launch_bounds__(256) void csc_scan_kernel(TopkParams p) {
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int q0 = a.cu_seqlens_q[b];
   const int Lq = a.cu_seqlens_q[b + 1] - q0;
-  const int nseg_b = (Lq + kSegRows - 1) / kSegRows;
+  const int nseg_b = (Lq + p.seg_rows - 1) / p.seg_rows;
   const int64_t bh = (int64_t)b * a.heads + h;
   int32_t *segc = p.segcnt + bh * p.nseg * p.max_cols;
   const int64_t base = ((int64_t)q0 * a.heads + (int64_t)Lq * h) * a.topk;
@@ -707,16 +718,16 @@ __global__ __launch_bounds__(256) void csc_scan_kernel(TopkParams p) {
   for (int64_t i = start + tid; i < end; i += 256) a.flat_indices[i] = 0;
 }
 
-// grid (nseg * W, heads, batch), block 64: one wave walks 2048 rows of one 32-chunk word column
+// grid (nseg * W, heads, batch), block 64: one wave walks the rows of one segment of one 32-chunk word column
 __global__ __launch_bounds__(64) void csc_fill_kernel(TopkParams p) {
   const fmoba_fused_topk_args &a = p.a;
   const int seg = blockIdx.x / p.W, wc = blockIdx.x - seg * p.W;
   const int h = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
   const int q0 = a.cu_seqlens_q[b];
   const int Lq = a.cu_seqlens_q[b + 1] - q0;
-  const int r0 = seg * kSegRows;
+  const int r0 = seg * p.seg_rows;
   if (r0 >= Lq) return;
-  const int r1 = min(Lq, r0 + kSegRows);
+  const int r1 = min(Lq, r0 + p.seg_rows);
   const int64_t bh = (int64_t)b * a.heads + h;
   int64_t pos = 0;
   {
@@ -841,7 +852,7 @@ extern "C" size_t fmoba_fused_topk_workspace_bytes(int32_t batch, int32_t total_
   if (batch <= 0 || heads <= 0 || chunk <= 0 || total_q < 0) return 0;
   const int64_t max_cols = ceil_div64(max_seqlen_k, chunk);
   const int64_t W = ceil_div64(max_cols, 32);
-  const int64_t nseg = ceil_div64(max_seqlen_q > 0 ? max_seqlen_q : 1, kSegRows);
+  const int64_t nseg = ceil_div64(max_seqlen_q > 0 ? max_seqlen_q : 1, csc_seg_rows(batch, heads, max_seqlen_q, W));
   return align256((size_t)heads * W * total_q * 4) + align256((size_t)batch * heads * nseg * max_cols * 4) + 256;
 }
 
@@ -954,7 +965,8 @@ extern "C" int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream) {
   p.a = *a;
   p.max_cols = max_cols;
   p.W = ceil_div(max_cols, 32);
-  p.nseg = ceil_div(a->max_seqlen_q > 0 ? a->max_seqlen_q : 1, kSegRows);
+  p.seg_rows = csc_seg_rows(a->batch, a->heads, a->max_seqlen_q, p.W);
+  p.nseg = ceil_div(a->max_seqlen_q > 0 ? a->max_seqlen_q : 1, p.seg_rows);
   const size_t sel_bytes = align256((size_t)a->heads * p.W * a->total_q * 4);
   const size_t seg_bytes = align256((size_t)a->batch * a->heads * p.nseg * max_cols * 4);
   FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= sel_bytes + seg_bytes, "fused_topk: workspace too small (%zu < %zu)",
