@@ -263,6 +263,30 @@ __device__ __forceinline__ int shfl_xor32_i(int v) {
   const UPair p = swap32((uint32_t)v);
   return (int)((threadIdx.x & 32) ? p.a : p.b);
 }
+// Column sums of a 32 x 32 bit matrix held one row per lane (row = lane % 32; both halves of the wave may hold a copy):
+// five block-swap steps transpose it (step S exchanges, between lanes l and l ^ S, the bits whose position differs
+// from the lane in bit S), then lane j holds column j and counts its bits.  The exchange is ds_swizzle in its
+// bit-mask mode, which permutes within groups of 32 lanes and touches no memory.
+template <int S>
+__device__ __forceinline__ uint32_t bit_transpose_step(uint32_t x, int lane) {
+  constexpr uint32_t m = S == 16 ? 0x0000ffffu : S == 8 ? 0x00ff00ffu : S == 4 ? 0x0f0f0f0fu : S == 2 ? 0x33333333u : 0x55555555u;
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t y = (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, (S << 10) | 0x1f);
+#else
+  const uint32_t y = x;
+#endif
+  return (lane & S) ? (((y >> S) & m) | (x & ~m)) : ((x & m) | ((y & m) << S));
+}
+__device__ __forceinline__ int bit_column_count32(uint32_t row_word, int lane) {
+  uint32_t x = row_word;
+  x = bit_transpose_step<16>(x, lane);
+  x = bit_transpose_step<8>(x, lane);
+  x = bit_transpose_step<4>(x, lane);
+  x = bit_transpose_step<2>(x, lane);
+  x = bit_transpose_step<1>(x, lane);
+  return __popc(x);
+}
+
 // reductions over the two halves of a wave (lanes l and l ^ 32), result in both lanes
 __device__ __forceinline__ int sum_xor32_i(int v) {
   const UPair p = swap32((uint32_t)v);

@@ -252,15 +252,9 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
       if (has_self && (pself >> 5) == t) w |= 1u << (pself & 31);
       if (!valid) w = 0u;
       if (valid && hh == 0) selp[(int64_t)t * a.total_q] = w;
-      // per-chunk counts of this wave's 32 rows
-      int mycnt = 0;
-      const uint32_t wc = (hh == 0) ? w : 0u;
-      if (__any(wc != 0u)) {
-#pragma unroll
-        for (int j = 0; j < 32; ++j) {
-          const unsigned long long m = __ballot((wc >> j) & 1u);
-          if (lane == j) mycnt = __popcll(m);
-        }
+      // per-chunk counts of this wave's 32 rows (both halves of the wave hold the rows' words)
+      if (__any(w != 0u)) {
+        const int mycnt = bit_column_count32(w, lane);
         if (lane < 32 && mycnt) atomicAdd(&sHist[t * 32 + lane], mycnt);
       }
     }
