@@ -102,9 +102,9 @@ def time_events(fn, iters, warmup=1):
 # what the same counter reads for a plain 1 GiB copy (the summary of those runs is kept under profiles/).
 # Counter runs cannot be made from inside this script, so the figures are the committed measurement.
 MEASURED_TRAFFIC_BYTES = {
-    ("headline", "attn_fwd_rows_kernel"): 1.503e9,
-    ("headline", "attn_bwd_dkdv_kernel"): 6.678e9,
-    ("headline", "attn_bwd_dq_kernel"): 5.079e9,
+    ("headline", "attn_fwd_rows_kernel"): 1.499e9,
+    ("headline", "attn_bwd_dkdv_kernel"): 6.676e9,
+    ("headline", "attn_bwd_dq_kernel"): 5.076e9,
 }
 
 
