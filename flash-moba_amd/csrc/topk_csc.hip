@@ -11,6 +11,8 @@
 //                      ascending, so no sort pass is needed afterwards.
 #include "fmoba_common.h"
 
+#include <mutex>
+
 namespace fmoba {
 
 constexpr int kGateRows = 128;   // query rows per workgroup (4 waves x 32)
@@ -911,7 +913,8 @@ static int launch_gate_hd(const TopkParams &p, dim3 grid, hipStream_t s) {
 }
 }  // namespace fmoba
 
-extern "C" int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream) {
+// The call behind both entry points: everything of `a` except its workspace fields, which come as arguments.
+static int fused_topk_run(const fmoba_fused_topk_args *a, void *workspace, size_t workspace_bytes, void *stream) {
   using namespace fmoba;
   FMOBA_REQUIRE(a != nullptr, "fused_topk: null args");
   FMOBA_REQUIRE(a->dtype == FMOBA_DTYPE_F16 || a->dtype == FMOBA_DTYPE_BF16, "FlashMoBA only supports fp16 and bf16 data types");
@@ -963,10 +966,10 @@ extern "C" int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream) {
   p.nseg = ceil_div(a->max_seqlen_q > 0 ? a->max_seqlen_q : 1, p.seg_rows);
   const size_t sel_bytes = align256((size_t)a->heads * p.W * a->total_q * 4);
   const size_t seg_bytes = align256((size_t)a->batch * a->heads * p.nseg * max_cols * 4);
-  FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= sel_bytes + seg_bytes, "fused_topk: workspace too small (%zu < %zu)",
-                a->workspace_bytes, sel_bytes + seg_bytes);
-  uintptr_t wsp = ((uintptr_t)a->workspace + 255) & ~(uintptr_t)255;
-  FMOBA_REQUIRE(wsp + sel_bytes + seg_bytes <= (uintptr_t)a->workspace + a->workspace_bytes, "fused_topk: workspace too small after alignment");
+  FMOBA_REQUIRE(workspace != nullptr && workspace_bytes >= sel_bytes + seg_bytes, "fused_topk: workspace too small (%zu < %zu)",
+                workspace_bytes, sel_bytes + seg_bytes);
+  uintptr_t wsp = ((uintptr_t)workspace + 255) & ~(uintptr_t)255;
+  FMOBA_REQUIRE(wsp + sel_bytes + seg_bytes <= (uintptr_t)workspace + workspace_bytes, "fused_topk: workspace too small after alignment");
   p.sel = reinterpret_cast<uint32_t *>(wsp);
   p.segcnt = reinterpret_cast<int32_t *>(wsp + sel_bytes);
 
@@ -1003,4 +1006,45 @@ extern "C" int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream) {
     FMOBA_LAUNCH_CHECK("topk_raw_kernel");
   }
   return 0;
+}
+
+extern "C" int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream) {
+  FMOBA_REQUIRE(a != nullptr, "fused_topk: null args");
+  return fused_topk_run(a, a->workspace, a->workspace_bytes, stream);
+}
+
+// ------------------------------------------------------------------------------------
+// The same call for callers that cannot allocate device memory (HIP graph capture, serving loops): selection bits and
+// segment counts live in a fixed array of the code object instead of a caller's workspace.  Every device that loads
+// the library holds its own copy of the array at its own address, which the runtime tells once per device.
+// ------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[FMOBA_STATIC_SCRATCH_BYTES];
+
+namespace fmoba {
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device, null until asked for
+}  // namespace fmoba
+
+extern "C" int fmoba_fused_topk_static(const fmoba_fused_topk_args *a, void *stream) {
+  using namespace fmoba;
+  FMOBA_REQUIRE(a != nullptr, "fused_topk_static: null args");
+  const size_t need = fmoba_fused_topk_workspace_bytes(a->batch, a->total_q, a->heads, a->max_seqlen_q, a->max_seqlen_k, a->chunk);
+  FMOBA_REQUIRE(need <= (size_t)FMOBA_STATIC_SCRATCH_BYTES,
+                "fused_topk_static: this call needs %zu bytes of scratch memory, the library's fixed buffer holds %zu; use fmoba_fused_topk with a workspace",
+                need, (size_t)FMOBA_STATIC_SCRATCH_BYTES);
+  int dev = -1;
+  FMOBA_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, "fused_topk_static: no current HIP device (or its index is above %d)", kMaxDevices - 1);
+  void *ptr = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+      void *p = nullptr;
+      const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      FMOBA_REQUIRE(e == hipSuccess && p != nullptr, "fused_topk_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+      g_scratch_ptr[dev] = p;
+    }
+    ptr = g_scratch_ptr[dev];
+  }
+  return fused_topk_run(a, ptr, (size_t)FMOBA_STATIC_SCRATCH_BYTES, stream);
 }

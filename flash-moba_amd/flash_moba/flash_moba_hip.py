@@ -86,6 +86,7 @@ EXPORTS = {
     "fmoba_mean_pool": (c_i32, [ctypes.POINTER(MeanPoolArgs), c_vp]),
     "fmoba_fused_topk_workspace_bytes": (c_sz, [c_i32, c_i32, c_i32, c_i32, c_i32, c_i32]),
     "fmoba_fused_topk": (c_i32, [ctypes.POINTER(FusedTopkArgs), c_vp]),
+    "fmoba_fused_topk_static": (c_i32, [ctypes.POINTER(FusedTopkArgs), c_vp]),
     "fmoba_varlen_sort_workspace_bytes": (c_sz, [c_i64]),
     "fmoba_varlen_sort": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_sz, c_vp]),
     "fmoba_attn_fwd_key_block": (c_i32, [c_i32]),

@@ -91,6 +91,18 @@ typedef struct {
 size_t fmoba_fused_topk_workspace_bytes(int32_t batch, int32_t total_q, int32_t heads,
                                         int32_t max_seqlen_q, int32_t max_seqlen_k, int32_t chunk);
 int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream);
+/* The same call without a workspace, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference, whose host code allocates on every call.  `workspace` / `workspace_bytes` of `a` are
+ * ignored: selection bits and segment counts live in a fixed array inside the library's code object
+ * (FMOBA_STATIC_SCRATCH_BYTES per device, held until the process ends).  The call fails with a clear
+ * error, before anything is launched, when fmoba_fused_topk_workspace_bytes() of the same sizes exceeds
+ * that limit (the headline shape -- 65536 tokens, 16 heads, 224 chunks -- needs 30.3 MB and fits).
+ * It calls no hipMalloc / hipFree.  All calls on one device share the array: calls that overlap on one
+ * device (different streams or threads) race; calls in stream order are safe, every call clears what
+ * it needs zeroed with a fill kernel of its own. */
+#define FMOBA_STATIC_SCRATCH_BYTES (32u << 20)
+int fmoba_fused_topk_static(const fmoba_fused_topk_args *a, void *stream);
 
 /* ------------------------------------------------------------------------------------
  * Segmented ascending sort of signed int32 keys with 64-bit segment offsets.
