@@ -954,10 +954,11 @@ __global__ __launch_bounds__(512, 4) void attn_bwd_dq_kernel(fmoba_attn_bwd_args
 // runs four of them side by side.  Lane li of a group owns the 16-byte piece li of the row.
 // ------------------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(256) void attn_bwd_dq_combine_kernel(fmoba_attn_bwd_args a, BwdWs ws) {
-  __shared__ int sOrd[16][16];
+__global__ __launch_bounds__(256) void attn_bwd_dq_combine_kernel(fmoba_attn_bwd_args a, BwdWs ws, int capl) {
+  extern __shared__ __attribute__((aligned(16))) int sOrdAll[];  // [16 groups][capl]: slot of the partial of rank r
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, grp = lane >> 4, li = lane & 15;
   const int sg = wv * 4 + grp;  // group of the block
+  int *sOrd = sOrdAll + (size_t)sg * capl;
   const int64_t total = (int64_t)a.total_q * a.heads;
   const int64_t rh_raw = (int64_t)blockIdx.x * 16 + sg;  // (global row) * heads + head
   const bool valid = rh_raw < total;
@@ -975,36 +976,25 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_combine_kernel(fmoba_attn_bwd
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-  for (int base = 0; base < nmax; base += 16) {
-    const int cntb = min(16, max(n - base, 0));
-    const int cj = li < cntb ? pid[base + li] : 0x7fffffff;
-    int rank = 0;
+  // ranks over the whole row: the order of the sum does not depend on which slot a visit got
+  group_rank_order(pid, 1, n, nmax, sOrd, lane);
+  if (mine) {
+    auto add = [&](const Pack8 &x) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int ci = __shfl(cj, (lane & 48) | i, 64);
-      rank += (ci < cj || (ci == cj && i < li)) ? 1 : 0;
-    }
-    wave_lds_fence();
-    if (li < cntb) sOrd[sg][rank] = li;
-    wave_lds_fence();
-    if (mine) {
-      auto add = [&](const Pack8 &x) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          acc[2 * k] += elem_to_float<T>((uint16_t)(x.w[k] & 0xffffu));
-          acc[2 * k + 1] += elem_to_float<T>((uint16_t)(x.w[k] >> 16));
-        }
-      };
-      int t = 0;
-      for (; t + 4 <= cntb; t += 4) {  // independent loads, four in flight
-        Pack8 x[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) x[u] = ld_global16(part + (int64_t)(base + sOrd[sg][t + u]) * D + c8);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) add(x[u]);
+      for (int k = 0; k < 4; ++k) {
+        acc[2 * k] += elem_to_float<T>((uint16_t)(x.w[k] & 0xffffu));
+        acc[2 * k + 1] += elem_to_float<T>((uint16_t)(x.w[k] >> 16));
       }
-      for (; t < cntb; ++t) add(ld_global16(part + (int64_t)(base + sOrd[sg][t]) * D + c8));
+    };
+    int t = 0;
+    for (; t + 4 <= n; t += 4) {  // independent loads, four in flight
+      Pack8 x[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) x[u] = ld_global16(part + (int64_t)sOrd[t + u] * D + c8);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) add(x[u]);
     }
+    for (; t < n; ++t) add(ld_global16(part + (int64_t)sOrd[t] * D + c8));
   }
   if (valid && mine) {
     Pack8 o;
@@ -1142,7 +1132,14 @@ static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hi
   if (phases & FMOBA_BWD_DQ) {
     if (partials) {
       const int64_t rows = (int64_t)a.total_q * a.heads;
-      hipLaunchKernelGGL(attn_bwd_dq_combine_kernel<T>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a, ws);
+      const int capl = combine_order_entries(ws.cap);
+      const size_t smem = (size_t)16 * capl * 4;
+      auto kern = attn_bwd_dq_combine_kernel<T>;
+      if (smem > 32 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+        set_error("attn_bwd: a row with up to %d visits needs %zu bytes of LDS for the order of its partial results", ws.cap, smem);
+        return 2;
+      }
+      hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 15) / 16)), dim3(256), smem, s, a, ws, capl);
     } else {
       int rc = a.head_dim <= 64 ? launch_dq<T, 64>(a, ws.ds, s) : launch_dq<T, 128>(a, ws.ds, s);
       if (rc) return rc;

@@ -381,11 +381,12 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
 // headers, order, rows) is mostly waiting, so a wave runs four of them side by side.  Lane li of a group owns the
 // 16-byte piece li of the row.
 template <typename T>
-__global__ __launch_bounds__(256) void attn_fwd_combine_kernel(fmoba_attn_fwd_args a, FwdWs ws) {
-  __shared__ int sOrd[16][16];
+__global__ __launch_bounds__(256) void attn_fwd_combine_kernel(fmoba_attn_fwd_args a, FwdWs ws, int capl) {
+  extern __shared__ __attribute__((aligned(16))) int sOrdAll[];  // [16 groups][capl]: slot of the partial of rank r
   __shared__ float sWgt[16][16], sWl[16][16];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, grp = lane >> 4, li = lane & 15;
   const int sg = wv * 4 + grp;  // group of the block
+  int *sOrd = sOrdAll + (size_t)sg * capl;
   const int64_t total = (int64_t)a.total_q * a.heads;
   const int64_t rh_raw = (int64_t)blockIdx.x * 16 + sg;  // (global row) * heads + head
   const bool valid = rh_raw < total;
@@ -404,23 +405,19 @@ __global__ __launch_bounds__(256) void attn_fwd_combine_kernel(fmoba_attn_fwd_ar
   float L = 0.f, M = -INFINITY;
   const float4 *hdr = ws.hdr + rh * ws.cap;
   const uint16_t *part = ws.part + rh * ws.cap * D;
-  // partials are merged in ascending key-block order (the slot a visit got is arbitrary), 16 at a time
+  // The slot a visit got is arbitrary (a counter handed it out), the sum must not depend on it: every partial gets
+  // its rank in ascending key-block order over the WHOLE row (equal ids, a malformed pattern, are ordered by slot),
+  // and the partials are merged in rank order, 16 at a time.
+  group_rank_order(reinterpret_cast<const int *>(hdr) + 2, 4, n, nmax, sOrd, lane);
   for (int base = 0; base < nmax; base += 16) {
     const int cntb = min(16, max(n - base, 0));
     float mj = -INFINITY, lj = 0.f;
-    int cj = 0x7fffffff;
+    int slot = 0;
     if (li < cntb) {
-      const float4 x = hdr[base + li];
+      slot = sOrd[base + li];
+      const float4 x = hdr[slot];
       mj = x.x;
       lj = x.y;
-      cj = __float_as_int(x.z);
-    }
-    // rank of this lane's partial in the batch; equal ids (malformed pattern) are ordered by slot
-    int rank = 0;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int ci = __shfl(cj, (lane & 48) | i, 64);
-      rank += (ci < cj || (ci == cj && i < li)) ? 1 : 0;
     }
     float mb = mj;
 #pragma unroll
@@ -435,9 +432,8 @@ __global__ __launch_bounds__(256) void attn_fwd_combine_kernel(fmoba_attn_fwd_ar
     const float wj = (li < cntb) ? __builtin_amdgcn_exp2f(mj - Mu) : 0.f;
     wave_lds_fence();
     if (li < cntb) {
-      sOrd[sg][rank] = li;
-      sWgt[sg][rank] = wj;
-      sWl[sg][rank] = wj * lj;
+      sWgt[sg][li] = wj;
+      sWl[sg][li] = wj * lj;
     }
     wave_lds_fence();
     // sums in rank order: every lane of the group adds the same sequence
@@ -456,13 +452,13 @@ __global__ __launch_bounds__(256) void attn_fwd_combine_kernel(fmoba_attn_fwd_ar
         float w[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          x[u] = ld_global16(part + (int64_t)(base + sOrd[sg][t + u]) * D + c8);
+          x[u] = ld_global16(part + (int64_t)sOrd[base + t + u] * D + c8);
           w[u] = sWgt[sg][t + u];
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) add(x[u], w[u]);
       }
-      for (; t < cntb; ++t) add(ld_global16(part + (int64_t)(base + sOrd[sg][t]) * D + c8), sWgt[sg][t]);
+      for (; t < cntb; ++t) add(ld_global16(part + (int64_t)sOrd[base + t] * D + c8), sWgt[sg][t]);
     }
   }
   if (!valid) return;
@@ -563,8 +559,16 @@ static int run_fwd(const fmoba_attn_fwd_args &a, const FwdWs &ws, int phases, hi
       rc = kb == 128 ? launch_fwd_col<T, 128, 128>(a, ws, s) : launch_fwd_col<T, 128, 64>(a, ws, s);
     if (rc) return rc;
   }
-  if (phases & FMOBA_FWD_COMBINE)
-    hipLaunchKernelGGL(attn_fwd_combine_kernel<T>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, a, ws);
+  if (phases & FMOBA_FWD_COMBINE) {
+    const int capl = combine_order_entries(ws.cap);
+    const size_t smem = (size_t)16 * capl * 4;
+    auto kern = attn_fwd_combine_kernel<T>;
+    if (smem > 32 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+      set_error("attn_fwd: a row with up to %d visits needs %zu bytes of LDS for the order of its partial results", ws.cap, smem);
+      return 2;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 15) / 16)), dim3(256), smem, s, a, ws, capl);
+  }
   return 0;
 }
 

@@ -356,6 +356,32 @@ __device__ __forceinline__ int lower_bound_wave_i32(const int32_t *p, int n, int
   return lo;
 }
 
+// Order of the n partial results of one (row, head) for the 16-lane group of `lane`: ord[r] = slot of the partial
+// whose key-block id (ids[slot * stride]) has rank r in ascending order, equal ids ordered by slot.  n may differ
+// between the four groups of a wave, nmax is the largest of them (the shuffles need all lanes).  Brute force: every
+// lane ranks its slots li, li + 16, ... against all ids, 16 at a time through shuffles; a row of 32 visits costs 64
+// comparisons per lane.  Ends with the group's LDS writes visible to its lanes.
+__device__ __forceinline__ void group_rank_order(const int *ids, int stride, int n, int nmax, int *ord, int lane) {
+  const int li = lane & 15;
+  for (int j0 = 0; j0 < nmax; j0 += 16) {
+    const int j = j0 + li;
+    const int cj = j < n ? ids[(int64_t)j * stride] : 0x7fffffff;
+    int rank = 0;
+    for (int i0 = 0; i0 < nmax; i0 += 16) {
+      const int cmine = (j0 == i0) ? cj : (i0 + li < n ? ids[(int64_t)(i0 + li) * stride] : 0x7fffffff);
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        const int ci = __shfl(cmine, (lane & 48) | t, 64);
+        rank += (ci < cj || (ci == cj && i0 + t < j)) ? 1 : 0;
+      }
+    }
+    if (j < n) ord[rank] = j;
+  }
+  wave_lds_fence();
+}
+// entries of a group's order list for rows of up to `cap` visits
+static inline int combine_order_entries(int cap) { return ((cap > 0 ? cap : 1) + 15) / 16 * 16; }
+
 // f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}): a loop whose index is a
 // compile-time constant inside the body (register arrays, template arguments)
 template <typename F, int... I>

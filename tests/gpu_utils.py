@@ -46,11 +46,26 @@ def assert_close(name, got, ref, atol, rtol):
     assert not bad.any(), f"{name}: {int(bad.sum())} / {bad.numel()} elements out of tolerance, max err {err.max().item():.4e}"
 
 
-def dense_ref_one_head(q, k, v, dout, km, chunk, topk, row_block=2048):
+def csc_selection_one_head(co, cn, ind, b, h, L):
+    """(L, maxC) bool selection of one (sequence, head) read from a CSC triple on its device: the lists of a
+    (sequence, head) are consecutive (offsets = exclusive scan of the counts), so one slice holds them all."""
+    maxC = co.shape[2]
+    counts = cn[b, h].long()
+    start = int(co[b, h, 0])
+    rows = ind[start:start + int(counts.sum())].long()
+    cols = torch.repeat_interleave(torch.arange(maxC, device=co.device), counts)
+    sel = torch.zeros((L, maxC), dtype=torch.bool, device=co.device)
+    sel[rows, cols] = True
+    return sel
+
+
+def dense_ref_one_head(q, k, v, dout, km, chunk, topk, row_block=2048, sel_override=None):
     """fp32 dense-masked MoBA of ONE (sequence, head) evaluated with plain torch ops on the
     tensors' device (test reference for sizes the CPU oracle cannot finish in seconds).
     q, k, v, dout: (L, D); km: (C, D) chunk means in the storage dtype.  Returns out, dq, dk, dv
-    (fp32) and the boolean (L, C) selection."""
+    (fp32), the boolean (L, C) selection of its own fp32 gating and the gate values.  With
+    sel_override (L, >= C) the attention uses that selection instead of the re-gated one (the
+    re-gated selection and the gates are still returned)."""
     L, D = q.shape
     C = km.shape[0]
     dev = q.device
@@ -69,11 +84,12 @@ def dense_ref_one_head(q, k, v, dout, km, chunk, topk, row_block=2048):
     tv, ti = sv[:, C - kk:], si[:, C - kk:]
     sel = torch.zeros((L, C), dtype=torch.bool, device=dev)
     sel.scatter_(1, ti, tv > float("-inf"))
+    use = sel if sel_override is None else sel_override[:, :C]
     outs = []
     scale = D ** -0.5
     for r0 in range(0, L, row_block):
         r1 = min(L, r0 + row_block)
-        m = sel[r0:r1].repeat_interleave(chunk, dim=1)[:, :L] & (torch.arange(L, device=dev)[None] <= r[r0:r1, None])
+        m = use[r0:r1].repeat_interleave(chunk, dim=1)[:, :L] & (torch.arange(L, device=dev)[None] <= r[r0:r1, None])
         s = (qf[r0:r1] @ kf.T) * scale
         s = s.masked_fill(~m, float("-inf"))
         outs.append(torch.softmax(s, -1) @ vf)

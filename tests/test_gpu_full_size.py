@@ -4,14 +4,15 @@ The CPU oracle cannot evaluate 64K-token configurations in seconds, so these tes
   * structural invariants of the CSC triple that hold for ANY input (ascending lists, offsets =
     exclusive scan of the counts from the region base, closed-form number of kept chunks);
   * linearity of attention in V and of the backward in dO for a fixed pattern;
-  * a dense fp32 evaluation of sampled (sequence, head) pairs with plain torch ops on the GPU
-    (gating included), compared under the bf16 tolerance 2e-2 abs / 1e-2 rel.
+  * a dense fp32 evaluation of sampled (sequence, head) pairs with plain torch ops on the GPU over the
+    kernel's own pattern (out, dQ, dK, dV under the bf16 tolerance 2e-2 abs / 1e-2 rel, every element),
+    and that pattern against an fp32 re-gating wherever the selection is unambiguous.
 """
 import numpy as np
 import pytest
 import torch
 
-from gpu_utils import dense_ref_one_head
+from gpu_utils import csc_selection_one_head, dense_ref_one_head
 
 pytestmark = pytest.mark.gpu
 
@@ -61,8 +62,14 @@ def _check_csc(co, cn, ind, seqlens, H, chunk, topk):
     assert bool((ind[~used] == 0).all())
 
 
-def _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, samples, grads):
+def _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, samples, grads, csc):
+    """Sampled (sequence, head) pairs against a dense fp32 evaluation.  The dense mask is the kernel's OWN pattern
+    (`csc`, the triple the same gating call produces: the gating is deterministic), so every row is comparable and
+    out, dQ, dK and dV are asserted without exception; the pattern itself is compared with an fp32 re-gating on
+    every row whose selection is unambiguous (gap between the last kept and the first rejected score above 1e-3
+    relative)."""
     max_len = max(seqlens)
+    co, cn, ind = csc
     qg, kg, vg = (t.clone().requires_grad_(grads) for t in (q, k, v))
     out = api.flash_moba_varlen_func(qg, kg, vg, cu, cu, max_len, max_len, chunk, topk, causal=True)
     if grads:
@@ -71,30 +78,30 @@ def _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, sam
     cun = cu.cpu().numpy()
     for (b, h) in samples:
         s, e = int(cun[b]), int(cun[b + 1])
+        sel_kernel = csc_selection_one_head(co, cn, ind, b, h, e - s)
         o_ref, dq_ref, dk_ref, dv_ref, sel, gate = dense_ref_one_head(
-            q[s:e, h], k[s:e, h], v[s:e, h], dout[s:e, h], km[int(cu_km[b]):int(cu_km[b + 1]), h], chunk, topk)
-        # rows whose selection is unambiguous (gap between last kept and first rejected score > 1e-3 relative)
+            q[s:e, h], k[s:e, h], v[s:e, h], dout[s:e, h], km[int(cu_km[b]):int(cu_km[b + 1]), h], chunk, topk,
+            sel_override=sel_kernel)
         C = gate.shape[1]
+        assert not bool(sel_kernel[:, C:].any()), "a column past the sequence's last chunk has rows"
         ok = torch.ones(e - s, dtype=torch.bool, device=q.device)
         if C > topk:
             sv, _ = torch.sort(gate, dim=-1, descending=True)
             a_, b_ = sv[:, topk - 1], sv[:, topk]
             fin = torch.isfinite(a_) & torch.isfinite(b_)
             ok = ~(fin & ((a_ - b_).abs() <= 1e-3 * torch.maximum(a_.abs(), b_.abs())))
-        err = (out[s:e, h].float() - o_ref).abs()
-        bad = (err > 2e-2 + 1e-2 * o_ref.abs()).any(-1)
-        assert not bool((bad & ok).any()), f"out mismatch at (b={b}, h={h}): {int((bad & ok).sum())} rows"
-        if grads and bool(ok.all()):
-            for name, got, ref in (("dq", qg.grad[s:e, h], dq_ref), ("dk", kg.grad[s:e, h], dk_ref), ("dv", vg.grad[s:e, h], dv_ref)):
-                err = (got.float() - ref).abs()
-                frac = (err > 2e-2 + 1e-2 * ref.abs()).float().mean().item()
-                assert frac == 0.0, (name, b, h, frac, err.max().item())
-        elif grads:
-            # a flipped chunk changes a few rows; everything else must still agree
-            for name, got, ref in (("dq", qg.grad[s:e, h], dq_ref),):
-                err = (got.float() - ref).abs()
-                badr = (err > 2e-2 + 1e-2 * ref.abs()).any(-1)
-                assert not bool((badr & ok).any()), name
+        assert int(ok.sum()) > 0.9 * (e - s)
+        differs = (sel_kernel[:, :C] != sel).any(-1)
+        assert not bool((differs & ok).any()), f"selection differs from the fp32 gating at (b={b}, h={h}): {int((differs & ok).sum())} unambiguous rows"
+        # every row keeps min(topk, visible chunks) chunks, ambiguous or not
+        assert torch.equal(sel_kernel.sum(-1), sel.sum(-1))
+        named = [("out", out[s:e, h], o_ref)]
+        if grads:
+            named += [("dq", qg.grad[s:e, h], dq_ref), ("dk", kg.grad[s:e, h], dk_ref), ("dv", vg.grad[s:e, h], dv_ref)]
+        for name, got, ref in named:
+            err = (got.float() - ref).abs()
+            nbad = int((err > 2e-2 + 1e-2 * ref.abs()).sum())
+            assert nbad == 0, (name, b, h, nbad, err.max().item())
     return out
 
 
@@ -111,7 +118,7 @@ def test_config2_forward_8k(mods):
     q, k, v, dout, cu = _inputs(seqlens, H, D, chunk, 1002)
     co, cn, ind = api.flash_topk_varlen_func(q, k, cu, cu, 8192, 8192, topk, chunk, causal=True)
     _check_csc(co, cn, ind, seqlens, H, chunk, topk)
-    _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, [(0, 0), (0, 7), (0, 15)], grads=False)
+    _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, [(0, 0), (0, 7), (0, 15)], grads=False, csc=(co, cn, ind))
 
 
 def test_config3_fwd_bwd_32k(mods):
@@ -120,7 +127,7 @@ def test_config3_fwd_bwd_32k(mods):
     q, k, v, dout, cu = _inputs(seqlens, H, D, chunk, 1003)
     co, cn, ind = api.flash_topk_varlen_func(q, k, cu, cu, 32768, 32768, topk, chunk, causal=True)
     _check_csc(co, cn, ind, seqlens, H, chunk, topk)
-    _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, [(0, 5)], grads=True)
+    _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, [(0, 5)], grads=True, csc=(co, cn, ind))
 
 
 def test_config4_headline_fwd_bwd_64k(mods):
@@ -138,7 +145,7 @@ def test_config4_headline_fwd_bwd_64k(mods):
     assert torch.equal(co, co2) and torch.equal(cn, cn2) and torch.equal(ind, ind2)
     # the standalone sort is idempotent on the (already ascending) lists
     assert torch.equal(torch.ops.flash_moba._varlen_sort(co, cn, ind), ind)
-    out = _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, [(0, 3), (5, 12), (1, 0)], grads=True)
+    out = _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, [(0, 3), (5, 12), (1, 0)], grads=True, csc=(co, cn, ind))
     # linearity in V for a fixed pattern: attn(v1 + v2) = attn(v1) + attn(v2)
     v2 = torch.randn_like(v)
     lg = api.flash_moba_interface.decide_lg_block_m(topk, chunk, max_len, True)

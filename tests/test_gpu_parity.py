@@ -470,6 +470,35 @@ def test_backward_both_dq_forms(fm, dq_mode, d, chunk):
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
 
 
+@pytest.mark.parametrize("chunk,topk,visits", [(64, 40, 40), (128, 24, 24), (256, 10, 20)])
+def test_partial_forms_are_bitwise_repeatable_beyond_16_visits_per_row(fm, chunk, topk, visits):
+    # Column forward and partial-sum dQ hand out a row's partial slots from a counter, in whatever order the
+    # workgroups arrive; the merge must not depend on it: ranks are taken over ALL of a row's visits (here 20 to 40
+    # per row, more than one batch of 16), so repeated runs give the same bits, and both agree with the oracle.
+    lens = [chunk * 50 + 17, 900]
+    q, k, v, cu, dout = O.make_inputs(lens, 4, 128, chunk, 62, torch.bfloat16, with_dout=True)
+    Q, K, V, CU, DO = q.cuda(), k.cuda(), v.cuda(), cu.cuda(), dout.cuda()
+    co, cn, ind = fm.api.flash_topk_varlen_func(Q, K, CU, CU, max(lens), max(lens), topk, chunk, causal=True)
+    scale = 128 ** -0.5
+    runs = []
+    for _ in range(3):  # (no hints: the visit bounds are counted from the pattern)
+        out, lse, _, _ = fm.hip.moba_varlen_fwd(Q, K, V, None, co, cn, ind, CU, CU, None, None, None, max(lens), max(lens), 0.0, scale,
+                                                False, True, 0.0, False, 128, chunk, None, _fwd_mode=1)
+        assert fm.hip.last_fwd_row_blocks() == 0 and fm.hip.last_fwd_visits() == visits
+        dq, dk, dv, _ = fm.hip.moba_varlen_bwd(DO, Q, K, V, out, lse, None, None, None, co, cn, ind, CU, CU, None, max(lens), max(lens),
+                                               0.0, scale, False, True, 0.0, False, 128, chunk, None, None, _dq_mode=2)
+        assert fm.hip.last_bwd_partials() == 1
+        runs.append((out, lse, dq, dk, dv))
+    for other in runs[1:]:
+        for x, y in zip(runs[0], other):
+            assert torch.equal(x, y)
+    o_ref, _, dq_ref, dk_ref, dv_ref = O.attn_fwd_bwd(q, k, v, dout, cu, cu, co.cpu(), cn.cpu(), ind.cpu(), chunk, None, True)
+    assert_close("out", runs[0][0], o_ref, 2e-2, 1e-2)
+    assert_close("dq", runs[0][2], dq_ref, 2e-2, 1e-2)
+    assert_close("dk", runs[0][3], dk_ref, 2e-2, 1e-2)
+    assert_close("dv", runs[0][4], dv_ref, 2e-2, 1e-2)
+
+
 @pytest.mark.parametrize("chunk,topk", [(64, 4), (128, 3), (64, 32)])
 def test_attention_on_gated_pattern(fm, chunk, topk):
     lens = [640, 1, 0, 1300]
