@@ -213,9 +213,11 @@ def main():
 
     # ---- algorithmic work -------------------------------------------------------------
     with torch.no_grad():
-        hip.keep_next_gate_selection()  # as flash_moba_varlen_func does: the forward may use the gating's selection bits
-        co, cn, ind = flash_moba.flash_topk_varlen_func(q, k, cu, cu, max_len, max_len, topk, chunk, causal=True)
-        selection = hip.take_gate_selection()
+        # as flash_moba_varlen_func does: the forward may use the gating's selection bits
+        km0, cu_km0, _ = mean_pool_nosync(k.detach(), cu, max_len, chunk)
+        co, cn, ind, _, _, selection = hip.moba_fused_topk(q.detach(), km0, cu, cu, cu_km0, max_len, max_len, topk, chunk, True,
+                                                           return_raw=False, return_selection=True)
+        del km0
     pairs = count_pairs(seqlens, cn, chunk, H)
     fwd_flops = 4.0 * D * pairs
     bwd_flops = 2.5 * fwd_flops
@@ -236,9 +238,9 @@ def main():
     visits = topk * (chunk // hip.fwd_key_block(chunk))  # the bound the gated path hands to the forward
 
     def fwd(**kw):
-        hip.set_visits_hint(visits, selection=selection)
         return hip.moba_varlen_fwd(qd, kd, vd, None, co, cn, ind, cu, cu, None, None, None, max_len, max_len, 0.0, scale,
-                                   False, True, 0.0, False, lg_m, chunk, None, _fwd_mode=args.fwd_mode, **kw)
+                                   False, True, 0.0, False, lg_m, chunk, None, _fwd_mode=args.fwd_mode, _max_visits=visits,
+                                   _selection=selection, **kw)
 
     fwd_phase_ms = {}
     fwd()
@@ -277,9 +279,9 @@ def main():
         bwd_visits = visits * (hip.fwd_key_block(chunk) // 64)
 
         def bwd(**kw):
-            hip.set_bwd_visits_hint(bwd_visits)
             return hip.moba_varlen_bwd(dout, qd, kd, vd, out, lse, dq, dk, dv, co, cn, ind, cu, cu, None, max_len, max_len, 0.0,
-                                       scale, False, True, 0.0, False, lg_m, chunk, None, None, _dq_mode=args.dq_mode, **kw)
+                                       scale, False, True, 0.0, False, lg_m, chunk, None, None, _dq_mode=args.dq_mode,
+                                       _max_visits=bwd_visits, **kw)
 
         bwd(_phases=run_phases)
         t_bwd = time_events(bwd, it)

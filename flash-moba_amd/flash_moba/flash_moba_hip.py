@@ -186,11 +186,15 @@ def mean_pool(k: torch.Tensor, km: torch.Tensor, cu_seqlens_k: torch.Tensor, cu_
 # --------------------------------------------------------------------------------------
 def moba_fused_topk(q: torch.Tensor, km: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
                     cu_seqlens_km: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, moba_topk: int,
-                    moba_chunk_size: int, is_causal: bool, return_raw: bool = True) -> List[Optional[torch.Tensor]]:
+                    moba_chunk_size: int, is_causal: bool, return_raw: bool = True,
+                    return_selection: bool = False) -> List[Optional[torch.Tensor]]:
     """Returns [col_offsets, col_nnz, flat_indices, values, indices]
     (csrc/flash_topk/flash_topk_api.cpp:257).  `flat_indices` already holds each column's
     rows in ascending order.  With return_raw=False the ordered per-row lists are not
-    produced and the last two entries are None."""
+    produced and the last two entries are None.  With return_selection=True a sixth entry
+    follows: the same pattern as one bit per (row, head, chunk), int32 words of shape
+    (heads, ceil(max_cols / 32), total_q) -- the head of the call's workspace, which the
+    row-block forward can read instead of deriving the bits from the lists."""
     dtype = q.dtype
     _require(dtype in (torch.float16, torch.bfloat16), "FlashMoBA only supports fp16 and bf16 data types")
     _require(km.dtype == dtype, "q and km must have the same dtype")
@@ -233,11 +237,17 @@ def moba_fused_topk(q: torch.Tensor, km: torch.Tensor, cu_seqlens_q: torch.Tenso
                           int(moba_topk), int(moba_chunk_size), int(bool(is_causal)), _dt(q),
                           q.stride(0), q.stride(1), km.stride(0), km.stride(1))
         _check(lib.fmoba_fused_topk(ctypes.byref(a), _stream()))
-        if getattr(_hint, "keep_selection", False):
+        res = [col_offsets, col_nnz, flat, values, indices]
+        if return_selection:
             # the selection bits sit at the first 256-byte boundary of the workspace: (heads, ceil(max_cols/32), total_q) words
-            _hint.keep_selection = False
-            _hint.selection = (ws, heads, (max_cols + 31) // 32, total_q)
-    return [col_offsets, col_nnz, flat, values, indices]
+            words = (max_cols + 31) // 32
+            off = (-ws.data_ptr()) % 256
+            nbytes = heads * words * total_q * 4
+            if max_cols == 0 or max_seqlen_k == 0 or ws_bytes < off + nbytes:  # (no keys: nothing was written)
+                res.append(torch.zeros((heads, words, total_q), dtype=torch.int32, device=dev))
+            else:
+                res.append(ws[off:off + nbytes].view(torch.int32).view(heads, words, total_q))
+    return res
 
 
 # --------------------------------------------------------------------------------------
@@ -292,41 +302,29 @@ def _reject_unsupported(p_dropout, softcap, alibi_slopes, seqused_k=None, leftpa
     _require(not return_softmax, "return_softmax is only supported when p_dropout > 0.0, which FlashMoBA does not support")
 
 
-# A caller that knows how many (row, key block) visits a query row can have (the gated path: top-k times the
-# key blocks per chunk) leaves the bound here for the next forward call; otherwise it is computed from the
-# pattern, which costs one device-to-host read.
-_hint = threading.local()
-
-
-def set_visits_hint(n, selection=None):
-    """Bound (in forward key blocks) for the next forward call of this thread, and optionally the
-    selection bits of the gating call that produced its pattern (take_gate_selection())."""
-    _hint.value = None if n is None else int(n)
-    _hint.fwd_selection = selection
-
-
-def keep_next_gate_selection():
-    """The next gating call of this thread keeps its workspace, whose head is the selection as one bit
-    per (row, head, chunk); take_gate_selection() hands it over once."""
-    _hint.keep_selection = True
-    _hint.selection = None
-
-
-def take_gate_selection():
-    sel = getattr(_hint, "selection", None)
-    _hint.selection = None
-    _hint.keep_selection = False
-    return sel
-
-
-def set_bwd_visits_hint(n):
-    """Bound (in 64-key blocks) for the next backward call of this thread."""
-    _hint.bwd = None if n is None else int(n)
+# What the last forward / backward call of this thread ran.  Read-only diagnostics for tests and benchmarks: nothing
+# in here influences a later call (bounds and selection bits are explicit arguments).
+_last = threading.local()
 
 
 def last_fwd_visits():
-    """The bound the last forward call of this thread used, in forward key blocks."""
-    return getattr(_hint, "last", None)
+    """The visits bound the last forward call of this thread used, in forward key blocks."""
+    return getattr(_last, "fwd_visits", None)
+
+
+def last_fwd_row_blocks():
+    """1 if the last forward of this thread ran the row-block form, 0 for the column form."""
+    return int(getattr(_last, "fwd_row_blocks", 0))
+
+
+def last_bwd_partials():
+    """1 if the last backward of this thread formed dQ from per-visit partials, 0 for the row-block form."""
+    return int(getattr(_last, "bwd_partials", 0))
+
+
+def fwd_key_block(n_lg_block_dim: int) -> int:
+    """Keys per forward visit (fmoba_attn_fwd_key_block): 128 for columns of a multiple of 128 keys, else 64."""
+    return 128 if int(n_lg_block_dim) % 128 == 0 else 64
 
 
 def _count_visits(lib, q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k, batch, total_q, total_k,
@@ -344,25 +342,35 @@ def _count_visits(lib, q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_s
     return max(1, int(counts[total_q * heads].item()))
 
 
-def last_fwd_row_blocks():
-    """1 if the last forward of this thread ran the row-block form, 0 for the column form."""
-    return int(getattr(_hint, "last_form", 0))
-
-
-def last_bwd_partials():
-    """1 if the last backward of this thread formed dQ from per-visit partials, 0 for the row-block form."""
-    return int(getattr(_hint, "last_bwd_partials", 0))
-
-
-def fwd_key_block(n_lg_block_dim):
-    return int(load_library().fmoba_attn_fwd_key_block(int(n_lg_block_dim)))
+def count_max_visits(q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k, total_k, heads_k,
+                     max_seqlen_q, max_seqlen_k, n_lg_block_dim) -> int:
+    """Largest number of (row, forward key block) visits of any (row, head) of a CSC pattern: the bound the attention
+    entry points need for a pattern that does not come from the gating.  One pass over the lists + one device-to-host
+    read."""
+    _require(q.is_cuda and q.dim() == 3, "q must be a (total_q, heads, head_size) tensor on CUDA")
+    batch = cu_seqlens_q.numel() - 1
+    _require(batch > 0, "batch size must be positive")
+    _check_cu("cu_seqlens_q", cu_seqlens_q, batch)
+    _check_cu("cu_seqlens_k", cu_seqlens_k, batch)
+    total_q, heads, d = q.shape
+    _check_csc(moba_col_offsets, moba_col_nnz, moba_row_indices, batch, heads)
+    _require(n_lg_block_dim % 64 == 0 and n_lg_block_dim > 0, "n_lg_block_dim must be a multiple of 64")
+    with _device_guard(q):
+        return _count_visits(load_library(), q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k,
+                             batch, total_q, int(total_k), heads, heads_k, d, max_seqlen_q, max_seqlen_k,
+                             moba_col_offsets.shape[2], 128, n_lg_block_dim)
 
 
 def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k,
                     seqused_k, leftpad_k, alibi_slopes, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                     zero_tensors, is_causal, softcap, return_softmax, m_lg_block_dim, n_lg_block_dim, gen=None, _phases=None,
-                    _fwd_mode=0):
-    """Returns [out, softmax_lse (H, total_q) fp32, p (empty), rng_state (2,) int64]."""
+                    _fwd_mode=0, _max_visits=None, _selection=None):
+    """Returns [out, softmax_lse (H, total_q) fp32, p (empty), rng_state (2,) int64].
+
+    Beyond the reference's arguments: _max_visits, a bound on the (row, forward key block) visits of any (row, head)
+    -- a gated pattern has top-k * lg_block_n / fwd_key_block(lg_block_n); None or a value below 1 makes the call count
+    them from the pattern (one device-to-host read) -- and _selection, the int32 selection words of the gating call that
+    produced exactly this pattern (moba_fused_topk(return_selection=True))."""
     dtype = q.dtype
     _require(dtype in (torch.float16, torch.bfloat16), "FlashMoBA only support fp16 and bf16 data type")
     _require(k.dtype == dtype, "query and key must have the same dtype")
@@ -402,13 +410,12 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
         p = torch.empty((0,), dtype=dtype, device=q.device)
         rng_state = torch.zeros((2,), dtype=torch.int64, device=q.device)
         lib = load_library()
-        hint = getattr(_hint, "value", None)
-        _hint.value = None
-        sel = getattr(_hint, "fwd_selection", None)
-        _hint.fwd_selection = None
         sel_ptr = None
-        if sel is not None and sel[1:] == (heads, (max_cols + 31) // 32, total_q) and sel[0].device == q.device:
-            sel_ptr = (sel[0].data_ptr() + 255) & ~255
+        if _selection is not None and max_cols > 0 and total_q > 0:
+            _require(_selection.dtype == torch.int32 and _selection.is_cuda and _selection.device == q.device and _selection.is_contiguous()
+                     and tuple(_selection.shape) == (heads, (max_cols + 31) // 32, total_q),
+                     "selection bits must be a contiguous int32 tensor of shape (num_heads, ceil(max_lg_col_num / 32), total_q) on q's device")
+            sel_ptr = _selection.data_ptr()
 
         def args(ws_ptr, ws_bytes, visits):
             return AttnFwdArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
@@ -420,16 +427,16 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
                                q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                                out.stride(0), out.stride(1))
 
-        visits = hint
-        if visits is None:
+        visits = _max_visits
+        if visits is None or int(visits) < 1:
             visits = _count_visits(lib, q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k, batch,
                                    total_q, total_k, heads, heads_k, d, max_seqlen_q, max_seqlen_k, max_cols,
                                    m_lg_block_dim, n_lg_block_dim)
         visits = max(1, int(visits))
-        _hint.last = visits
+        _last.fwd_visits = visits
         a = args(None, 0, visits)
         ws_bytes = lib.fmoba_attn_fwd_workspace_bytes(ctypes.byref(a))
-        _hint.last_form = int(lib.fmoba_attn_fwd_uses_row_blocks(ctypes.byref(a)))
+        _last.fwd_row_blocks = int(lib.fmoba_attn_fwd_uses_row_blocks(ctypes.byref(a)))
         ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=q.device)
         a = args(ws.data_ptr(), ws_bytes, visits)
         if _phases is None:
@@ -445,8 +452,12 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
 def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_offsets, moba_col_nnz, moba_row_indices,
                     cu_seqlens_q, cu_seqlens_k, alibi_slopes, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                     zero_tensors, is_causal, softcap, deterministic, m_lg_block_dim, n_lg_block_dim, gen=None,
-                    rng_state=None, _phases=None, _dq_mode=0):
-    """Returns [dq, dk, dv, softmax_d (H, total_q + 128*batch) fp32]."""
+                    rng_state=None, _phases=None, _dq_mode=0, _max_visits=None):
+    """Returns [dq, dk, dv, softmax_d (H, total_q + 128*batch) fp32].
+
+    Beyond the reference's arguments: _max_visits, a bound on the visits of any (row, head) in 64-KEY blocks (a gated
+    pattern has top-k * lg_block_n / 64); None or a value below 1 makes the call count them from the pattern (one
+    device-to-host read)."""
     dtype = q.dtype
     _require(dtype in (torch.float16, torch.bfloat16), "FlashMoBA only support fp16 and bf16 data type")
     _require(k.dtype == dtype, "query and key must have the same dtype")
@@ -501,10 +512,9 @@ def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_off
         else:
             dk_e, dv_e = dk, dv
         lib = load_library()
-        visits = getattr(_hint, "bwd", None)
-        _hint.bwd = None
-        if visits is None:
-            kb = int(lib.fmoba_attn_fwd_key_block(int(n_lg_block_dim)))
+        visits = _max_visits
+        if visits is None or int(visits) < 1:
+            kb = fwd_key_block(n_lg_block_dim)
             visits = (kb // 64) * _count_visits(lib, q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q,
                                                 cu_seqlens_k, batch, total_q, total_k, heads, heads_k, d, max_seqlen_q,
                                                 max_seqlen_k, max_cols, 128, n_lg_block_dim)
@@ -520,7 +530,7 @@ def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_off
                         out.stride(0), out.stride(1), dout.stride(0), dout.stride(1),
                         dq.stride(0), dq.stride(1), dk_e.stride(0), dk_e.stride(1), dv_e.stride(0), dv_e.stride(1))
         ws_bytes = lib.fmoba_attn_bwd_workspace_bytes(ctypes.byref(a))
-        _hint.last_bwd_partials = int(lib.fmoba_attn_bwd_uses_partials(ctypes.byref(a)))
+        _last.bwd_partials = int(lib.fmoba_attn_bwd_uses_partials(ctypes.byref(a)))
         ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
         a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
         if _phases is None:

@@ -195,59 +195,207 @@ def _flash_moba_attn_varlen_backward_fake(dout, q, k, v, out, softmax_lse, dq, d
     return torch.empty((heads, total_q + 128 * batch), device=q.device, dtype=torch.float32)
 
 
+# --------------------------------------------------------------------------------------
+# private ops of the fused path.  The reference's four ops above keep their schemas; these carry, as ordinary
+# arguments, what the MI355X kernels need beyond them -- the bound on a row's (row, key block) visits, which sizes
+# the partial-result workspace and selects the kernel form, and the gating's selection bits -- so that a traced or
+# compiled graph carries them too (the reference has no counterpart: its row-wise scratch needs no bound).
+# --------------------------------------------------------------------------------------
+@torch.library.custom_op("flash_moba::_mean_pool", mutates_args=(), device_types="cuda")
+def _mean_pool(k: torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_k: int, chunk: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    km, cu_km, _ = mean_pool_nosync(k, cu_seqlens_k, max_seqlen_k, chunk)
+    return km, cu_km
+
+
+@torch.library.register_fake("flash_moba::_mean_pool")
+def _mean_pool_fake(k, cu_seqlens_k, max_seqlen_k, chunk):
+    batch = cu_seqlens_k.numel() - 1
+    return (torch.empty((k.shape[0] // chunk + batch, k.shape[1], k.shape[2]), dtype=k.dtype, device=k.device),
+            torch.empty(cu_seqlens_k.shape, dtype=torch.int32, device=k.device))
+
+
+@torch.library.custom_op("flash_moba::_gated_topk", mutates_args=(), device_types="cuda")
+def _gated_topk(
+    q: torch.Tensor,
+    km: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    cu_seqlens_k: torch.Tensor,
+    cu_seqlens_km: torch.Tensor,
+    max_seqlen_q: int,
+    max_seqlen_k: int,
+    moba_topk: int,
+    moba_chunk_size: int,
+    causal: bool,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """_moba_fused_topk plus the selection as one bit per (row, head, chunk): int32 (heads, ceil(cols/32), total_q)."""
+    q, km = maybe_contiguous(q), maybe_contiguous(km)
+    col_offsets, col_nnz, indices, _, _, selection = flash_moba_gpu.moba_fused_topk(
+        q, km, cu_seqlens_q, cu_seqlens_k, cu_seqlens_km, max_seqlen_q, max_seqlen_k,
+        moba_topk, moba_chunk_size, causal, return_raw=False, return_selection=True)
+    return col_offsets, col_nnz, indices, selection
+
+
+@torch.library.register_fake("flash_moba::_gated_topk")
+def _gated_topk_fake(q, km, cu_seqlens_q, cu_seqlens_k, cu_seqlens_km, max_seqlen_q, max_seqlen_k,
+                     moba_topk, moba_chunk_size, causal):
+    co, cn, ind = _moba_fused_topk_fake(q, km, cu_seqlens_q, cu_seqlens_k, cu_seqlens_km, max_seqlen_q, max_seqlen_k,
+                                        moba_topk, moba_chunk_size, causal)
+    total_q, heads, _ = q.shape
+    return co, cn, ind, torch.empty((heads, (co.shape[2] + 31) // 32, total_q), device=q.device, dtype=torch.int32)
+
+
+@torch.library.custom_op("flash_moba::_attn_varlen_forward_bounded", mutates_args=(), device_types="cuda")
+def _attn_varlen_forward_bounded(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    cu_seqlens_k: torch.Tensor,
+    max_seqlen_q: int,
+    max_seqlen_k: int,
+    moba_col_offsets: torch.Tensor,
+    moba_col_nnz: torch.Tensor,
+    moba_row_indices: torch.Tensor,
+    lg_block_m: int,
+    lg_block_n: int,
+    softmax_scale: float,
+    causal: bool,
+    max_visits: int,
+    selection_bits: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """_flash_moba_attn_varlen_forward with the visits bound (in forward key blocks; below 1 = count them from the
+    pattern) and, optionally, the gating's selection bits as arguments."""
+    q, k, v = (maybe_contiguous(x) for x in (q, k, v))
+    csc = [maybe_contiguous(x) for x in (moba_col_offsets, moba_col_nnz, moba_row_indices)]
+    out, softmax_lse, S_dmask, rng_state = flash_moba_gpu.moba_varlen_fwd(
+        q, k, v, None, csc[0], csc[1], csc[2], cu_seqlens_q, cu_seqlens_k, None, None, None,
+        max_seqlen_q, max_seqlen_k, 0.0, softmax_scale, False, causal, 0.0, False,
+        lg_block_m, lg_block_n, None, _max_visits=max_visits, _selection=selection_bits)
+    return out, softmax_lse, S_dmask, rng_state
+
+
+@torch.library.register_fake("flash_moba::_attn_varlen_forward_bounded")
+def _attn_varlen_forward_bounded_fake(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                      moba_col_offsets, moba_col_nnz, moba_row_indices, lg_block_m, lg_block_n,
+                                      softmax_scale, causal, max_visits, selection_bits=None):
+    return _flash_moba_attn_varlen_forward_fake(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                                moba_col_offsets, moba_col_nnz, moba_row_indices, lg_block_m, lg_block_n,
+                                                0.0, softmax_scale, causal)
+
+
+@torch.library.custom_op("flash_moba::_attn_varlen_backward_bounded", mutates_args=("dq", "dk", "dv"), device_types="cuda")
+def _attn_varlen_backward_bounded(
+    dout: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    softmax_lse: torch.Tensor,
+    dq: torch.Tensor,
+    dk: torch.Tensor,
+    dv: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    cu_seqlens_k: torch.Tensor,
+    max_seqlen_q: int,
+    max_seqlen_k: int,
+    moba_col_offsets: torch.Tensor,
+    moba_col_nnz: torch.Tensor,
+    moba_row_indices: torch.Tensor,
+    lg_block_m: int,
+    lg_block_n: int,
+    softmax_scale: float,
+    causal: bool,
+    deterministic: bool,
+    max_visits: int,
+) -> torch.Tensor:
+    """_flash_moba_attn_varlen_backward with the visits bound (in 64-key blocks; below 1 = count them) as an argument."""
+    dout, q, k, v, out = (maybe_contiguous(x) for x in (dout, q, k, v, out))
+    _, _, _, softmax_d = flash_moba_gpu.moba_varlen_bwd(
+        dout, q, k, v, out, softmax_lse, dq, dk, dv, moba_col_offsets, moba_col_nnz, moba_row_indices,
+        cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q, max_seqlen_k, 0.0, softmax_scale,
+        False, causal, 0.0, deterministic, lg_block_m, lg_block_n, None, None, _max_visits=max_visits)
+    return softmax_d
+
+
+@torch.library.register_fake("flash_moba::_attn_varlen_backward_bounded")
+def _attn_varlen_backward_bounded_fake(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
+                                       max_seqlen_q, max_seqlen_k, moba_col_offsets, moba_col_nnz, moba_row_indices,
+                                       lg_block_m, lg_block_n, softmax_scale, causal, deterministic, max_visits):
+    batch = cu_seqlens_q.numel() - 1
+    total_q, heads, _ = q.shape
+    return torch.empty((heads, total_q + 128 * batch), device=q.device, dtype=torch.float32)
+
+
 _wrapped_moba_fused_topk = torch.ops.flash_moba._moba_fused_topk
 _wrapped_varlen_sort = torch.ops.flash_moba._varlen_sort
 _wrapped_flash_moba_attn_varlen_forward = torch.ops.flash_moba._flash_moba_attn_varlen_forward
 _wrapped_flash_moba_attn_varlen_backward = torch.ops.flash_moba._flash_moba_attn_varlen_backward
+_wrapped_mean_pool = torch.ops.flash_moba._mean_pool
+_wrapped_gated_topk = torch.ops.flash_moba._gated_topk
+_wrapped_attn_varlen_forward_bounded = torch.ops.flash_moba._attn_varlen_forward_bounded
+_wrapped_attn_varlen_backward_bounded = torch.ops.flash_moba._attn_varlen_backward_bounded
+
+
+def _fwd_key_block(lg_block_n: int) -> int:
+    """Keys per visit of the forward's column form (fmoba_attn_fwd_key_block of the library, as plain arithmetic so
+    that a traced graph can fold it)."""
+    return 128 if lg_block_n % 128 == 0 else 64
 
 
 # --------------------------------------------------------------------------------------
 # autograd
 # --------------------------------------------------------------------------------------
 class FlashMobaAttnVarlenFunc(torch.autograd.Function):
-    """Forward/backward over a given CSC pattern (flash_moba_interface.py:400-513)."""
+    """Forward/backward over a given CSC pattern (flash_moba_interface.py:400-513).
+
+    Two trailing arguments beyond the reference's twenty, both optional: max_visits, the bound on a row's visits in
+    forward key blocks when the caller knows it (a gated pattern: top-k * lg_block_n / key block), and the gating's
+    selection bits.  Without a bound it is counted from the pattern once, here (eager mode; one device-to-host read)
+    or inside each op (while a graph is being traced, where a data-dependent integer cannot leave an op)."""
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                 moba_col_offsets, moba_col_nnz, moba_row_indices, lg_block_m, lg_block_n,
                 dropout_p, softmax_scale, causal, softcap, alibi_slopes, deterministic,
-                return_softmax, is_grad_enabled):
+                return_softmax, is_grad_enabled, max_visits=None, selection_bits=None):
         needs_grad = is_grad_enabled and any(x.requires_grad for x in (q, k, v))
         if softmax_scale is None:
             softmax_scale = q.shape[-1] ** (-0.5)
+        flash_moba_gpu._reject_unsupported(dropout_p, softcap, alibi_slopes, None, None, return_softmax and dropout_p > 0)
         head_size_og = q.size(2)
         q, k, v = _pad8(q, k, v)
-        out_padded, softmax_lse, S_dmask, rng_state = _wrapped_flash_moba_attn_varlen_forward(
+        if max_visits is None:
+            if torch.compiler.is_compiling() or lg_block_n <= 0 or lg_block_n % 64 != 0:
+                max_visits = -1  # counted inside the ops (a malformed lg_block_n is reported there)
+            else:
+                max_visits = flash_moba_gpu.count_max_visits(
+                    q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k, k.shape[0], k.shape[1],
+                    max_seqlen_q, max_seqlen_k, lg_block_n)
+        out_padded, softmax_lse, S_dmask, rng_state = _wrapped_attn_varlen_forward_bounded(
             q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
             moba_col_offsets, moba_col_nnz, moba_row_indices, lg_block_m, lg_block_n,
-            dropout_p, softmax_scale, causal=causal, softcap=softcap, alibi_slopes=alibi_slopes,
-            return_softmax=return_softmax and dropout_p > 0)
+            softmax_scale, causal, max_visits, selection_bits)
         if needs_grad:
-            # visits bound the forward worked with, converted to the backward's 64-key blocks
-            fwd_visits = flash_moba_gpu.last_fwd_visits()
-            ctx.bwd_visits = None if fwd_visits is None else fwd_visits * (flash_moba_gpu.fwd_key_block(lg_block_n) // 64)
-            ctx.save_for_backward(q, k, v, out_padded, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state,
+            # the same bound in the backward's 64-key blocks
+            ctx.bwd_visits = max_visits * (_fwd_key_block(lg_block_n) // 64) if max_visits > 0 else -1
+            ctx.save_for_backward(q, k, v, out_padded, softmax_lse, cu_seqlens_q, cu_seqlens_k,
                                   moba_col_offsets, moba_col_nnz, moba_row_indices)
-            ctx.cfg = (max_seqlen_q, max_seqlen_k, lg_block_m, lg_block_n, dropout_p, softmax_scale, causal,
-                       softcap, alibi_slopes, deterministic)
+            ctx.cfg = (max_seqlen_q, max_seqlen_k, lg_block_m, lg_block_n, softmax_scale, causal, deterministic)
         out = out_padded[..., :head_size_og]
         return out if not return_softmax else (out, softmax_lse, S_dmask)
 
     @staticmethod
     def backward(ctx, dout, *args):
-        (q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state,
-         col_offsets, col_nnz, row_indices) = ctx.saved_tensors
-        (max_seqlen_q, max_seqlen_k, lg_block_m, lg_block_n, dropout_p, softmax_scale, causal,
-         softcap, alibi_slopes, deterministic) = ctx.cfg
+        (q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, col_offsets, col_nnz, row_indices) = ctx.saved_tensors
+        (max_seqlen_q, max_seqlen_k, lg_block_m, lg_block_n, softmax_scale, causal, deterministic) = ctx.cfg
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         (dout_padded,) = _pad8(dout)
-        flash_moba_gpu.set_bwd_visits_hint(ctx.bwd_visits)
-        _wrapped_flash_moba_attn_varlen_backward(
+        _wrapped_attn_varlen_backward_bounded(
             dout_padded, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
             max_seqlen_q, max_seqlen_k, col_offsets, col_nnz, row_indices, lg_block_m, lg_block_n,
-            dropout_p, softmax_scale, causal, softcap, alibi_slopes, deterministic, rng_state=rng_state)
+            softmax_scale, causal, deterministic, ctx.bwd_visits)
         d = dout.shape[-1]  # the head dimension may have been padded
-        return (dq[..., :d], dk[..., :d], dv[..., :d]) + (None,) * 17
+        return (dq[..., :d], dk[..., :d], dv[..., :d]) + (None,) * 19
 
 
 # --------------------------------------------------------------------------------------
@@ -269,7 +417,7 @@ def flash_topk_varlen_func(q, k, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_s
     int32, indices: (total_q * num_heads * moba_topk,) int32.
     """
     q, k = _pad8(q, k)
-    km, cu_seqlens_km, _ = mean_pool_nosync(k, cu_seqlens_k, max_seqlen_k, moba_chunk_size)
+    km, cu_seqlens_km = _wrapped_mean_pool(maybe_contiguous(k), cu_seqlens_k, max_seqlen_k, moba_chunk_size)
     # The row lists come back ascending, so the reference's second step
     # (_wrapped_varlen_sort, flash_moba_interface.py:570-572) has nothing left to do.
     return _wrapped_moba_fused_topk(q, km, cu_seqlens_q, cu_seqlens_k, cu_seqlens_km,
@@ -306,19 +454,17 @@ def flash_moba_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_
 def flash_moba_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                            moba_chunk_size, moba_topk, causal=True):
     """MoBA attention end to end: gate (mean-pool + top-k + CSC), then sparse attention."""
-    flash_moba_gpu.keep_next_gate_selection()
-    try:
-        col_offsets, col_nnz, indices = flash_topk_varlen_func(
-            q, k, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-            moba_topk, moba_chunk_size, causal=causal)
-    finally:
-        selection = flash_moba_gpu.take_gate_selection()
+    qp, kp = _pad8(q, k)
+    km, cu_seqlens_km = _wrapped_mean_pool(maybe_contiguous(kp), cu_seqlens_k, max_seqlen_k, moba_chunk_size)
+    col_offsets, col_nnz, indices, selection = _wrapped_gated_topk(
+        qp, km, cu_seqlens_q, cu_seqlens_k, cu_seqlens_km, max_seqlen_q, max_seqlen_k, moba_topk, moba_chunk_size, causal)
     lg_block_m = decide_lg_block_m(moba_topk, moba_chunk_size, max_seqlen_k, causal)
-    if moba_chunk_size % 64 == 0:
+    max_visits = None
+    if moba_chunk_size > 0 and moba_chunk_size % 64 == 0:
         # a gated row visits at most top-k chunks: the forward needs no pass over the pattern to size its scratch,
         # and the gating's own selection bits spare its row-block form the pass that derives them from the lists
-        flash_moba_gpu.set_visits_hint(moba_topk * (moba_chunk_size // flash_moba_gpu.fwd_key_block(moba_chunk_size)),
-                                       selection=selection)
-    return flash_moba_attn_varlen_func(
+        max_visits = moba_topk * (moba_chunk_size // _fwd_key_block(moba_chunk_size))
+    return FlashMobaAttnVarlenFunc.apply(
         q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-        col_offsets, col_nnz, indices, lg_block_m, moba_chunk_size, dropout_p=0.0, causal=causal)
+        col_offsets, col_nnz, indices, lg_block_m, moba_chunk_size,
+        0.0, None, causal, 0.0, None, False, False, torch.is_grad_enabled(), max_visits, selection)

@@ -166,3 +166,39 @@ def test_fake_shape_functions():
         sd = torch.ops.flash_moba._flash_moba_attn_varlen_backward(
             q, q, q, q, out, lse, None, None, None, cu, cu, 60, 60, co, cn, ind, 128, 64, 0.0, 0.125, True, 0.0, None, False)
         assert sd.shape == (4, 100 + 128 * 2)
+        # the private ops of the fused path: the visits bound and the selection bits are ordinary arguments
+        km2, cu_km = torch.ops.flash_moba._mean_pool(q, cu, 60, 16)
+        assert km2.shape == (100 // 16 + 2, 4, 64) and cu_km.dtype == torch.int32 and cu_km.shape == cu.shape
+        co, cn, ind, sel = torch.ops.flash_moba._gated_topk(q, km, cu, cu, cu, 60, 60, 3, 16, True)
+        assert sel.shape == (4, 1, 100) and sel.dtype == torch.int32 and ind.shape == (100 * 4 * 3,)
+        out, lse, p, rng = torch.ops.flash_moba._attn_varlen_forward_bounded(
+            q, q, q, cu, cu, 60, 60, co, cn, ind, 128, 64, 0.125, True, 3, sel)
+        assert out.shape == q.shape and lse.shape == (4, 100) and p.shape == (0,) and rng.shape == (2,)
+        dq = torch.empty_like(q)
+        sd = torch.ops.flash_moba._attn_varlen_backward_bounded(
+            q, q, q, q, out, lse, dq, dq, dq, cu, cu, 60, 60, co, cn, ind, 128, 64, 0.125, True, False, 3)
+        assert sd.shape == (4, 100 + 128 * 2)
+
+
+def test_fused_path_traces_end_to_end_on_fake_tensors():
+    # flash_moba_varlen_func touches the GPU only through custom ops with fake-shape functions: on fake tensors the
+    # whole forward runs without a device and without any state outside the op arguments
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    import flash_moba
+
+    with FakeTensorMode():
+        q, k, v = (torch.empty(700, 4, 72, dtype=torch.bfloat16, device="cuda", requires_grad=True) for _ in range(3))
+        cu = torch.empty(3, dtype=torch.int32, device="cuda")
+        out = flash_moba.flash_moba_varlen_func(q, k, v, cu, cu, 400, 400, 64, 3, causal=True)
+        assert out.shape == q.shape and out.dtype == q.dtype
+        assert out.grad_fn is not None  # (running the backward needs the autograd engine's device thread: GPU test)
+
+
+def test_key_block_rule_of_the_host_code_matches_the_library():
+    from flash_moba import flash_moba_interface as I
+
+    lib = H.load_library()
+    for n in (64, 128, 192, 256, 320, 1024):
+        assert I._fwd_key_block(n) == H.fwd_key_block(n) == lib.fmoba_attn_fwd_key_block(n)
+
