@@ -155,40 +155,14 @@ def cpu_baseline(q, k, v, cu, seqlens, chunk, topk, budget_s=12.0):
     }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="headline", choices=sorted(CONFIGS))
-    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--dq-mode", type=int, default=0, choices=(0, 1, 2),
-                    help="dQ form of the per-stage timings: 0 = the library's choice (what the timed steps run), 1 = row blocks, 2 = partials")
-    ap.add_argument("--fwd-mode", type=int, default=0, choices=(0, 1, 2),
-                    help="forward form of the per-stage timings: 0 = the library's choice (what the timed steps run), 1 = columns, 2 = row blocks")
-    ap.add_argument("--calib-copy", action="store_true",
-                    help="run one plain 1 GiB device copy first, so that a counter run has a kernel of known traffic to scale by")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(2)
-
+def run_config(name, steps, warmup, args, dev, cpu_budget_s):
+    """Measures one configuration: K timed steps, then per-stage and per-kernel timings, the roofline object of its
+    dominant kernel and (cpu_budget_s > 0) the CPU leg on a bounded sample of the same inputs."""
     import flash_moba
     from flash_moba import flash_moba_hip as hip
     from flash_moba.mean_pool import mean_pool_nosync
 
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    if args.calib_copy:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
-    seqlens, H, D, chunk, topk, backward = CONFIGS[args.config]
+    seqlens, H, D, chunk, topk, backward = CONFIGS[name]
     if seqlens is None:
         seqlens = headline_seqlens()
     T, nb, max_len = sum(seqlens), len(seqlens), max(seqlens)
@@ -202,14 +176,14 @@ def main():
             out.backward(dout)
         return out
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
 
     # ---- algorithmic work -------------------------------------------------------------
     with torch.no_grad():
@@ -228,7 +202,7 @@ def main():
     gate_bytes = T * H * D * 2 + sumC * H * D * 2 + T * H * topk * 4 + nb * H * maxC * 12
 
     # ---- per-stage times (events on the launch stream) ----------------------------------
-    it = max(5, args.steps)
+    it = max(3, min(steps, 20))
     lg_m = flash_moba.flash_moba_interface.decide_lg_block_m(topk, chunk, max_len, True)
     scale = D ** -0.5
     qd, kd, vd = q.detach(), k.detach(), v.detach()
@@ -301,7 +275,7 @@ def main():
     dom = max(kernels, key=lambda n: kernels[n][0])
     d_ms, d_flops, _ = kernels[dom]
     roofline = {"kernel": dom, "bound": "mfma", "achieved": d_flops / d_ms / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
+                "frac": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get((name, dom)),
                 "traffic_unit": "bytes/launch", "avg_launch_ms": d_ms,
                 "flops_per_launch": d_flops}
 
@@ -310,15 +284,15 @@ def main():
         "value": step_flops / ms_per_step / 1e9,
         "unit": "TFLOP/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": f"{args.config}: varlen packed batch, {nb} sequences totalling {T} tokens "
+        "config": {"workload": f"{name}: varlen packed batch, {nb} sequences totalling {T} tokens "
                                f"(lengths {seqlens}), causal, {H} heads, head_dim {D}, chunk {chunk}, top-k {topk}, "
                                + ("fwd+bwd" if backward else "fwd only"),
                    "tokens": T, "heads": H, "head_dim": D, "chunk": chunk, "topk": topk},
@@ -329,8 +303,55 @@ def main():
         "stages": stages,
         "roofline": roofline,
     }
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(qd, kd, vd, cu, seqlens, chunk, topk)
+    if cpu_budget_s > 0:
+        result["cpu_baseline"] = cpu_baseline(qd, kd, vd, cu, seqlens, chunk, topk, budget_s=cpu_budget_s)
+    return result
+
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="headline", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline legs")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="headline run only: skip the `configs` array (the other BASELINE configs, measured after the headline)")
+    ap.add_argument("--dq-mode", type=int, default=0, choices=(0, 1, 2),
+                    help="dQ form of the per-stage timings: 0 = the library's choice (what the timed steps run), 1 = row blocks, 2 = partials")
+    ap.add_argument("--fwd-mode", type=int, default=0, choices=(0, 1, 2),
+                    help="forward form of the per-stage timings: 0 = the library's choice (what the timed steps run), 1 = columns, 2 = row blocks")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="run one plain 1 GiB device copy first, so that a counter run has a kernel of known traffic to scale by")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.calib_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+    result = run_config(args.config, args.steps, args.warmup, args, dev, 0.0 if args.no_cpu else 12.0)
+    if args.config == "headline" and not args.no_configs:
+        # every other BASELINE config that runs on the GPU, a few steps each, same measurements
+        result["configs"] = []
+        for name, k_steps in (("c2", 20), ("c3", 10), ("c5", 3)):
+            torch.cuda.empty_cache()
+            r = run_config(name, k_steps, 2, args, dev, 0.0 if args.no_cpu else 4.0)
+            keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "frac_of_bf16_mfma_peak", "pairs", "flops_per_step",
+                    "topk_csc_ms", "stages", "roofline", "cpu_baseline")
+            entry = {"name": name, "workload": r["config"]["workload"]}
+            entry.update({k: r[k] for k in keep if k in r})
+            result["configs"].append(entry)
     print(json.dumps(result))
 
 
