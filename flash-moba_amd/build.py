@@ -17,7 +17,7 @@ LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libflash_moba_hip.so")
 SOURCES = ["fmoba_host.hip", "mean_pool.hip", "topk_csc.hip", "varlen_sort.hip", "attn_fwd.hip", "attn_fwd_rows.hip", "attn_bwd.hip"]
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # keep packed-fp32 VALU ops out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",

@@ -276,12 +276,17 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
 // running winners after the last group are exactly the global top-K'.  Selection words
 // and counts are then assembled in LDS and written out like the small kernel's.
 // ------------------------------------------------------------------------------------
-constexpr int kBigCap = 32;  // running winners per row (K' = scored chunks kept)
+constexpr int kBigCap = 32;   // running winners per row (K' = scored chunks kept) of the common variants
+constexpr int kBigCapMax = 64;  // ... of the variant for top-k above 33: moba_topk goes up to 64 at any sequence length
 
-// CAP: entries of a row's list of running winners (16 or kBigCap).  With 16 and groups of 128 chunks the kernel needs
-// half the LDS and fewer registers, and two workgroups share a compute unit.
+// CAP: entries of a row's list of running winners (16, kBigCap or kBigCapMax).  With 16 and groups of 128 chunks the
+// kernel needs half the LDS and fewer registers, and two workgroups share a compute unit.  With 64 a row has ONE list
+// (two would not fit the LDS): every group then takes the general path, which has read the whole list into registers
+// before it writes the winners back; the streaming update of the smaller variants needs the second list for its entrants.
 template <typename T, int HD, int NT, int CAP>
 __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kernel(TopkParams p) {
+  constexpr bool TWO_LISTS = CAP <= kBigCap;
+  constexpr int NLIST = TWO_LISTS ? 2 : 1;
   constexpr int KS = HD / 16;
   constexpr int LD = HD + 16;
   constexpr int GC = NT * 32;        // chunks per group
@@ -289,9 +294,9 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint16_t *sKm = reinterpret_cast<uint16_t *>(smem);
   uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [W][128], reuses the chunk-mean tile after the last group
-  float *sVal = reinterpret_cast<float *>(smem + (size_t)GC * LD * 2);   // [2][128][CAP]
-  int *sIdx = reinterpret_cast<int *>(sVal + 2 * kGateRows * CAP);   // [2][128][CAP]
-  int *sCnt = sIdx + 2 * kGateRows * CAP;                            // [2][128]
+  float *sVal = reinterpret_cast<float *>(smem + (size_t)GC * LD * 2);   // [NLIST][128][CAP]
+  int *sIdx = reinterpret_cast<int *>(sVal + NLIST * kGateRows * CAP);   // [NLIST][128][CAP]
+  int *sCnt = sIdx + NLIST * kGateRows * CAP;                            // [2][128]
   int *sHist = sCnt + 2 * kGateRows;                                     // [max_cols]
   int *sTrash = sHist + p.max_cols;                                      // [256]: takes the stores of lanes that have nothing to store
 
@@ -371,8 +376,8 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
     for (int j = 0; j < PL; ++j) {
       const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
       const bool ok = e < m_prev;
-      pv[j] = ok ? sVal[(cur * kGateRows + rs) * CAP + e] : -INFINITY;
-      pi[j] = ok ? sIdx[(cur * kGateRows + rs) * CAP + e] : -1;
+      pv[j] = ok ? sVal[((TWO_LISTS ? cur : 0) * kGateRows + rs) * CAP + e] : -INFINITY;
+      pi[j] = ok ? sIdx[((TWO_LISTS ? cur : 0) * kGateRows + rs) * CAP + e] : -1;
       vmin = fminf(vmin, ok ? pv[j] : INFINITY);
       vmax = fmaxf(vmax, pv[j]);
     }
@@ -408,7 +413,7 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
     // the place of the weakest winner if it beats it.  That is the top kp of the union, in the same total order
     // (score descending, chunk descending) as the bisection below, which stays for the first group and for rows
     // with more entrants than a list holds.
-    if (g > 0 && __all(m_prev == kp || nc <= c0)) {
+    if (TWO_LISTS && g > 0 && __all(m_prev == kp || nc <= c0)) {
       float pmin = INFINITY;
 #pragma unroll
       for (int j = 0; j < PL; ++j) pmin = fminf(pmin, pi[j] >= 0 ? pv[j] : INFINITY);
@@ -598,8 +603,9 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
     }
     int slot = 0;
     if (nwin > 0) slot = atomicAdd(&sCnt[nxt * kGateRows + rs], nwin);
-    float *ov = sVal + (size_t)(nxt * kGateRows + rs) * CAP;
-    int *oi = sIdx + (size_t)(nxt * kGateRows + rs) * CAP;
+    float *ov = sVal + (size_t)((TWO_LISTS ? nxt : 0) * kGateRows + rs) * CAP;
+    int *oi = sIdx + (size_t)((TWO_LISTS ? nxt : 0) * kGateRows + rs) * CAP;
+    if (!TWO_LISTS) wave_lds_fence();  // (one list: both lanes of the row have read it into registers)
     if (__any(nwin > 0)) {  // (no branches inside: a lane without a winner at a position stores to its trash word)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
@@ -636,7 +642,7 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
     for (int j = 0; j < PL; ++j) {
       const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
       if (e < m) {
-        const int c = sIdx[(cur * kGateRows + rs) * CAP + e];
+        const int c = sIdx[((TWO_LISTS ? cur : 0) * kGateRows + rs) * CAP + e];
         atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
         atomicAdd(&sHist[c], 1);
       }
@@ -874,7 +880,7 @@ template <int HD, int NT, int CAP>
 static size_t gate_big_smem(const TopkParams &p) {
   const size_t tile = (size_t)NT * 32 * (HD + 16) * 2;
   if ((size_t)p.W * kGateRows * 4 > tile) return (size_t)1 << 30;  // the selection words reuse the tile
-  return tile + (size_t)2 * kGateRows * CAP * 8 + (size_t)2 * kGateRows * 4 + (size_t)p.max_cols * 4 + 256 * 4;
+  return tile + (size_t)(CAP <= kBigCap ? 2 : 1) * kGateRows * CAP * 8 + (size_t)2 * kGateRows * 4 + (size_t)p.max_cols * 4 + 256 * 4;
 }
 template <typename T, int HD, int NT, int CAP>
 static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
@@ -896,13 +902,16 @@ static int launch_gate_big_hd(const TopkParams &p, dim3 grid, hipStream_t s) {
   // up to 16 running winners per row: short lists and groups of 128 chunks, if that lets two workgroups share a compute unit
   const int kp = p.a.is_causal ? p.a.topk - 1 : p.a.topk;
   if (p.a.head_dim <= 64) {
+    if (kp > kBigCap) return launch_gate_big<T, 64, 4, kBigCapMax>(p, grid, s);
     if (kp <= 16 && gate_big_smem<64, 4, 16>(p) <= 80 * 1024) return launch_gate_big<T, 64, 4, 16>(p, grid, s);
     return launch_gate_big<T, 64, 8, kBigCap>(p, grid, s);
   }
   if (p.a.head_dim <= 128) {
+    if (kp > kBigCap) return launch_gate_big<T, 128, 4, kBigCapMax>(p, grid, s);
     if (kp <= 16 && gate_big_smem<128, 4, 16>(p) <= 80 * 1024) return launch_gate_big<T, 128, 4, 16>(p, grid, s);
     return launch_gate_big<T, 128, 8, kBigCap>(p, grid, s);
   }
+  if (kp > kBigCap) return launch_gate_big<T, 256, 2, kBigCapMax>(p, grid, s);
   return launch_gate_big<T, 256, 4, kBigCap>(p, grid, s);
 }
 template <typename T>
@@ -947,11 +956,6 @@ static int fused_topk_run(const fmoba_fused_topk_args *a, void *workspace, size_
     return 0;
   }
   const bool big = max_cols > 256;  // more chunks than the register-resident gate holds: grouped gate
-  if (big) {
-    const int kp = a->is_causal ? a->topk - 1 : a->topk;
-    FMOBA_REQUIRE(kp <= kBigCap, "fused_topk: with more than 256 key chunks per sequence moba_topk is limited to %d (got %d)",
-                  kBigCap + (a->is_causal ? 1 : 0), a->topk);
-  }
   FMOBA_REQUIRE(a->q && a->km, "fused_topk: null q/km pointer");
   FMOBA_REQUIRE(a->q_row_stride % 8 == 0 && a->q_head_stride % 8 == 0 && a->km_row_stride % 8 == 0 && a->km_head_stride % 8 == 0,
                 "fused_topk: strides must be multiples of 8 elements");

@@ -170,15 +170,25 @@ def test_gating_headline_shape_small(fm):
 
 
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("topk", [1, 4, 16, 33])
+@pytest.mark.parametrize("topk", [1, 4, 16, 33, 40, 64])
 def test_gating_more_than_256_chunks_per_sequence(fm, topk, causal):
     # the grouped gate: 550 and 500/175 chunks per sequence, (b, h, s) in the spirit of tests/test_fused_topk.py:119-122
-    if topk == 33 and not causal:
-        topk = 32
+    # (running lists of 16, 32 and -- top-k above 33 -- 64 winners per row)
     q, k, cuq, cuk = _gate_case(fm, 3, [1100], [1100], 2, 2, 64, 2, topk, causal, torch.float16)
     _check_gating(fm, q, k, cuq, cuk, 2, topk, causal)
     q, k, cuq, cuk = _gate_case(fm, 4, [2000, 0, 700], [2000, 0, 700], 4, 2, 128, 4, topk, causal)
     _check_gating(fm, q, k, cuq, cuk, 4, topk, causal)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("topk", [16, 33, 64])
+def test_gating_reference_grid_point_1024_chunks(fm, topk, causal):
+    # (b, h, s) = (8, 2, 1024) with chunk size 1 of tests/test_fused_topk.py:115-122: 1024 chunks per sequence
+    q, k, cuq, cuk = _gate_case(fm, 0, [1024] * 8, [1024] * 8, 2, 2, 64, 1, topk, causal, torch.bfloat16)
+    _check_gating(fm, q, k, cuq, cuk, 1, topk, causal)
+    # head_dim 256 takes the variants with the smallest groups
+    q, k, cuq, cuk = _gate_case(fm, 1, [1024], [1024], 2, 1, 256, 2, topk, causal, torch.float16)
+    _check_gating(fm, q, k, cuq, cuk, 2, topk, causal)
 
 
 @pytest.mark.parametrize("causal", [True, False])
@@ -187,12 +197,10 @@ def test_gating_more_than_256_chunks_exact_ties(fm, causal):
     _check_gating(fm, q, k, cuq, cuk, 4, 6, causal, integer=True)
 
 
-def test_gating_more_than_256_chunks_topk_limit(fm):
-    q = torch.zeros(600, 2, 64, dtype=torch.bfloat16).cuda()
-    cu = torch.tensor([0, 600], dtype=torch.int32).cuda()
-    km, cu_km, _ = fm.pool.flash_topk_mean_pool(q, cu, 600, 2)
-    with pytest.raises(RuntimeError, match="limited to 33"):
-        fm.hip.moba_fused_topk(q, km, cu, cu, cu_km, 600, 600, 40, 2, True)
+@pytest.mark.parametrize("causal", [True, False])
+def test_gating_more_than_256_chunks_exact_ties_long_lists(fm, causal):
+    q, k, cuq, cuk = _gate_case(fm, 10, [1500], [1500], 2, 1, 64, 4, 50, causal, integer=True)
+    _check_gating(fm, q, k, cuq, cuk, 4, 50, causal, integer=True)
 
 
 def test_gating_no_keys(fm):
