@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libflash_moba_hip.so")
-SOURCES = ["fmoba_host.hip", "mean_pool.hip", "topk_csc.hip", "varlen_sort.hip", "attn_fwd.hip", "attn_fwd_rows.hip", "attn_bwd.hip"]
+SOURCES = ["fmoba_host.hip", "mean_pool.hip", "topk_csc.hip", "varlen_sort.hip", "attn_fwd.hip", "attn_fwd_rows.hip", "attn_bwd.hip", "attn_bwd_wide.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # keep packed-fp32 VALU ops out of the generated code

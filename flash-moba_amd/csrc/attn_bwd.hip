@@ -674,7 +674,7 @@ __device__ __forceinline__ DqItem dq_decode_item(int id, int npairs, int nsb_max
 }
 
 template <typename T, int HD>
-__global__ __launch_bounds__(512, 4) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a, const uint16_t *ds_ws, int nsb_max) {
+__global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a, const uint16_t *ds_ws, int nsb_max) {
   typedef DqSmem<HD> SM;
   constexpr int LDQ = SM::LDQ, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
   constexpr int KVV = 64 * VPR / 256;  // K-tile vectors per loader thread
@@ -934,14 +934,15 @@ __global__ __launch_bounds__(512, 4) void attn_bwd_dq_kernel(fmoba_attn_bwd_args
             make_uint2(pack2<T>(acc[dt][4 * g] * a.softmax_scale, acc[dt][4 * g + 1] * a.softmax_scale),
                        pack2<T>(acc[dt][4 * g + 2] * a.softmax_scale, acc[dt][4 * g + 3] * a.softmax_scale));
     wave_lds_fence();
-    if ((lane & 15) * 8 < D) {
+    {
       uint16_t *op = reinterpret_cast<uint16_t *>(a.dq) + (int64_t)(q0 + m0) * a.dq_row_stride + (int64_t)h * a.dq_head_stride;
+      // rows leave as 16-byte pieces, VPR of them per row, consecutive lanes taking consecutive pieces
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int rl = 4 * k + (lane >> 4);
+      for (int v0 = 0; v0 < 32 * VPR; v0 += 64) {
+        const int v = v0 + lane, rl = v / VPR, e = (v - rl * VPR) * 8;
         const int r2 = wave * 32 + rl;
-        if (r2 < rows_sb)
-          *reinterpret_cast<Pack8 *>(op + (int64_t)r2 * a.dq_row_stride + (lane & 15) * 8) = *reinterpret_cast<const Pack8 *>(sOut + rl * LDO + (lane & 15) * 8);
+        if (r2 < rows_sb && e < D)
+          *reinterpret_cast<Pack8 *>(op + (int64_t)r2 * a.dq_row_stride + e) = *reinterpret_cast<const Pack8 *>(sOut + rl * LDO + e);
       }
     }
   }
@@ -1085,6 +1086,9 @@ static int launch_dq(const fmoba_attn_bwd_args &a, const uint16_t *ws, hipStream
   return 0;
 }
 
+// head dimensions above 128 (attn_bwd_wide.hip)
+int run_bwd_dkdv_wide(const fmoba_attn_bwd_args &a, uint16_t *ds_ws, hipStream_t s);
+
 // columns of a multiple of 128 keys: one workgroup (and one dQ partial per visit) per 128 keys
 static inline bool bwd_wide_blocks(const fmoba_attn_bwd_args &a) { return a.head_dim > 64 && a.lg_block_n % 128 == 0; }
 
@@ -1094,6 +1098,7 @@ static inline bool bwd_wide_blocks(const fmoba_attn_bwd_args &a) { return a.head
 // top-k 8 to 32): a row selects a tenth of the chunks it may see (64-key blocks), three eighths with 128-key blocks,
 // where a visit leaves one partial per 128 keys.
 static int bwd_dq_partials(const fmoba_attn_bwd_args &a) {
+  if (a.head_dim > 128) return 0;  // head dimensions above 128: dS tiles and the row-block pass only
   if (a.dq_mode == 1) return 0;
   if (a.dq_mode == 2) return 1;
   const double chunks_per_seq = (double)a.total_k / a.batch / a.lg_block_n;
@@ -1116,6 +1121,14 @@ static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hi
     while (lpr * 8 < a.head_dim) lpr <<= 1;
     const int rows_per_block = 256 / lpr;
     hipLaunchKernelGGL(bwd_prep_kernel<T>, dim3(ceil_div(a.max_seqlen_q, rows_per_block), a.heads, a.batch), dim3(256), 0, s, a, lpr);
+  }
+  if (a.head_dim > 128) {
+    // the plain feature-split dK/dV kernel (attn_bwd_wide.hip), then the row-block dQ pass over its dS tiles
+    if (phases & FMOBA_BWD_DKDV)
+      if (int rc = run_bwd_dkdv_wide(a, ws.ds, s)) return rc;
+    if (phases & FMOBA_BWD_DQ)
+      if (int rc = launch_dq<T, 256>(a, ws.ds, s)) return rc;
+    return 0;
   }
   if (phases & FMOBA_BWD_DKDV) {
     int rc;
@@ -1176,7 +1189,6 @@ extern "C" int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phase
   FMOBA_REQUIRE(a->batch > 0, "batch size must be positive");
   FMOBA_REQUIRE(a->head_dim > 0 && a->head_dim % 8 == 0, "head_size should be a multiple of 8");
   FMOBA_REQUIRE(a->head_dim <= 256, "FlashMoBA backward only supports head dimension at most 256");
-  FMOBA_REQUIRE(a->head_dim <= 128, "attn_bwd: head dimensions above 128 are not built yet (got %d)", a->head_dim);
   FMOBA_REQUIRE(a->heads > 0 && a->heads_k > 0 && a->heads % a->heads_k == 0, "Number of heads in key/value must divide number of heads in query");
   FMOBA_REQUIRE(a->lg_block_m % 64 == 0, "m_lg_block_dim must be a multiple of 64");
   FMOBA_REQUIRE(a->lg_block_n > 0 && a->lg_block_n % 64 == 0, "n_lg_block_dim must be a multiple of 64");
@@ -1220,6 +1232,7 @@ extern "C" int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phase
   FMOBA_REQUIRE(a->k && a->v && a->col_offsets && a->col_nnz && a->row_indices, "attn_bwd: null k/v/CSC pointer");
   FMOBA_REQUIRE(a->max_visits_per_row > 0, "attn_bwd: max_visits_per_row must be positive");
   FMOBA_REQUIRE(a->dq_mode >= 0 && a->dq_mode <= 2, "attn_bwd: dq_mode must be 0 (automatic), 1 (row blocks) or 2 (partials)");
+  FMOBA_REQUIRE(a->dq_mode != 2 || a->head_dim <= 128, "attn_bwd: head dimensions above 128 only have the row-block form of dQ");
   FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= fmoba_attn_bwd_workspace_bytes(a), "attn_bwd: workspace too small");
   const size_t rows = (size_t)a->total_q * a->heads;
   uintptr_t wp = ((uintptr_t)a->workspace + 255) & ~(uintptr_t)255;

@@ -521,6 +521,7 @@ int run_fwd_rows(const fmoba_attn_fwd_args &a, int phases, hipStream_t s);
 // visit: the first wins while a row selects more than about a fifth of the chunks it may see (64-key blocks) or
 // more than about three eighths of them (128-key blocks, whose visits cost the column form less per key).
 static bool fwd_use_rows(const fmoba_attn_fwd_args &a) {
+  if (a.head_dim > 128) return true;  // head dimensions above 128 only have the row-block form
   if (a.fwd_mode == 1) return false;
   if (!fwd_rows_feasible(a)) return false;
   if (a.fwd_mode == 2) return true;
@@ -603,7 +604,6 @@ static int fwd_check_common(const fmoba_attn_fwd_args *a) {
   FMOBA_REQUIRE(a->batch > 0, "batch size must be positive");
   FMOBA_REQUIRE(a->head_dim > 0 && a->head_dim <= 256, "FlashMoBA forward only supports head dimension at most 256");
   FMOBA_REQUIRE(a->head_dim % 8 == 0, "query, key, value, and out_ must have a head_size that is a multiple of 8");
-  FMOBA_REQUIRE(a->head_dim <= 128, "attn_fwd: head dimensions above 128 are not built yet (got %d)", a->head_dim);
   FMOBA_REQUIRE(a->heads > 0 && a->heads_k > 0 && a->heads % a->heads_k == 0, "Number of heads in key/value must divide number of heads in query");
   FMOBA_REQUIRE(a->lg_block_m >= 128 && a->lg_block_m <= 1024, "m_lg_block_dim must be at least 128 and at most 1024");
   FMOBA_REQUIRE(a->lg_block_m % 64 == 0, "m_lg_block_dim must be a multiple of 64");
@@ -658,7 +658,8 @@ extern "C" int fmoba_attn_fwd_phases(const fmoba_attn_fwd_args *a, int32_t phase
                 "attn_fwd: q, k, v and out must be 16-byte aligned");
   FMOBA_REQUIRE(a->max_visits_per_row > 0, "attn_fwd: max_visits_per_row must be positive");
   FMOBA_REQUIRE(a->fwd_mode >= 0 && a->fwd_mode <= 2, "attn_fwd: fwd_mode must be 0 (automatic), 1 (columns) or 2 (row blocks)");
-  FMOBA_REQUIRE(a->fwd_mode != 2 || fwd_rows_feasible(*a), "attn_fwd: the row-block form does not take this shape (more than %d chunks or %d keys per sequence)",
+  FMOBA_REQUIRE(a->fwd_mode != 1 || a->head_dim <= 128, "attn_fwd: head dimensions above 128 only have the row-block form");
+  FMOBA_REQUIRE((a->fwd_mode != 2 && a->head_dim <= 128) || fwd_rows_feasible(*a), "attn_fwd: the row-block form does not take this shape (more than %d chunks or %d keys per sequence)",
                 32 * 128, 64 * 4096);
   const size_t need = fmoba_attn_fwd_workspace_bytes(a);
   FMOBA_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, "attn_fwd: workspace too small (%zu < %zu)", a->workspace_bytes, need);

@@ -384,16 +384,14 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
     if (valid && hh == 0)
       a.softmax_lse[(int64_t)h * a.total_q + q0 + row] = empty ? INFINITY : (m_run * scale_log2 + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
     wave_lds_fence();
-    // rows leave as 16-byte pieces: lane -> (row 4k + lane / 16, features 8 * (lane % 16))
-    if ((lane & 15) * 8 < D) {
+    // rows leave as 16-byte pieces, VPR of them per row, consecutive lanes taking consecutive pieces
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int rl = 4 * k + (lane >> 4);
-        const int r2 = r0 + wave * 32 + rl;
-        if (r2 < Lq) {
-          const Pack8 x = *reinterpret_cast<const Pack8 *>(sOut + rl * LDO + (lane & 15) * 8);
-          *reinterpret_cast<Pack8 *>(reinterpret_cast<uint16_t *>(a.out) + (int64_t)(q0 + r2) * a.o_row_stride + (int64_t)h * a.o_head_stride + (lane & 15) * 8) = x;
-        }
+    for (int v0 = 0; v0 < 32 * VPR; v0 += 64) {
+      const int v = v0 + lane, rl = v / VPR, e = (v - rl * VPR) * 8;
+      const int r2 = r0 + wave * 32 + rl;
+      if (r2 < Lq && e < D) {
+        const Pack8 x = *reinterpret_cast<const Pack8 *>(sOut + rl * LDO + e);
+        *reinterpret_cast<Pack8 *>(reinterpret_cast<uint16_t *>(a.out) + (int64_t)(q0 + r2) * a.o_row_stride + (int64_t)h * a.o_head_stride + e) = x;
       }
     }
   }
@@ -417,7 +415,7 @@ static int launch_rows(const fmoba_attn_fwd_args &a, const uint32_t *bm, int nw,
 }
 
 bool fwd_rows_feasible(const fmoba_attn_fwd_args &a) {
-  return a.head_dim <= 128 && ceil_div(a.max_cols, 32) <= kRowsWordCap && ceil_div(a.max_seqlen_k, 64) <= kRowsStepCap &&
+  return a.head_dim <= 256 && ceil_div(a.max_cols, 32) <= kRowsWordCap && ceil_div(a.max_seqlen_k, 64) <= kRowsStepCap &&
          a.max_cols < 32768 && a.lg_block_n % 64 == 0;
 }
 
@@ -445,8 +443,10 @@ int run_fwd_rows(const fmoba_attn_fwd_args &a, int phases, hipStream_t s) {
     int rc;
     if (a.head_dim <= 64)
       rc = bf ? launch_rows<bf16_t, 64>(a, bm, nw, s) : launch_rows<f16_t, 64>(a, bm, nw, s);
-    else
+    else if (a.head_dim <= 128)
       rc = bf ? launch_rows<bf16_t, 128>(a, bm, nw, s) : launch_rows<f16_t, 128>(a, bm, nw, s);
+    else
+      rc = bf ? launch_rows<bf16_t, 256>(a, bm, nw, s) : launch_rows<f16_t, 256>(a, bm, nw, s);
     if (rc) return rc;
   }
   return 0;

@@ -370,6 +370,40 @@ def test_attention_random_pattern(fm, sq, sk, d, mha, causal, dtype):
     _check_attention(fm, q, k, v, dout, cuq, cuk, co, cn, ind, 64, causal)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("mha", ["mha", "gqa"])
+@pytest.mark.parametrize("d", [32, 80, 111, 160, 192, 224, 256])
+@pytest.mark.parametrize("sq,sk", [(113, 203), (256, 512), (1023, 1024)])
+def test_attention_random_pattern_more_head_dims(fm, sq, sk, d, mha, causal, dtype):
+    # the rest of the head dimensions tests/test_moba_attn.py:48-49 sweeps (32 .. 256, odd ones padded to a multiple
+    # of 8 by the interface); above 128 the forward runs its row-block form and the backward its feature-split kernels
+    H = 4
+    Hk = {"mha": 4, "gqa": 2}[mha]
+    rng = np.random.RandomState(sq + sk + d)
+    lens_q = [max(1, sq - int(x)) for x in rng.randint(0, 20, 2)]
+    lens_k = [max(1, sk - int(x)) for x in rng.randint(0, 20, 2)]
+    q, k, v, dout, cuq, cuk = _attn_inputs(d, lens_q, lens_k, H, Hk, d, dtype)
+    co, cn, ind = _random_csc(3, lens_q, lens_k, H, 64, 4, causal)
+    _check_attention(fm, q, k, v, dout, cuq, cuk, co, cn, ind, 64, causal)
+
+
+def test_attention_head_dim_256_on_gated_patterns_with_wide_chunks(fm):
+    # chunk 128 (two 64-key blocks per column) and the fused path at head dimension 256 / 192
+    for d, chunk, topk in ((256, 128, 3), (192, 64, 5)):
+        lens = [700, 130, 0, 1300]
+        q, k, v, cu, dout = O.make_inputs(lens, 2, d, chunk, 23, torch.bfloat16, with_dout=True)
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        out = fm.api.flash_moba_varlen_func(qg, kg, vg, cu.cuda(), cu.cuda(), max(lens), max(lens), chunk, topk, causal=True)
+        out.backward(dout.cuda())
+        co, cn, ind = fm.api.flash_topk_varlen_func(q.cuda(), k.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens), topk, chunk, causal=True)
+        o_ref, _, dq_ref, dk_ref, dv_ref = O.attn_fwd_bwd(q, k, v, dout, cu, cu, co.cpu(), cn.cpu(), ind.cpu(), chunk, None, True)
+        assert_close("out", out, o_ref, 2e-2, 1e-2)
+        assert_close("dq", qg.grad, dq_ref, 2e-2, 1e-2)
+        assert_close("dk", kg.grad, dk_ref, 2e-2, 1e-2)
+        assert_close("dv", vg.grad, dv_ref, 2e-2, 1e-2)
+
+
 @pytest.mark.parametrize("form", [1, 2])
 @pytest.mark.parametrize("sq,sk,d,Hk,chunk,topk,causal,dtype", [
     (300, 300, 128, 4, 64, 3, True, torch.bfloat16),
