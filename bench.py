@@ -38,7 +38,8 @@ CONFIGS = {
     "c2": ([8192], 16, 128, 128, 8, False),
     "c3": ([32768], 32, 128, 128, 16, True),
     "c5": ([262144], 16, 128, 128, 16, True),
-    # one point of the reference's own sequence-length sweep (benchmarks/bench_flash_moba.py): batch 2, top-k 8
+    # two points of the reference's own sequence-length sweep (benchmarks/bench_flash_moba.py): batch 2, chunk 128, top-k 8
+    "sweep16k": ([16384, 16384], 16, 128, 128, 8, True),
     "sweep64k": ([65536, 65536], 16, 128, 128, 8, True),
 }
 
@@ -153,6 +154,21 @@ def cpu_baseline(q, k, v, cu, seqlens, chunk, topk, budget_s=12.0):
                   + f"; {dt:.1f} s of CPU time; effective sparse FLOPs / time",
         "seconds": dt,
     }
+
+
+def dense_sdpa_ms(cfg, dev, iters=3):
+    """Forward + backward of dense causal attention (torch scaled_dot_product_attention, bf16) on a sweep shape: the
+    baseline benchmarks/bench_flash_moba.py of the reference compares with."""
+    seqlens, H, D, _, _, _ = cfg
+    B, L = len(seqlens), seqlens[0]
+    q, k, v = (torch.randn((B, H, L, D), device=dev, dtype=torch.bfloat16, requires_grad=True) for _ in range(3))
+    g = torch.randn((B, H, L, D), device=dev, dtype=torch.bfloat16)
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True).backward(g)
+
+    return time_events(step, iters)
 
 
 def run_config(name, steps, warmup, args, dev, cpu_budget_s):
@@ -344,11 +360,13 @@ def main():
     if args.config == "headline" and not args.no_configs:
         # every other BASELINE config that runs on the GPU, a few steps each, same measurements
         result["configs"] = []
-        for name, k_steps in (("c2", 20), ("c3", 10), ("c5", 3)):
+        for name, k_steps, cpu_s in (("c2", 20, 4.0), ("c3", 10, 4.0), ("c5", 3, 4.0), ("sweep16k", 10, 0.0), ("sweep64k", 5, 0.0)):
             torch.cuda.empty_cache()
-            r = run_config(name, k_steps, 2, args, dev, 0.0 if args.no_cpu else 4.0)
+            r = run_config(name, k_steps, 2, args, dev, 0.0 if args.no_cpu else cpu_s)
+            if name == "sweep16k":
+                r["dense_sdpa_fwd_bwd_ms"] = dense_sdpa_ms(CONFIGS[name], dev)  # the dense baseline of the reference's benchmark
             keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "frac_of_bf16_mfma_peak", "pairs", "flops_per_step",
-                    "topk_csc_ms", "stages", "roofline", "cpu_baseline")
+                    "topk_csc_ms", "stages", "roofline", "cpu_baseline", "dense_sdpa_fwd_bwd_ms")
             entry = {"name": name, "workload": r["config"]["workload"]}
             entry.update({k: r[k] for k in keep if k in r})
             result["configs"].append(entry)

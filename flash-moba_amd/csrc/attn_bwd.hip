@@ -967,7 +967,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_combine_kernel(fmoba_attn_bwd
   const int64_t row = rh / a.heads;
   const int h = (int)(rh - row * a.heads);
   const int D = a.head_dim;
-  const int n = valid ? min(ws.cnt[rh], ws.cap) : 0;
+  const int nall = valid ? ws.cnt[rh] : 0;
+  const int n = min(nall, ws.cap);
+  if (nall > ws.cap && li == 0 && a.visits_overflow != nullptr) atomicMax(a.visits_overflow, nall);  // visits were dropped
   int nmax = max(n, __shfl_xor(n, 16, 64));
   nmax = max(nmax, __shfl_xor(nmax, 32, 64));  // the wave walks the longest of its four rows
   const int c8 = li * 8;

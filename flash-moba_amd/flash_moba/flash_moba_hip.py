@@ -59,7 +59,8 @@ class AttnFwdArgs(ctypes.Structure):
                 ("lg_block_m", c_i32), ("lg_block_n", c_i32), ("is_causal", c_i32), ("dtype", c_i32),
                 ("max_visits_per_row", c_i32), ("fwd_mode", c_i32), ("softmax_scale", c_f32),
                 ("q_row_stride", c_i64), ("q_head_stride", c_i64), ("k_row_stride", c_i64), ("k_head_stride", c_i64),
-                ("v_row_stride", c_i64), ("v_head_stride", c_i64), ("o_row_stride", c_i64), ("o_head_stride", c_i64)]
+                ("v_row_stride", c_i64), ("v_head_stride", c_i64), ("o_row_stride", c_i64), ("o_head_stride", c_i64),
+                ("visits_overflow", c_vp)]
 
 
 class AttnBwdArgs(ctypes.Structure):
@@ -76,7 +77,7 @@ class AttnBwdArgs(ctypes.Structure):
                 ("v_row_stride", c_i64), ("v_head_stride", c_i64), ("o_row_stride", c_i64), ("o_head_stride", c_i64),
                 ("do_row_stride", c_i64), ("do_head_stride", c_i64),
                 ("dq_row_stride", c_i64), ("dq_head_stride", c_i64), ("dk_row_stride", c_i64), ("dk_head_stride", c_i64),
-                ("dv_row_stride", c_i64), ("dv_head_stride", c_i64)]
+                ("dv_row_stride", c_i64), ("dv_head_stride", c_i64), ("visits_overflow", c_vp)]
 
 
 EXPORTS = {
@@ -337,7 +338,7 @@ def _count_visits(lib, q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_s
                      moba_col_offsets.data_ptr(), moba_col_nnz.data_ptr(), moba_row_indices.data_ptr(),
                      cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), None, None, 0,
                      batch, total_q, total_k, heads, heads_k, d, int(max_seqlen_q), int(max_seqlen_k), max_cols,
-                     int(m_lg_block_dim), int(n_lg_block_dim), 0, _dt(q), 0, 0, 1.0, 0, 0, 0, 0, 0, 0, 0, 0)
+                     int(m_lg_block_dim), int(n_lg_block_dim), 0, _dt(q), 0, 0, 1.0, 0, 0, 0, 0, 0, 0, 0, 0, None)
     _check(lib.fmoba_csc_max_row_visits(ctypes.byref(a0), counts.data_ptr(), counts[total_q * heads:].data_ptr(), _stream()))
     return max(1, int(counts[total_q * heads].item()))
 
@@ -364,13 +365,14 @@ def count_max_visits(q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seq
 def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k,
                     seqused_k, leftpad_k, alibi_slopes, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                     zero_tensors, is_causal, softcap, return_softmax, m_lg_block_dim, n_lg_block_dim, gen=None, _phases=None,
-                    _fwd_mode=0, _max_visits=None, _selection=None):
+                    _fwd_mode=0, _max_visits=None, _selection=None, _overflow=None):
     """Returns [out, softmax_lse (H, total_q) fp32, p (empty), rng_state (2,) int64].
 
     Beyond the reference's arguments: _max_visits, a bound on the (row, forward key block) visits of any (row, head)
     -- a gated pattern has top-k * lg_block_n / fwd_key_block(lg_block_n); None or a value below 1 makes the call count
     them from the pattern (one device-to-host read) -- and _selection, the int32 selection words of the gating call that
-    produced exactly this pattern (moba_fused_topk(return_selection=True))."""
+    produced exactly this pattern (moba_fused_topk(return_selection=True)); _overflow, a zeroed int32 tensor of one
+    element that a form with per-visit partial results raises to the visit count of a row that exceeds the bound."""
     dtype = q.dtype
     _require(dtype in (torch.float16, torch.bfloat16), "FlashMoBA only support fp16 and bf16 data type")
     _require(k.dtype == dtype, "query and key must have the same dtype")
@@ -425,7 +427,7 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
                                int(m_lg_block_dim), int(n_lg_block_dim), int(bool(is_causal)), _dt(q), visits,
                                int(_fwd_mode), float(softmax_scale),
                                q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
-                               out.stride(0), out.stride(1))
+                               out.stride(0), out.stride(1), _ptr(_overflow))
 
         visits = _max_visits
         if visits is None or int(visits) < 1:
@@ -452,7 +454,7 @@ def moba_varlen_fwd(q, k, v, out_, moba_col_offsets, moba_col_nnz, moba_row_indi
 def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_offsets, moba_col_nnz, moba_row_indices,
                     cu_seqlens_q, cu_seqlens_k, alibi_slopes, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                     zero_tensors, is_causal, softcap, deterministic, m_lg_block_dim, n_lg_block_dim, gen=None,
-                    rng_state=None, _phases=None, _dq_mode=0, _max_visits=None):
+                    rng_state=None, _phases=None, _dq_mode=0, _max_visits=None, _overflow=None):
     """Returns [dq, dk, dv, softmax_d (H, total_q + 128*batch) fp32].
 
     Beyond the reference's arguments: _max_visits, a bound on the visits of any (row, head) in 64-KEY blocks (a gated
@@ -528,7 +530,7 @@ def moba_varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, moba_col_off
                         visits, int(_dq_mode), float(softmax_scale),
                         q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                         out.stride(0), out.stride(1), dout.stride(0), dout.stride(1),
-                        dq.stride(0), dq.stride(1), dk_e.stride(0), dk_e.stride(1), dv_e.stride(0), dv_e.stride(1))
+                        dq.stride(0), dq.stride(1), dk_e.stride(0), dk_e.stride(1), dv_e.stride(0), dv_e.stride(1), _ptr(_overflow))
         ws_bytes = lib.fmoba_attn_bwd_workspace_bytes(ctypes.byref(a))
         _last.bwd_partials = int(lib.fmoba_attn_bwd_uses_partials(ctypes.byref(a)))
         ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)

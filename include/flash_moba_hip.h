@@ -128,7 +128,7 @@ int fmoba_varlen_sort(const int64_t *seg_starts, const int64_t *seg_ends, int64_
  * block is fmoba_attn_fwd_key_block(lg_block_n) keys (128 if lg_block_n is a multiple of 128,
  * else 64).  max_visits_per_row bounds the number of visits of any (row, head): for a pattern
  * from the gating, topk * lg_block_n / key_block; for an arbitrary pattern,
- * fmoba_csc_max_row_visits() computes it.  Visits beyond the bound are dropped.
+ * fmoba_csc_max_row_visits() computes it.  Visits beyond the bound are dropped (and reported: visits_overflow).
  * workspace: fmoba_attn_fwd_workspace_bytes() bytes, contents undefined on entry and return.
  * ---------------------------------------------------------------------------------- */
 typedef struct {
@@ -155,6 +155,11 @@ typedef struct {
   float softmax_scale;
   int64_t q_row_stride, q_head_stride, k_row_stride, k_head_stride;
   int64_t v_row_stride, v_head_stride, o_row_stride, o_head_stride;
+  /* optional (may be NULL): one int32 the caller has set to 0.  A form that stores per-visit partial results
+   * raises it (atomic max) to the visit count of any (row, head) that exceeds max_visits_per_row -- such a
+   * row's result is wrong, its surplus visits were dropped -- so that a caller who passed a bound of its own
+   * can tell afterwards (a device-to-host read after the stream has passed the call).  Stays 0 otherwise. */
+  int32_t *visits_overflow;
 } fmoba_attn_fwd_args;
 int32_t fmoba_attn_fwd_key_block(int32_t lg_block_n);
 /* Bytes of workspace for the call described by `a` (sizes, max_visits_per_row and fwd_mode are read,
@@ -196,7 +201,7 @@ int fmoba_attn_fwd_phases(const fmoba_attn_fwd_args *a, int32_t phases, void *st
  *   col_nnz[i] must be <= it).  max_visits_per_row bounds the visits of any (row, head): for a
  *   pattern from the gating topk * lg_block_n / 64; for an arbitrary pattern
  *   fmoba_csc_max_row_visits() counts them in forward key blocks, multiply by
- *   fmoba_attn_fwd_key_block(lg_block_n) / 64.  Visits beyond the bound are dropped.
+ *   fmoba_attn_fwd_key_block(lg_block_n) / 64.  Visits beyond the bound are dropped (and reported: visits_overflow).
  *   No floating-point atomics: results are bitwise reproducible whatever `deterministic` says.
  * ---------------------------------------------------------------------------------- */
 typedef struct {
@@ -222,6 +227,7 @@ typedef struct {
   int64_t do_row_stride, do_head_stride;
   int64_t dq_row_stride, dq_head_stride, dk_row_stride, dk_head_stride;
   int64_t dv_row_stride, dv_head_stride;
+  int32_t *visits_overflow;  /* optional, as in fmoba_attn_fwd_args (counts are in the backward's key blocks) */
 } fmoba_attn_bwd_args;
 int32_t fmoba_attn_bwd_uses_partials(const fmoba_attn_bwd_args *a);
 size_t fmoba_attn_bwd_workspace_bytes(const fmoba_attn_bwd_args *a);

@@ -572,6 +572,22 @@ def test_attention_rows_without_keys_and_no_keys_at_all(fm):
     assert (out == 0).all() and (lse == float("inf")).all()
 
 
+def test_a_visits_bound_that_is_too_small_is_reported(fm):
+    # a caller's own bound on a row's visits sizes the partial-result buffers; visits beyond it are dropped, and the
+    # optional status word then holds the largest visit count seen (0 when the bound held)
+    lens = [900]
+    q, k, v, cu, dout = O.make_inputs(lens, 2, 128, 64, 13, torch.bfloat16, with_dout=True)
+    Q, K, V, CU, DO = q.cuda(), k.cuda(), v.cuda(), cu.cuda(), dout.cuda()
+    co, cn, ind = fm.api.flash_topk_varlen_func(Q, K, CU, CU, 900, 900, 6, 64, causal=True)
+    for bound, want in ((6, 0), (4, 6)):
+        st = torch.zeros(2, dtype=torch.int32, device="cuda")
+        out, lse, _, _ = fm.hip.moba_varlen_fwd(Q, K, V, None, co, cn, ind, CU, CU, None, None, None, 900, 900, 0.0, 128 ** -0.5, False, True,
+                                                0.0, False, 128, 64, None, _fwd_mode=1, _max_visits=bound, _overflow=st[0:1])
+        fm.hip.moba_varlen_bwd(DO, Q, K, V, out, lse, None, None, None, co, cn, ind, CU, CU, None, 900, 900, 0.0, 128 ** -0.5, False, True,
+                               0.0, False, 128, 64, None, None, _dq_mode=2, _max_visits=bound, _overflow=st[1:2])
+        assert st.tolist() == [want, want]
+
+
 def test_attention_rejects_unsupported_options(fm):
     q, k, v, dout, cuq, cuk = _attn_inputs(4, [128], [128], 2, 2, 64, torch.bfloat16)
     co, cn, ind = _random_csc(1, [128], [128], 2, 64, 2, True)
