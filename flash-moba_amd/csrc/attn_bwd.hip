@@ -650,8 +650,8 @@ struct DqSmem {
   static constexpr int LDQ = HD + 16;  // elements, K tile
   static constexpr int LDO = HD + 8;   // elements, per-wave output tile [32 rows][LDO] (reuses the K tiles at the end)
   static constexpr size_t oK = 0;                                   // [2][64][LDQ]
-  static constexpr size_t oTag = oK + (size_t)2 * 64 * LDQ * 2;    // int[3][128]: (step tag << 8) | list position of the row in that step
-  static constexpr size_t oLo = oTag + 3 * kDqRows * 4;
+  static constexpr size_t oTag = oK + (size_t)2 * 64 * LDQ * 2;    // int[3][rows of the block, at most 256]: (step tag << 8) | list position of the row in that step
+  static constexpr size_t oLo = oTag + 3 * 2 * kDqRows * 4;
   static constexpr size_t oCnt = oLo + kDqColBatch * 4;
   static constexpr size_t oStep = oCnt + kDqColBatch * 4;
   static constexpr size_t oOff = oStep + kDqMaxSteps * 4;          // int64[kDqColBatch]
@@ -673,9 +673,12 @@ __device__ __forceinline__ DqItem dq_decode_item(int id, int npairs, int nsb_max
   return w;
 }
 
-template <typename T, int HD>
-__global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a, const uint16_t *ds_ws, int nsb_max) {
+// RT: 32-row tiles per compute wave.  With two, a workgroup owns 256 rows and every K^T operand read from LDS feeds two
+// MFMAs; the accumulators then take 128 registers, and one workgroup fits a compute unit instead of two.
+template <typename T, int HD, int RT>
+__global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a, const uint16_t *ds_ws, int nsb_max) {
   typedef DqSmem<HD> SM;
+  constexpr int ROWS = kDqRows * RT;  // query rows of the workgroup
   constexpr int LDQ = SM::LDQ, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
   constexpr int KVV = 64 * VPR / 256;  // K-tile vectors per loader thread
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -692,10 +695,10 @@ __global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmob
   if (wi.pair < 0) return;
   const int b = wi.pair / a.heads, h = wi.pair - b * a.heads, sb = wi.sb;
   const int q0 = a.cu_seqlens_q[b], Lq = a.cu_seqlens_q[b + 1] - q0;
-  const int m0 = sb * kDqRows;
+  const int m0 = sb * ROWS;
   if (m0 >= Lq) return;
   const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
-  const int rows_sb = min(kDqRows, Lq - m0);
+  const int rows_sb = min(ROWS, Lq - m0);
   const int off = Lk - Lq;
   const int D = a.head_dim;
   const int hk = h / (a.heads / a.heads_k);
@@ -705,7 +708,7 @@ __global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmob
   const int ltid = tid & 255;
   const bool causal = a.is_causal != 0;
 
-  for (int v = tid; v < 3 * kDqRows; v += 512) sPos[v] = 0;  // step tags start at 1
+  for (int v = tid; v < 3 * ROWS; v += 512) sPos[v] = 0;  // step tags start at 1
 
   int ncols = min((Lk + Bn - 1) / Bn, a.max_cols);
   const int last_rowpos = m0 + rows_sb - 1 + off;
@@ -727,8 +730,8 @@ __global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmob
         base = coff[c];
         const int32_t *list = a.row_indices + base;
         lo = lower_bound_i32(list, nnz, m0);
-        const int hi = lo + lower_bound_i32(list + lo, nnz - lo, m0 + kDqRows);
-        cnt = min(hi - lo, kDqRows);
+        const int hi = lo + lower_bound_i32(list + lo, nnz - lo, m0 + ROWS);
+        cnt = min(hi - lo, ROWS);
       }
       sLo[c - cb] = lo;
       sCnt[c - cb] = cnt;
@@ -791,15 +794,15 @@ __global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmob
         const int4 info = sInfo[min(step, nsteps - 1)];
         const int n = __builtin_amdgcn_readfirstlane(info.y);
         const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
-        return a.row_indices[pos0 + min(ltid & 127, n - 1)];
+        return a.row_indices[pos0 + min(ltid & (ROWS - 1), n - 1)];
       };
       auto put_pos = [&](int step, int rr) {  // positions of the rows of `step`
-        if (step < nsteps && ltid < kDqRows) {
+        if (step < nsteps && ltid < ROWS) {
           const int4 info = sInfo[step];
           const int key0 = info.x, n = info.y;
           const int first_rel = causal ? key0 - off - m0 : -0x40000000;  // rows before it see no key of the block
           const int rel = rr - m0;
-          if ((ltid < n) & ((uint32_t)rel < (uint32_t)rows_sb) & (rel >= first_rel)) sPos[(step % 3) * kDqRows + rel] = ((tag_base + step + 1) << 8) | ltid;
+          if ((ltid < n) & ((uint32_t)rel < (uint32_t)rows_sb) & (rel >= first_rel)) sPos[(step % 3) * ROWS + rel] = ((tag_base + step + 1) << 8) | ltid;
         }
       };
       // K of `step`, row ids of `step + 2`
@@ -858,19 +861,23 @@ __global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmob
     }
     __syncthreads();  // the compute waves are done with the K tiles
   } else {
-    f32x16 acc[NDT];
+    f32x16 acc[RT][NDT];
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
-    const int myrow = wave * 32 + (lane & 31);
+      for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[rt][dt][i] = 0.f;
+    int myrow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) myrow[rt] = (wave * RT + rt) * 32 + (lane & 31);
     int tag_base = 0;
-    Pack8 df[NR][4];   // this lane's dS row of NR consecutive steps (B operands)
-    bool dfp[NR];
+    Pack8 df[NR][RT][4];   // this lane's dS rows of NR consecutive steps (B operands)
+    bool dfp[NR][RT];
     for (int cb = 0; cb < ncols; cb += cols_per_batch) {
       const int nsteps = prepare_batch(cb, min(ncols, cb + cols_per_batch));
       if (nsteps == 0) continue;
-      // fetch this lane's dS row of `step` into ring entry R (unconditional: an absent row reads position 0)
+      // fetch this lane's dS rows of `step` into ring entry R (unconditional: an absent row reads position 0)
       auto fetch = [&](auto rc, int step) {
         constexpr int R = decltype(rc)::value;
         const int sc_ = min(step, nsteps - 1);
@@ -878,25 +885,32 @@ __global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmob
         const int key0 = __builtin_amdgcn_readfirstlane(info.x);
         const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
         const int koff = key0 - (key0 / Bn) * Bn;
-        const int v = sPos[(sc_ % 3) * kDqRows + myrow];
-        const bool pres = (step < nsteps) & ((v >> 8) == tag_base + sc_ + 1);
-        const uint32_t j = pres ? (uint32_t)(v & 255) : 0u;
         const uint16_t *rp = ds_ws + pos0 * Bn + koff + 8 * hh;
 #pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) df[R][s4] = ld_global16(rp + j * (uint32_t)Bn + 16 * s4);
-        dfp[R] = pres;
+        for (int rt = 0; rt < RT; ++rt) {
+          const int v = sPos[(sc_ % 3) * ROWS + myrow[rt]];
+          const bool pres = (step < nsteps) & ((v >> 8) == tag_base + sc_ + 1);
+          const uint32_t j = pres ? (uint32_t)(v & 255) : 0u;
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4) df[R][rt][s4] = ld_global16(rp + j * (uint32_t)Bn + 16 * s4);
+          dfp[R][rt] = pres;
+        }
       };
       auto compute = [&](auto rc, int step) {
         constexpr int R = decltype(rc)::value;
-        const bool present = dfp[R];
-        if (!__any(present)) return;
-        Pack8 dz[4];
+        bool anyp = false;
 #pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4)
+        for (int rt = 0; rt < RT; ++rt) anyp |= dfp[R][rt];
+        if (!__any(anyp)) return;
+        Pack8 dz[RT][4];
 #pragma unroll
-          for (int w = 0; w < 4; ++w) dz[s4].w[w] = present ? df[R][s4].w[w] : 0u;
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) dz[rt][s4].w[w] = dfp[R][rt] ? df[R][rt][s4].w[w] : 0u;
         lds_cu16 *trK = tr_lane_base(sK + (size_t)(step & 1) * 64 * LDQ, LDQ, lane) + 8 * hh * LDQ;
-        // K^T operands half a feature tile (two products) ahead of their use
+        // K^T operands half a feature tile (two products per row tile) ahead of their use
         Pack8 kf[2][2];
         auto kread = [&](int u, Pack8 (&dst)[2]) {  // unit u: feature tile u / 2, keys 32 (u % 2) .. + 31
           const int dt = u >> 1, sb = 2 * (u & 1);
@@ -908,7 +922,9 @@ __global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmob
         for (int u = 0; u < 2 * NDT; ++u) {
           if (u + 1 < 2 * NDT) kread(u + 1, kf[(u + 1) & 1]);
 #pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) acc[u >> 1] = mfma32<T>(kf[u & 1][s2], dz[2 * (u & 1) + s2], acc[u >> 1]);
+          for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) acc[rt][u >> 1] = mfma32<T>(kf[u & 1][s2], dz[rt][2 * (u & 1) + s2], acc[rt][u >> 1]);
           __builtin_amdgcn_sched_barrier(0);
         }
       };
@@ -924,26 +940,28 @@ __global__ __launch_bounds__(512, HD > 128 ? 2 : 4) void attn_bwd_dq_kernel(fmob
         });
       tag_base += nsteps;
     }
-    __syncthreads();  // every wave is done with the K tiles: they now hold the output tiles
+    __syncthreads();  // every wave is done with the K tiles: they now hold the output tiles (one 32-row tile per wave)
     uint16_t *sOut = reinterpret_cast<uint16_t *>(smem + SM::oK) + (size_t)wave * 32 * LDO;
+    uint16_t *op = reinterpret_cast<uint16_t *>(a.dq) + (int64_t)(q0 + m0) * a.dq_row_stride + (int64_t)h * a.dq_head_stride;
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
+    for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
-        *reinterpret_cast<uint2 *>(sOut + (lane & 31) * LDO + dt * 32 + 8 * g + 4 * hh) =
-            make_uint2(pack2<T>(acc[dt][4 * g] * a.softmax_scale, acc[dt][4 * g + 1] * a.softmax_scale),
-                       pack2<T>(acc[dt][4 * g + 2] * a.softmax_scale, acc[dt][4 * g + 3] * a.softmax_scale));
-    wave_lds_fence();
-    {
-      uint16_t *op = reinterpret_cast<uint16_t *>(a.dq) + (int64_t)(q0 + m0) * a.dq_row_stride + (int64_t)h * a.dq_head_stride;
+      for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          *reinterpret_cast<uint2 *>(sOut + (lane & 31) * LDO + dt * 32 + 8 * g + 4 * hh) =
+              make_uint2(pack2<T>(acc[rt][dt][4 * g] * a.softmax_scale, acc[rt][dt][4 * g + 1] * a.softmax_scale),
+                         pack2<T>(acc[rt][dt][4 * g + 2] * a.softmax_scale, acc[rt][dt][4 * g + 3] * a.softmax_scale));
+      wave_lds_fence();
       // rows leave as 16-byte pieces, VPR of them per row, consecutive lanes taking consecutive pieces
 #pragma unroll
       for (int v0 = 0; v0 < 32 * VPR; v0 += 64) {
         const int v = v0 + lane, rl = v / VPR, e = (v - rl * VPR) * 8;
-        const int r2 = wave * 32 + rl;
+        const int r2 = (wave * RT + rt) * 32 + rl;
         if (r2 < rows_sb && e < D)
           *reinterpret_cast<Pack8 *>(op + (int64_t)r2 * a.dq_row_stride + e) = *reinterpret_cast<const Pack8 *>(sOut + rl * LDO + e);
       }
+      wave_lds_fence();
     }
   }
 }
@@ -1070,15 +1088,15 @@ static int launch_dkdv(const fmoba_attn_bwd_args &a, const BwdWs &ws, hipStream_
   return 0;
 }
 
-template <typename T, int HD>
+template <typename T, int HD, int RT>
 static int launch_dq(const fmoba_attn_bwd_args &a, const uint16_t *ws, hipStream_t s) {
-  auto kern = attn_bwd_dq_kernel<T, HD>;
+  auto kern = attn_bwd_dq_kernel<T, HD, RT>;
   const size_t smem = DqSmem<HD>::bytes;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("attn_bwd: cannot reserve %zu bytes of LDS", smem);
     return 2;
   }
-  const int nsb_max = ceil_div(a.max_seqlen_q, kDqRows);
+  const int nsb_max = ceil_div(a.max_seqlen_q, kDqRows * RT);
   const int64_t items = (int64_t)a.heads * a.batch * nsb_max;
   if (items >= ((int64_t)1 << 31)) {
     set_error("attn_bwd: too many (sequence, head, superblock) work items");
@@ -1129,7 +1147,7 @@ static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hi
     if (phases & FMOBA_BWD_DKDV)
       if (int rc = run_bwd_dkdv_wide(a, ws.ds, s)) return rc;
     if (phases & FMOBA_BWD_DQ)
-      if (int rc = launch_dq<T, 256>(a, ws.ds, s)) return rc;
+      if (int rc = launch_dq<T, 256, 1>(a, ws.ds, s)) return rc;
     return 0;
   }
   if (phases & FMOBA_BWD_DKDV) {
@@ -1156,7 +1174,7 @@ static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hi
       }
       hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 15) / 16)), dim3(256), smem, s, a, ws, capl);
     } else {
-      int rc = a.head_dim <= 64 ? launch_dq<T, 64>(a, ws.ds, s) : launch_dq<T, 128>(a, ws.ds, s);
+      int rc = a.head_dim <= 64 ? launch_dq<T, 64, 1>(a, ws.ds, s) : launch_dq<T, 128, 2>(a, ws.ds, s);
       if (rc) return rc;
     }
   }
