@@ -760,11 +760,14 @@ __global__ __launch_bounds__(64) void csc_fill_kernel(TopkParams p) {
 
 // ------------------------------------------------------------------------------------
 // ordered per-row lists (indices / values), only produced on request: one wave per
-// (row, head); plain FMA scores, then topk rounds of wave-wide arg-max under the total
-// order (score desc, chunk desc).
+// (row, head).  The SET of chunks is the gate's own (its selection bits: the lists name
+// exactly the chunks whose columns hold the row, also where two scores are so close that
+// another summation order would rank them the other way round); the scores that order the
+// set are plain FMA sums, then rounds of wave-wide arg-max under the total order (score
+// desc, chunk desc).
 // ------------------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(64) void topk_raw_kernel(fmoba_fused_topk_args a, int kr) {
+__global__ __launch_bounds__(64) void topk_raw_kernel(fmoba_fused_topk_args a, int kr, const uint32_t *sel, int W) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float *sScore = reinterpret_cast<float *>(smem);  // [Cpad]
   const int row_g = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -789,10 +792,15 @@ __global__ __launch_bounds__(64) void topk_raw_kernel(fmoba_fused_topk_args a, i
   int nc = a.is_causal ? (rp >= 0 ? min(rp / a.chunk, Cb) : 0) : Cb;
   const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)row_g * a.q_row_stride + (int64_t)h * a.q_head_stride;
   const uint16_t *kmp = reinterpret_cast<const uint16_t *>(a.km) + (int64_t)hk * a.km_head_stride;
+  const uint32_t *selrow = sel + (int64_t)h * W * a.total_q + row_g;
   for (int c = lane; c < nc; c += 64) {
-    float s = 0.f;
-    const uint16_t *kr_ = kmp + (int64_t)(km0 + c) * a.km_row_stride;
-    for (int d = 0; d < a.head_dim; ++d) s = fmaf(elem_to_float<T>(qp[d]), elem_to_float<T>(kr_[d]), s);
+    float s = -INFINITY;  // (chunks the gate did not select never enter the lists)
+    if ((c >> 5) < W && ((selrow[(int64_t)(c >> 5) * a.total_q] >> (c & 31)) & 1u)) {
+      s = 0.f;
+      const uint16_t *kr_ = kmp + (int64_t)(km0 + c) * a.km_row_stride;
+      for (int d = 0; d < a.head_dim; ++d) s = fmaf(elem_to_float<T>(qp[d]), elem_to_float<T>(kr_[d]), s);
+      if (s == -INFINITY) s = -3.4028234663852886e38f;  // a selected chunk keeps its place in the list
+    }
     sScore[c] = s;
   }
   __syncthreads();
@@ -1004,9 +1012,9 @@ static int fused_topk_run(const fmoba_fused_topk_args *a, void *workspace, size_
     const size_t smem = (size_t)(max_cols + 64) * 4;
     dim3 rgrid(a->total_q, a->heads);
     if (a->dtype == FMOBA_DTYPE_BF16)
-      hipLaunchKernelGGL(topk_raw_kernel<bf16_t>, rgrid, dim3(64), smem, s, *a, kr);
+      hipLaunchKernelGGL(topk_raw_kernel<bf16_t>, rgrid, dim3(64), smem, s, *a, kr, p.sel, p.W);
     else
-      hipLaunchKernelGGL(topk_raw_kernel<f16_t>, rgrid, dim3(64), smem, s, *a, kr);
+      hipLaunchKernelGGL(topk_raw_kernel<f16_t>, rgrid, dim3(64), smem, s, *a, kr, p.sel, p.W);
     FMOBA_LAUNCH_CHECK("topk_raw_kernel");
   }
   return 0;

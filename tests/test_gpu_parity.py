@@ -136,6 +136,17 @@ def _check_gating(fm, q, k, cuq, cuk, chunk, topk, causal, integer=False):
     if integer:
         assert torch.equal(indices.cpu(), idx_ref)
         assert torch.equal(values.cpu(), val_ref)
+    # the ordered lists name exactly the chunks whose columns hold the row, near-ties included (one selection feeds both)
+    ic = indices.cpu().numpy()
+    cuq_np = cuq.numpy()
+    for b in range(len(cuq_np) - 1):
+        s0, Lq = int(cuq_np[b]), int(cuq_np[b + 1] - cuq_np[b])
+        for h in range(H):
+            got = selection_sets(co, cn, flat, b, h, Lq, maxC)
+            raw = np.zeros_like(got)
+            rows, slots = np.nonzero(ic[s0:s0 + Lq, h] >= 0)
+            raw[rows, ic[s0:s0 + Lq, h][rows, slots]] = True
+            assert (raw == got).all(), (b, h)
 
 
 @pytest.mark.parametrize("topk", [1, 2, 4, 8, 16, 24, 32, 33, 64])
