@@ -189,8 +189,9 @@ int fmoba_attn_fwd_phases(const fmoba_attn_fwd_args *a, int32_t phases, void *st
  *   dK/dV come from one column-stationary pass.  dQ has two forms (dq_mode: 0 = the library
  *   chooses, 1 = row blocks, 2 = partials; fmoba_attn_bwd_uses_partials() tells the choice):
  *     row blocks: the dK/dV pass leaves the dS tiles (16-bit, lg_block_n entries per entry of
- *       row_indices) in the workspace and a row-stationary pass (128 query rows per workgroup,
- *       accumulators in LDS) multiplies them with K;
+ *       row_indices) in the workspace and a row-stationary pass (128 or 256 query rows per
+ *       workgroup, accumulators in registers) multiplies them with K; the only form for
+ *       head_dim > 128;
  *     partials: the dK/dV pass leaves one dQ partial row (16-bit) per visit of a (query row,
  *       key block) pair, a second launch adds the partials of each row in key order.  This is
  *       the form that scales when sequences have thousands of chunks.  (Key blocks have 128 keys
