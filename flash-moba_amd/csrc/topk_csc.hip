@@ -667,6 +667,457 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
   }
 }
 
+// ------------------------------------------------------------------------------------
+// The grouped gate for at most 16 running winners per row (top-k up to 17 causal, 16 otherwise): the common case of
+// long sequences.  Same total order and result as topk_gate_big_kernel; what differs is where things live:
+//  * a row's winners stay in REGISTERS across the groups: eight doubles per lane of the row's lane pair, each lane's
+//    share sorted, so that the weakest is at hand and a new winner goes in with one pass of minimum / maximum;
+//  * the chunk means of the next group are fetched into registers while the current group is worked on;
+//  * the scores of a later group that reach the row's weakest winner ("entrants") are compacted into one list per
+//    row in LDS -- the lane with chunks 0..3 of every eight fills it from the bottom, its partner from the top, so
+//    that no counter is shared; every score is stored at the lane's next slot and the slot advances only for an
+//    entrant, so there are no branches and no address selects -- and each then replaces the weakest winner if it
+//    beats it.  More than 16 entrants in some row of a wave, the first group, and rows whose list is not full yet
+//    take the bisection over this group's scores and the winners.
+// ------------------------------------------------------------------------------------
+// A winner is ONE double: order key of its score * 8192 + chunk (exact: below 2^45), so that the order "score
+// descending, chunk descending" is the order of the doubles and minimum / maximum are single instructions.
+constexpr double kChunkSpan = 8192.0;   // more chunks per sequence than the LDS of these kernels can hold anyway
+constexpr double kSlotFiller = INFINITY;  // unused slot of a complete list: above every winner, never the weakest
+constexpr double kSlotEmpty = -1.0;       // unused slot of a list that is still filling: below every winner
+
+__device__ __forceinline__ double winner_word(float score, int chunk) {
+  // (x + 0 turns -0 into +0: the order keys must agree with the float compares of the bisection)
+  return fma((double)float_order_key(score + 0.f), kChunkSpan, (double)chunk);
+}
+__device__ __forceinline__ bool winner_real(double w) { return w >= 0.0 && w < (double)INFINITY; }
+__device__ __forceinline__ uint32_t winner_key(double w) { return (uint32_t)(w * (1.0 / kChunkSpan)); }  // (truncates)
+__device__ __forceinline__ int winner_chunk(double w) { return (int)fma(-(double)winner_key(w), kChunkSpan, w); }
+__device__ __forceinline__ double shfl_xor32_d(double v) {
+  const uint64_t u = (uint64_t)__double_as_longlong(v);
+  const uint64_t o = ((uint64_t)(uint32_t)shfl_xor32_i((int)(u >> 32)) << 32) | (uint32_t)shfl_xor32_i((int)(uint32_t)u);
+  return __longlong_as_double((long long)o);
+}
+
+// a * b + c on 24-bit operands, one instruction (the compiler picks a 64-bit multiply-add for this address pattern)
+__device__ __forceinline__ uint32_t mad24_u32(int a, int b, uint32_t c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  uint32_t d;
+  asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+  return d;
+#else
+  return (uint32_t)(a * b) + c;
+#endif
+}
+// n + (x >= y): the compare and an add with carry (left alone, the compiler materialises the flag as 0 / 1 first)
+__device__ __forceinline__ int count_if_ge(int n, float x, float y) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm("v_cmp_ge_f32 vcc, %1, %2\n\ts_nop 1\n\tv_addc_co_u32 %0, vcc, 0, %0, vcc" : "+v"(n) : "v"(x), "v"(y) : "vcc");
+  return n;
+#else
+  return n + (x >= y ? 1 : 0);
+#endif
+}
+
+template <typename T, int HD, int NT>
+__global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(TopkParams p) {
+  constexpr int CAP = 16, PL = 8;
+  constexpr int KS = HD / 16;
+  constexpr int LD = HD + 16;
+  constexpr int GC = NT * 32;             // chunks per group
+  constexpr int VPR = HD / 8;             // 16-byte pieces of a row of chunk means
+  constexpr int NV = GC * VPR / 256;      // ... of a group's tile per thread
+  static_assert(GC * VPR % 256 == 0, "the tile is loaded in whole passes of the workgroup");
+  constexpr int LS = CAP + 2;                 // slots of a row's list: 16 entries and the two lanes' next slots
+  constexpr int EW = kGateRows * LS + 256;    // words of an entrant array: the lists, then a trash word per thread
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint16_t *sKm = reinterpret_cast<uint16_t *>(smem);
+  uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [W][128], reuses the tile and the lists after the last group
+  float *sEv = reinterpret_cast<float *>(smem + (size_t)GC * LD * 2);  // [EW] scores of the entrants
+  const size_t head = max((size_t)GC * LD * 2 + (size_t)2 * EW * 4, (size_t)p.W * kGateRows * 4);
+  int *sHist = reinterpret_cast<int *>(smem + head);                   // [max_cols]
+
+  const fmoba_fused_topk_args &a = p.a;
+  const int mb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int q0 = a.cu_seqlens_q[b];
+  const int Lq = a.cu_seqlens_q[b + 1] - q0;
+  const int m0 = mb * kGateRows;
+  if (m0 >= Lq) return;
+  const int Lk = a.cu_seqlens_k[b + 1] - a.cu_seqlens_k[b];
+  const int km0 = a.cu_seqlens_km[b];
+  const int Cb = min(a.cu_seqlens_km[b + 1] - km0, p.max_cols);
+  const int off = Lk - Lq;
+  const int B = a.chunk;
+  const int D = a.head_dim;
+  const int hk = h / (a.heads / a.heads_k);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
+  const int rs = wave * 32 + (lane & 31);  // row slot inside the block
+
+  int nsc;  // chunks [0, nsc) can be candidates of some row of this block
+  if (a.is_causal) {
+    const int rmax = min(m0 + kGateRows - 1, Lq - 1) + off;
+    nsc = rmax < 0 ? 0 : min(Cb, rmax / B);
+  } else {
+    nsc = Cb;
+  }
+  const int ngroups = (nsc + GC - 1) / GC;
+
+  const int r = m0 + rs;
+  const bool valid = r < Lq;
+  Pack8 qf[KS];
+  {
+    const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + (int64_t)(q0 + (valid ? r : 0)) * a.q_row_stride + (int64_t)h * a.q_head_stride;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int e = (hh * KS + ks) * 8;
+      qf[ks] = (valid && e < D) ? ld_global16(qp + e) : zero_pack8();
+    }
+  }
+  const int rp = r + off;
+  int nc;  // candidate chunks of this row: chunks strictly before its own chunk
+  if (a.is_causal)
+    nc = (valid && rp >= 0) ? min(rp / B, Cb) : 0;
+  else
+    nc = valid ? Cb : 0;
+  const int kp = a.is_causal ? a.topk - 1 : a.topk;
+
+  const uint16_t *kmp = reinterpret_cast<const uint16_t *>(a.km) + (int64_t)hk * a.km_head_stride;
+  Pack8 pre[NV];
+  auto fetch = [&](int g) {
+    const int c0 = g * GC, gsc = min(GC, nsc - c0);
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int x = tid + v * 256, c = x / VPR, e = (x - c * VPR) * 8;
+      pre[v] = (c < gsc && e < D) ? ld_global16(kmp + (int64_t)(km0 + c0 + c) * a.km_row_stride + e) : zero_pack8();
+    }
+  };
+  double win[PL];  // this lane's share of the row's winners, ascending (win[0] is the weakest the lane holds)
+#pragma unroll
+  for (int j = 0; j < PL; ++j) win[j] = kSlotEmpty;
+  int m_prev = 0;    // winners the row holds
+  float *const my_list_v = sEv + rs * LS;
+  float *const my_trash = sEv + kGateRows * LS + tid;
+  constexpr int kToIdx = EW;  // from a score of the entrant arrays to its chunk, in words
+
+  if (ngroups > 0) fetch(0);
+#pragma nounroll
+  for (int g = 0; g < ngroups; ++g) {
+    const int c0 = g * GC;
+    const int gsc = min(GC, nsc - c0);
+    const int n_tiles = (gsc + 31) >> 5;
+    __syncthreads();  // the previous group's tile is no longer read
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int x = tid + v * 256, c = x / VPR, e = (x - c * VPR) * 8;
+      *reinterpret_cast<Pack8 *>(sKm + c * LD + e) = pre[v];
+    }
+    if (g + 1 < ngroups) fetch(g + 1);
+    __syncthreads();
+
+    // this group's scores; chunks that are no candidates of the row (its own chunk and later ones) count as -inf
+    float sc[NT][16];
+    const bool all_cand = __all(nc >= c0 + GC);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (t < n_tiles) {
+        f32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const Pack8 af = *reinterpret_cast<const Pack8 *>(sKm + (t * 32 + (lane & 31)) * LD + (hh * KS + ks) * 8);
+          acc = mfma32<T>(af, qf[ks], acc);
+        }
+        if (all_cand) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sc[t][i] = acc[i];
+        } else {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sc[t][i] = (c0 + t * 32 + acc_row(i, hh) < nc) ? acc[i] : -INFINITY;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[t][i] = -INFINITY;
+      }
+    }
+
+    // ---- later groups: streaming update ---------------------------------------------------------
+    // A row that still has candidates in this group had at least GC of them in the first one, so it already holds
+    // kp winners.  Only the new scores that reach its weakest winner can enter (a new chunk has a higher index than
+    // every earlier one, so an equal score wins the tie).
+    bool streamed = false;
+    if (g > 0 && __all(m_prev == kp || nc <= c0)) {
+      const double weakest = fmin(win[0], shfl_xor32_d(win[0]));
+      // (a row without winners, or one whose list is not full because it has no candidates left, admits nothing)
+      const float pmin = winner_real(weakest) ? order_key_float(winner_key(weakest)) : INFINITY;
+      // slot c of the lane with chunks 0..3 is entry c, of its partner entry LS - 1 - c; beyond the list both stay
+      // on the row's last slot
+      const uint32_t slot0 = (uint32_t)(uintptr_t)(my_list_v + (hh ? LS - 1 : 0));
+      const int slot_step = hh ? -4 : 4;  // bytes
+      int cbase = c0 + 4 * hh;
+      asm volatile("" : "+v"(cbase));  // (one register: the compiler would add its scalar and vector parts per position)
+      int cnt = 0;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            // (before position LS - 1 the lane cannot have that many entrants)
+            const uint32_t d = mad24_u32(t * 16 + i < LS - 1 ? cnt : min(cnt, LS - 1), slot_step, slot0);
+            lds_write_vec<float>(d, sc[t][i]);
+            lds_write_vec<int>(d + (uint32_t)kToIdx * 4u, cbase + t * 32 + 8 * (i >> 2) + (i & 3));
+            cnt = count_if_ge(cnt, sc[t][i], pmin);
+          }
+        }
+      const int cnt_o = shfl_xor32_i(cnt);
+      const int ne_row = cnt + cnt_o;
+      if (__all(ne_row <= CAP)) {
+        wave_lds_fence();
+        const int ne_lo = hh ? cnt_o : cnt;  // entrants that came from the bottom of the list
+        auto stream = [&](auto plc) {
+          constexpr int PLX = decltype(plc)::value;
+#pragma nounroll
+          for (int e = 0; __any(e < ne_row); ++e) {
+            const bool has = e < ne_row;
+            const int at = has ? (e < ne_lo ? e : LS - 1 - (e - ne_lo)) : 0;
+            const double x = winner_word(my_list_v[at], reinterpret_cast<const int *>(my_list_v)[kToIdx + at]);
+            // the row's weakest winner is the lower of the two lanes' first entries; the lane that holds it drops it
+            // and passes the entrant up its sorted entries (a lane that keeps its entries passes its own first entry)
+            const double vo = shfl_xor32_d(win[0]);
+            const bool rep = has & (win[0] <= vo) & (x > win[0]);
+            const double xs = rep ? x : win[0];
+            double nw[PLX];
+            nw[0] = fmin(xs, win[1]);
+#pragma unroll
+            for (int j = 1; j + 1 < PLX; ++j) nw[j] = fmin(fmax(win[j], xs), win[j + 1]);
+            nw[PLX - 1] = fmax(win[PLX - 1], xs);
+#pragma unroll
+            for (int j = 0; j < PLX; ++j) win[j] = nw[j];
+          }
+        };
+        // (a lane holds at most (kp + 1) / 2 winners; the fillers above them never move)
+        if (kp <= PL)
+          stream(std::integral_constant<int, PL / 2>{});
+        else
+          stream(std::integral_constant<int, PL>{});
+        wave_lds_fence();  // (the list takes the next entrants)
+        streamed = true;
+      }
+    }
+    if (streamed) continue;
+
+    // ---- first group, lists that are filling, too many entrants: bisection over scores and winners ------------
+    float pv[PL];
+    int pi[PL];
+    float vmin = INFINITY, vmax = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PL; ++j) {
+      const bool ok = winner_real(win[j]);
+      pv[j] = ok ? order_key_float(winner_key(win[j])) : -INFINITY;
+      pi[j] = ok ? winner_chunk(win[j]) : -1;
+      vmin = fminf(vmin, ok ? pv[j] : INFINITY);
+      vmax = fmaxf(vmax, pv[j]);
+    }
+    // A full list bounds the search from below: its kp winners all reach its weakest one, so the new threshold cannot
+    // lie below that score (if nothing enters, the search closes on it and the tie rule keeps the list as it is).
+    const float floor_v = (m_prev == kp && kp > 0) ? min_xor32_f(vmin) : -INFINITY;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      if (t < n_tiles) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const bool cand = c0 + t * 32 + acc_row(i, hh) < nc;
+          vmin = fminf(vmin, cand ? sc[t][i] : INFINITY);
+          vmax = fmaxf(vmax, sc[t][i]);
+        }
+      }
+    vmin = min_xor32_f(vmin);
+    vmax = max_xor32_f(vmax);
+    const int ntot = m_prev + max(0, min(nc - c0, GC));  // candidates that compete in this group
+    const bool need = (ntot > kp) && (kp > 0);
+
+    auto count_gt = [&](float probe) {
+      int cnt = 0;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) cnt += (sc[t][i] > probe) ? 1 : 0;
+        }
+#pragma unroll
+      for (int j = 0; j < PL; ++j) cnt += (pv[j] > probe) ? 1 : 0;
+      return sum_xor32_i(cnt);
+    };
+    float tau = -INFINITY, tau_eq = INFINITY;
+    int n_eq = 0;
+    uint32_t iota = 0u;
+    {
+      uint32_t lo_k = float_order_key(fmaxf(vmin, floor_v)) - 1u;
+      uint32_t hi_k = float_order_key(vmax);
+      int c_hi = 0;
+      bool open = need;
+#pragma nounroll
+      for (int iter = 0;; ++iter) {
+        if (open && hi_k - lo_k <= 1u) {
+          tau = order_key_float(hi_k);
+          if (tau != -INFINITY) {
+            tau_eq = tau;
+            n_eq = kp - c_hi;
+          }
+          open = false;
+        }
+        if (!__any(open)) break;
+        uint32_t pk = lo_k + ((hi_k - lo_k) >> 1);
+        if (iter < 12) {
+          const float mf = 0.5f * order_key_float(lo_k + 1u) + 0.5f * order_key_float(hi_k);
+          const uint32_t mk = float_order_key(mf);
+          if (mk > lo_k && mk < hi_k) pk = mk;
+        }
+        const float probe = order_key_float(pk);
+        const int cnt = count_gt(probe);
+        if (open) {
+          if (cnt == kp) {
+            tau = probe;
+            open = false;
+          } else if (cnt > kp) {
+            lo_k = pk;
+          } else {
+            hi_k = pk;
+            c_hi = cnt;
+          }
+        }
+      }
+      const bool tie = n_eq > 0;
+      if (__any(tie)) {
+        auto count_eq_ge = [&](uint32_t trial) {
+          int cnt = 0;
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            if (t < n_tiles) {
+#pragma unroll
+              for (int i = 0; i < 16; ++i) {
+                const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
+                cnt += ((sc[t][i] == tau_eq) & (c >= trial)) ? 1 : 0;
+              }
+            }
+#pragma unroll
+          for (int j = 0; j < PL; ++j) cnt += ((pv[j] == tau_eq) & ((uint32_t)pi[j] >= trial) & (pi[j] >= 0)) ? 1 : 0;
+          return sum_xor32_i(cnt);
+        };
+        const int ceq = count_eq_ge(0u);
+        const bool split = tie && ceq > n_eq;
+        if (__any(split)) {
+          uint32_t i_acc = 0u;
+#pragma nounroll
+          for (int bit = 23; bit >= 0; --bit) {
+            const uint32_t trial = i_acc | (1u << bit);
+            const int cnt = count_eq_ge(trial);
+            if (cnt >= n_eq) i_acc = trial;
+          }
+          if (split) iota = i_acc;
+        }
+      }
+    }
+
+    // the winners of this round go through the row's LDS list (densely: the partner lane starts where this one ends)
+    // and come back as alternate entries per lane
+    int nwin = 0;
+    if (kp > 0) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
+            const float x = sc[t][i];
+            nwin += ((x > tau) | ((x == tau_eq) & (c >= iota))) ? 1 : 0;
+          }
+        }
+#pragma unroll
+      for (int j = 0; j < PL; ++j) nwin += ((pi[j] >= 0) & ((pv[j] > tau) | ((pv[j] == tau_eq) & ((uint32_t)pi[j] >= iota)))) ? 1 : 0;
+    }
+    const int nwin_o = shfl_xor32_i(nwin);
+    const int m_new = min(nwin + nwin_o, CAP);
+    int slot = hh ? nwin_o : 0;
+    if (__any(nwin > 0)) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const uint32_t c = (uint32_t)(c0 + t * 32 + acc_row(i, hh));
+            const float x = sc[t][i];
+            const bool w = (kp > 0) & ((x > tau) | ((x == tau_eq) & (c >= iota))) & (slot < CAP);
+            float *d = w ? my_list_v + slot : my_trash;
+            d[0] = x;
+            reinterpret_cast<int *>(d)[kToIdx] = (int)c;
+            slot += w ? 1 : 0;
+          }
+        }
+#pragma unroll
+      for (int j = 0; j < PL; ++j) {
+        const bool w = (kp > 0) & (pi[j] >= 0) & ((pv[j] > tau) | ((pv[j] == tau_eq) & ((uint32_t)pi[j] >= iota))) & (slot < CAP);
+        float *d = w ? my_list_v + slot : my_trash;
+        d[0] = pv[j];
+        reinterpret_cast<int *>(d)[kToIdx] = pi[j];
+        slot += w ? 1 : 0;
+      }
+    }
+    wave_lds_fence();
+#pragma unroll
+    for (int j = 0; j < PL; ++j) {
+      const int e = 2 * j + hh;
+      const bool ok = e < m_new;
+      const double x = winner_word(my_list_v[ok ? e : 0], reinterpret_cast<const int *>(my_list_v)[kToIdx + (ok ? e : 0)]);
+      win[j] = ok ? x : (m_new == kp ? kSlotFiller : kSlotEmpty);
+    }
+    wave_lds_fence();  // (the list takes this row's entrants next)
+    // each lane's share in ascending order (odd-even transposition: this path runs once or twice per row)
+#pragma unroll
+    for (int rnd = 0; rnd < PL; ++rnd)
+#pragma unroll
+      for (int j = rnd & 1; j + 1 < PL; j += 2) {
+        const double lo = fmin(win[j], win[j + 1]), hi = fmax(win[j], win[j + 1]);
+        win[j] = lo;
+        win[j + 1] = hi;
+      }
+    m_prev = m_new;
+  }
+  __syncthreads();
+
+  // selection words and per-chunk counts of the block, assembled in LDS
+  for (int v = tid; v < p.W * kGateRows; v += 256) sSel[v] = 0u;
+  for (int c = tid; c < p.max_cols; c += 256) sHist[c] = 0;
+  __syncthreads();
+  if (valid) {
+#pragma unroll
+    for (int j = 0; j < PL; ++j) {
+      if (winner_real(win[j])) {
+        const uint32_t c = (uint32_t)winner_chunk(win[j]);
+        atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
+        atomicAdd(&sHist[c], 1);
+      }
+    }
+    if (hh == 0 && a.is_causal && rp >= 0) {
+      const int c = rp / B;  // the own chunk is always selected
+      if (c < p.max_cols) {
+        atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
+        atomicAdd(&sHist[c], 1);
+      }
+    }
+  }
+  __syncthreads();
+  for (int v = tid; v < p.W * kGateRows; v += 256) {
+    const int t = v / kGateRows, slot_r = v - t * kGateRows;
+    if (m0 + slot_r < Lq) p.sel[((int64_t)h * p.W + t) * a.total_q + q0 + m0 + slot_r] = sSel[v];
+  }
+  const int seg = m0 / p.seg_rows;
+  for (int c = tid; c < p.max_cols; c += 256) {
+    const int v = sHist[c];
+    if (v) atomicAdd(&p.segcnt[(((int64_t)b * a.heads + h) * p.nseg + seg) * p.max_cols + c], v);
+  }
+}
+
 // grid (heads, batch), block 256
 __global__ __launch_bounds__(256) void csc_scan_kernel(TopkParams p) {
   const fmoba_fused_topk_args &a = p.a;
@@ -905,21 +1356,43 @@ static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
   hipLaunchKernelGGL(kern, grid, dim3(256), smem, s, p);
   return 0;
 }
+template <int HD, int NT>
+static size_t gate_stream_smem(const TopkParams &p) {
+  const size_t lists = (size_t)2 * (kGateRows * 18 + 256) * 4;
+  return std::max((size_t)NT * 32 * (HD + 16) * 2 + lists, (size_t)p.W * kGateRows * 4) + (size_t)p.max_cols * 4;
+}
+template <typename T, int HD, int NT>
+static int launch_gate_stream(const TopkParams &p, dim3 grid, hipStream_t s) {
+  const size_t smem = gate_stream_smem<HD, NT>(p);
+  if (smem > 160 * 1024 || p.max_cols > (int)kChunkSpan) {  // (the second follows from the first; the winners' encoding relies on it)
+    set_error("fused_topk: %d key chunks per sequence exceed what the LDS of this build holds", p.max_cols);
+    return 1;
+  }
+  auto kern = topk_gate_stream_kernel<T, HD, NT>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+    set_error("fused_topk: cannot reserve %zu bytes of LDS", smem);
+    return 2;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), smem, s, p);
+  return 0;
+}
 template <typename T>
 static int launch_gate_big_hd(const TopkParams &p, dim3 grid, hipStream_t s) {
-  // up to 16 running winners per row: short lists and groups of 128 chunks, if that lets two workgroups share a compute unit
+  // up to 16 running winners per row: the kernel that keeps them in registers, in groups of 64 chunks (three workgroups
+  // per compute unit; with groups of 128 and two workgroups it took 6.4 ms instead of 5.1 at 262144 tokens)
   const int kp = p.a.is_causal ? p.a.topk - 1 : p.a.topk;
   if (p.a.head_dim <= 64) {
     if (kp > kBigCap) return launch_gate_big<T, 64, 4, kBigCapMax>(p, grid, s);
-    if (kp <= 16 && gate_big_smem<64, 4, 16>(p) <= 80 * 1024) return launch_gate_big<T, 64, 4, 16>(p, grid, s);
+    if (kp <= 16) return launch_gate_stream<T, 64, 2>(p, grid, s);
     return launch_gate_big<T, 64, 8, kBigCap>(p, grid, s);
   }
   if (p.a.head_dim <= 128) {
     if (kp > kBigCap) return launch_gate_big<T, 128, 4, kBigCapMax>(p, grid, s);
-    if (kp <= 16 && gate_big_smem<128, 4, 16>(p) <= 80 * 1024) return launch_gate_big<T, 128, 4, 16>(p, grid, s);
+    if (kp <= 16) return launch_gate_stream<T, 128, 2>(p, grid, s);
     return launch_gate_big<T, 128, 8, kBigCap>(p, grid, s);
   }
   if (kp > kBigCap) return launch_gate_big<T, 256, 2, kBigCapMax>(p, grid, s);
+  if (kp <= 16) return launch_gate_stream<T, 256, 2>(p, grid, s);
   return launch_gate_big<T, 256, 4, kBigCap>(p, grid, s);
 }
 template <typename T>
