@@ -257,11 +257,16 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
         "attn_fwd": {"ms": t_fwd, "TFLOPs": fwd_flops / t_fwd / 1e9, "frac_mfma": fwd_flops / t_fwd / 1e9 / PEAK_BF16_TFLOPS,
                      "phases_ms": fwd_phase_ms},
     }
+    # Compulsory HBM bytes of a launch: every tensor once, plus what the form of the kernel writes or reads per list
+    # entry (partial results, dS tiles); rows that a kernel gathers again per visit count once.
+    entries = int(cn.sum().item())
+    qkv_once = T * H * D * 2
+    fwd_visits = entries * (chunk // hip.fwd_key_block(chunk))
     # one kernel runs both forward GEMMs: the row-block pass, or the column pass (its combine only merges partial rows)
     if row_blocks:
-        kernels = {"attn_fwd_rows_kernel": (fwd_phase_ms["row_blocks"], fwd_flops, "mfma")}
+        kernels = {"attn_fwd_rows_kernel": (fwd_phase_ms["row_blocks"], fwd_flops, 4 * qkv_once + T * H * ((maxC + 31) // 32) * 4)}
     else:
-        kernels = {"attn_fwd_col_kernel": (fwd_phase_ms["columns"], fwd_flops, "mfma")}
+        kernels = {"attn_fwd_col_kernel": (fwd_phase_ms["columns"], fwd_flops, 3 * qkv_once + fwd_visits * (D * 2 + 16))}
     if backward:
         dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
         phase_ms = {}
@@ -282,23 +287,35 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
         t_bwd = time_events(bwd, it)
         stages["attn_bwd"] = {"ms": t_bwd, "TFLOPs": bwd_flops / t_bwd / 1e9, "frac_mfma": bwd_flops / t_bwd / 1e9 / PEAK_BF16_TFLOPS,
                               "phases_ms": phase_ms}
-        # the dK/dV kernel runs four of the five backward GEMMs (S, dP, dV, dK); the fifth is in it as well when the
-        # library picks the partial-sum form of dQ (long sequences), else in the dQ kernel (this figure assumes the latter)
-        kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 8.0 * D * pairs, "mfma")
-        if not hip.last_bwd_partials():
-            kernels["attn_bwd_dq_kernel"] = (phase_ms["dq"], 2.0 * D * pairs, "mfma")
+        # the dK/dV kernel runs four of the five backward GEMMs (S, dP, dV, dK) and writes the dS tiles for the dQ
+        # kernel; when the library picks the partial-sum form of dQ (long sequences) the fifth GEMM is in it as well and
+        # it writes one dQ partial row per visit instead
+        if hip.last_bwd_partials():
+            bwd_kb = 128 if (chunk % 128 == 0 and D > 64) else 64
+            kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 10.0 * D * pairs, 6 * qkv_once + entries * (chunk // bwd_kb) * (D * 2 + 4))
+        else:
+            kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 8.0 * D * pairs, 6 * qkv_once + entries * chunk * 2)
+            kernels["attn_bwd_dq_kernel"] = (phase_ms["dq"], 2.0 * D * pairs, 2 * qkv_once + entries * chunk * 2)
     # sort alone, on the CSC the gating produced (already sorted input; same traffic)
     t_sort = time_events(lambda: torch.ops.flash_moba._varlen_sort(co, cn, ind), it)
     sort_bytes = 2 * int(cn.sum().item()) * 4 + 2 * cn.numel() * 8
     stages["varlen_sort"] = {"ms": t_sort, "GBps": sort_bytes / t_sort / 1e6, "frac_hbm": sort_bytes / t_sort / 1e6 / PEAK_HBM_GBS}
 
     # ---- roofline of the dominant kernel ---------------------------------------------------
+    # The bound is the roof that lies lower for this launch: the larger of flops / MFMA peak and bytes / HBM peak.
     dom = max(kernels, key=lambda n: kernels[n][0])
-    d_ms, d_flops, _ = kernels[dom]
-    roofline = {"kernel": dom, "bound": "mfma", "achieved": d_flops / d_ms / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get((name, dom)),
-                "traffic_unit": "bytes/launch", "avg_launch_ms": d_ms,
-                "flops_per_launch": d_flops}
+    d_ms, d_flops, d_bytes = kernels[dom]
+    t_mfma_ms = d_flops / (PEAK_BF16_TFLOPS * 1e9)
+    t_hbm_ms = d_bytes / (PEAK_HBM_GBS * 1e6)
+    if t_hbm_ms > t_mfma_ms:
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": d_bytes / d_ms / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": d_bytes / d_ms / 1e6 / PEAK_HBM_GBS}
+    else:
+        roofline = {"kernel": dom, "bound": "mfma", "achieved": d_flops / d_ms / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS}
+    roofline.update({"traffic": MEASURED_TRAFFIC_BYTES.get((name, dom)), "traffic_unit": "bytes/launch", "avg_launch_ms": d_ms,
+                     "flops_per_launch": d_flops, "bytes_per_launch": d_bytes,
+                     "frac_mfma": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS, "frac_hbm": d_bytes / d_ms / 1e6 / PEAK_HBM_GBS})
 
     result = {
         "metric": "moba_fwd_bwd_effective_sparse_tflops" if backward else "moba_fwd_effective_sparse_tflops",

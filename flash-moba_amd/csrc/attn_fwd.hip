@@ -192,7 +192,9 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
   auto meta_store = [&](int sr) {
     if (tid < kFwdRoundRows) {
       sRow[(sr & 1) * kFwdRoundRows + ft] = m_rid;
-      sSlot[(sr & 1) * kFwdRoundRows + ft] = m_slot;
+      // where the visit's partial goes, as an index of partial rows (it fits 32 bits: 2^31 partial rows would be half a
+      // terabyte), or -1 for a row that is absent or has more visits than the caller's bound
+      sSlot[(sr & 1) * kFwdRoundRows + ft] = (m_rid >= 0 && m_slot < ws.cap) ? ((q0 + m_rid) * a.heads + h) * ws.cap + m_slot : -1;
     }
   };
   auto tile_issue = [&](int sr) {  // tile `wave` of round sr
@@ -233,7 +235,12 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
 #endif
   };
   const uint32_t ldsOut = (uint32_t)(uintptr_t)sOut, ldsRow = (uint32_t)(uintptr_t)(smem + SM::oRow) + (uint32_t)(wave * 32 * 4);
-  auto process_tile = [&](auto pc) {
+  // A tile in two steps: the products and the softmax (the partial goes to the wave's LDS tile), then the stores.
+  // Between them the round waits for the loads of the next tile: one counter covers loads and stores alike, so
+  // stores issued before that wait would be waited for as well instead of completing under the next round.
+  float t_m = 0.f, t_l = 0.f;
+  int t_rid = -1;
+  auto compute_tile = [&](auto pc) {
     constexpr int PB = decltype(pc)::value;
     const int sidx = PB * kFwdRoundRows + wave * 32 + (lane & 31);
     const int rid = sRow[sidx];
@@ -267,26 +274,24 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
     __builtin_amdgcn_sched_barrier(0);
     // block-local softmax of the row, log2 domain; keys beyond lim are masked
     const int lim = rid < 0 ? -1 : min(causal ? rid + off : 0x7fffffff, Lk - 1) - key0;  // last visible key, relative
+    // (the scores stay raw: the scale, positive, goes into the exponent's multiply-add)
     float m = -INFINITY;
     if (__all(lim >= KB - 1)) {
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          st[kt][i] *= scale_log2;
-          m = fmaxf(m, st[kt][i]);
-        }
+        for (int i = 0; i < 16; ++i) m = fmaxf(m, st[kt][i]);
     } else {
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int jrel = kt * 32 + 8 * (i >> 2) + (i & 3) + 4 * hh;
-          st[kt][i] = jrel <= lim ? st[kt][i] * scale_log2 : -INFINITY;
+          st[kt][i] = jrel <= lim ? st[kt][i] : -INFINITY;
           m = fmaxf(m, st[kt][i]);
         }
     }
-    m = max_xor32_f(m);
+    m = max_xor32_f(m) * scale_log2;
     const float m_use = m == -INFINITY ? 0.f : m;
     float l = 0.f;
     Pack8 pf[KT][2];  // P^T as the B operand of O^T = V^T P^T, straight from the accumulators
@@ -296,8 +301,8 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-          const float p0 = __builtin_amdgcn_exp2f(st[kt][8 * s2 + 2 * w] - m_use);
-          const float p1 = __builtin_amdgcn_exp2f(st[kt][8 * s2 + 2 * w + 1] - m_use);
+          const float p0 = __builtin_amdgcn_exp2f(fmaf(st[kt][8 * s2 + 2 * w], scale_log2, -m_use));
+          const float p1 = __builtin_amdgcn_exp2f(fmaf(st[kt][8 * s2 + 2 * w + 1], scale_log2, -m_use));
           l += p0 + p1;
           pf[kt][s2].w[w] = pack2<T>(p0, p1);
         }
@@ -333,27 +338,34 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
         lds_write_vec<uint2>(bo + (uint32_t)((dt * 32 + 8 * g) * 2), make_uint2(pack2<T>(o[4 * g], o[4 * g + 1]), pack2<T>(o[4 * g + 2], o[4 * g + 3])));
       __builtin_amdgcn_sched_barrier(0);
     }
+    t_m = m;
+    t_l = l;
+    t_rid = rid;
+  };
+  auto store_tile = [&](auto pc) {
+    constexpr int PB = decltype(pc)::value;
+    const int sidx = PB * kFwdRoundRows + wave * 32 + (lane & 31);
+    const int rid = t_rid;
+    const float m = t_m, l = t_l;
     // header of the partial
-    const int slot = sSlot[sidx];
-    const bool keep = rid >= 0 && slot < ws.cap;
-    const int64_t pidx = ((int64_t)(q0 + max(rid, 0)) * a.heads + h) * ws.cap + slot;
-    if (keep && hh == 0) ws.hdr[pidx] = make_float4(m, l, __int_as_float(nb), 0.f);
+    const int pidx = sSlot[sidx];
+    if (pidx >= 0 && hh == 0) ws.hdr[pidx] = make_float4(m, l, __int_as_float(nb), 0.f);
     wave_lds_fence();
     // rows leave as 16-byte pieces: lane -> (row 4k + lane / 16, features 8 * (lane % 16))
     if ((lane & 15) * 8 < D) {
       uint32_t br = ldsRow + (uint32_t)((lane >> 4) * 4), bx = ldsOut + (uint32_t)(((lane >> 4) * LDO + (lane & 15) * 8) * 2);
       opaque(br);
       opaque(bx);
+      // all indices, then all rows, then the stores: one LDS latency each instead of sixteen in a chain
+      int p2[8];
+      Pack8 x[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int row = 4 * k + (lane >> 4);
-        const int r2 = lds_read_vec<int>(br + (uint32_t)((PB * kFwdRoundRows + 4 * k) * 4));
-        const int s2 = lds_read_vec<int>(br + (uint32_t)((PB * kFwdRoundRows + 4 * k) * 4) + (uint32_t)(SM::oSlot - SM::oRow));
-        if (r2 >= 0 && s2 < ws.cap) {
-          const Pack8 x = lds_read16(bx + (uint32_t)(4 * k * LDO * 2));
-          *reinterpret_cast<Pack8 *>(ws.part + (((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2) * D + (lane & 15) * 8) = x;
-        }
-      }
+      for (int k = 0; k < 8; ++k) p2[k] = lds_read_vec<int>(br + (uint32_t)((PB * kFwdRoundRows + 4 * k) * 4) + (uint32_t)(SM::oSlot - SM::oRow));
+#pragma unroll
+      for (int k = 0; k < 8; ++k) x[k] = lds_read16(bx + (uint32_t)(4 * k * LDO * 2));
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (p2[k] >= 0) *reinterpret_cast<Pack8 *>(ws.part + ((uint64_t)(uint32_t)p2[k] * (uint32_t)D + (uint32_t)((lane & 15) * 8))) = x[k];
     }
     wave_lds_fence();
   };
@@ -365,10 +377,12 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
     rid_issue(r + 2);
     meta_issue(v_rid);
     tile_issue(r + 1);
-    if (4 * r + wave < ntile) process_tile(pc);
+    const bool mine = 4 * r + wave < ntile;
+    if (mine) compute_tile(pc);
+    wait_all_loads();
     meta_store(r + 1);
     rid_store(r + 2);
-    wait_all_loads();
+    if (mine) store_tile(pc);
     __syncthreads();  // round r + 1 is in LDS; everyone is done with round r
   };
   for (int r = 0; r < nround; r += 2) {
@@ -671,6 +685,9 @@ extern "C" int fmoba_attn_fwd_phases(const fmoba_attn_fwd_args *a, int32_t phase
     return 0;
   }
   const size_t rows = (size_t)a->total_q * a->heads;
+  FMOBA_REQUIRE(rows * (size_t)a->max_visits_per_row < ((size_t)1 << 31),
+                "attn_fwd: %zu partial rows exceed the 2^31 the column form indexes (their workspace would not fit any device either)",
+                rows * (size_t)a->max_visits_per_row);
   uintptr_t p = ((uintptr_t)a->workspace + 255) & ~(uintptr_t)255;
   FwdWs ws;
   ws.cap = a->max_visits_per_row;
