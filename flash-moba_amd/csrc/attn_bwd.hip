@@ -556,6 +556,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           dq_mma(gc);
           fence();
         });
+        // The tiles of the next round must be in LDS before the barrier that ends this one, and one counter covers
+        // loads and stores alike: the round's last partial rows are issued after that wait, so that they complete
+        // under the next round instead of being waited for.
+        if constexpr (KB == 1 || decltype(pp)::value == 1) {
+          wait_all_loads();
+          meta_store(r + 1);
+          rid_store(r + 2);
+        }
         dq_store(pc, pp, C1{});
       }
     };
@@ -568,9 +576,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       tile_issue(r + 1);
       process_round(pc, C0{}, r);
       if constexpr (KB == 2) process_round(pc, C1{}, r);
-      meta_store(r + 1);
-      rid_store(r + 2);
-      wait_all_loads();
+      if constexpr (!DQP) {
+        meta_store(r + 1);
+        rid_store(r + 2);
+        wait_all_loads();
+      }
       __syncthreads();  // round r + 1 is in LDS; everyone is done with round r
     };
     for (int r = 0; r < nround; r += 2) {
