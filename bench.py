@@ -103,14 +103,14 @@ def time_events(fn, iters, warmup=1):
 # same counter reads for a plain 1 GiB copy (the summaries of those runs are kept under profiles/, one per workload).
 # Counter runs cannot be made from inside this script, so the figures are the committed measurement.
 MEASURED_TRAFFIC_BYTES = {
-    ("headline", "attn_fwd_rows_kernel"): 1.499e9,
-    ("headline", "attn_bwd_dkdv_kernel"): 6.680e9,
-    ("headline", "attn_bwd_dq_kernel"): 5.008e9,
-    ("c2", "attn_fwd_col_kernel"): 4.719e8,
-    ("c3", "attn_fwd_col_kernel"): 8.568e9,
-    ("c3", "attn_bwd_dkdv_kernel"): 1.260e10,
-    ("c5", "attn_fwd_col_kernel"): 3.978e10,
-    ("c5", "attn_bwd_dkdv_kernel"): 6.465e10,
+    ("headline", "attn_fwd_rows_kernel"): 1.497e9,
+    ("headline", "attn_bwd_dkdv_kernel"): 6.675e9,
+    ("headline", "attn_bwd_dq_kernel"): 5.011e9,
+    ("c2", "attn_fwd_col_kernel"): 4.727e8,
+    ("c3", "attn_fwd_col_kernel"): 8.464e9,
+    ("c3", "attn_bwd_dkdv_kernel"): 1.257e10,
+    ("c5", "attn_fwd_col_kernel"): 3.976e10,
+    ("c5", "attn_bwd_dkdv_kernel"): 6.463e10,
 }
 
 

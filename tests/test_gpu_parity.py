@@ -203,9 +203,20 @@ def test_gating_reference_grid_point_1024_chunks(fm, topk, causal):
 
 
 @pytest.mark.parametrize("causal", [True, False])
-def test_gating_more_than_256_chunks_exact_ties(fm, causal):
-    q, k, cuq, cuk = _gate_case(fm, 9, [900, 1300], [900, 1300], 2, 1, 64, 4, 6, causal, integer=True)
-    _check_gating(fm, q, k, cuq, cuk, 4, 6, causal, integer=True)
+@pytest.mark.parametrize("topk", [6, 12, 17])
+def test_gating_more_than_256_chunks_exact_ties(fm, topk, causal):
+    # (up to 16 running winners per row: the lanes hold four or eight of them each)
+    q, k, cuq, cuk = _gate_case(fm, 9, [900, 1300], [900, 1300], 2, 1, 64, 4, topk, causal, integer=True)
+    _check_gating(fm, q, k, cuq, cuk, 4, topk, causal, integer=True)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("topk", [3, 9, 16])
+def test_gating_thousands_of_chunks_exact_ties(fm, topk, causal):
+    # dozens of groups per row, scores from a small set of integers: many scores equal the weakest winner, rows get
+    # more entrants than a list holds, exact zeros of both signs occur
+    q, k, cuq, cuk = _gate_case(fm, 12, [3000, 700], [3000, 700], 2, 2, 64, 1, topk, causal, integer=True)
+    _check_gating(fm, q, k, cuq, cuk, 1, topk, causal, integer=True)
 
 
 @pytest.mark.parametrize("causal", [True, False])
