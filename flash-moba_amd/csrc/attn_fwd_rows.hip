@@ -1,14 +1,16 @@
-// Sparse attention forward, row-block form, for patterns dense enough that most 128-row blocks
+// Sparse attention forward, row-block form, for patterns dense enough that most row blocks
 // touch most of the chunks they may see (flash_fwd_kernel.h:325-700 of the reference walks the
 // same (row block, key block) grid through its CSC lists).
 //
-// One workgroup owns 128 consecutive query rows of one (sequence, head): four compute waves of
-// 32 rows each and four loader waves (one per SIMD, so that their instructions slow every compute wave
-// alike).  The workgroup walks, in ascending key order, the 64-key
-// blocks of every chunk that at least one of its rows selected; all rows take part in the matrix
-// products of a step, and the rows that did not select the chunk are masked out of the softmax
-// (their probabilities are exact zeros).  The running maximum, the running sum and the output
-// accumulators stay in registers for the whole walk, so nothing but Q, K, V and the output moves.
+// One workgroup owns a block of consecutive query rows of one (sequence, head) and walks, in ascending
+// key order, the 64-key blocks of every chunk that at least one of its rows selected; all rows take
+// part in the matrix products of a step, and the rows that did not select the chunk are masked out
+// of the softmax (their probabilities are exact zeros).  The running maximum, the running sum and
+// the output accumulators stay in registers for the whole walk, so nothing but Q, K, V and the
+// output moves.  Two kernels: attn_fwd_rows_kernel (256 rows, eight compute waves that fetch the
+// K/V tiles straight into LDS themselves; head dimensions up to 128 and up to 512 chunks per
+// sequence) and attn_fwd_rows_loader_kernel (128 rows, four compute and four loader waves; every
+// other shape, head dimension 256 included).
 //
 // The selection of a row is one bit per chunk (a bitmap built from the CSC lists by
 // csc_bitmap_kernel); the chunks a workgroup walks are the OR of its rows' bitmaps.
@@ -55,7 +57,7 @@ __global__ void fwd_zero_u32_kernel(uint32_t *p, int64_t n) {
 }
 
 template <typename T, int HD>
-__global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args a, const uint32_t *bm, int nw) {
+__global__ __launch_bounds__(512) void attn_fwd_rows_loader_kernel(fmoba_attn_fwd_args a, const uint32_t *bm, int nw) {
   typedef FwdRowsSmem<HD> SM;
   constexpr int KS = HD / 16, LDQ = SM::LDQ, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
   constexpr int NTHR = 512;
@@ -426,7 +428,7 @@ struct FwdRows8Smem {
 };
 
 template <typename T, int HD>
-__global__ __launch_bounds__(512) void attn_fwd_rows8_kernel(fmoba_attn_fwd_args a, const uint32_t *bm, int nw) {
+__global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args a, const uint32_t *bm, int nw) {
   typedef FwdRows8Smem<HD> SM;
   constexpr int KS = HD / 16, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
   constexpr int NTHR = 512;
@@ -524,24 +526,40 @@ __global__ __launch_bounds__(512) void attn_fwd_rows8_kernel(fmoba_attn_fwd_args
   const uint32_t ldsK = (uint32_t)(uintptr_t)(smem + SM::oK), ldsV = (uint32_t)(uintptr_t)(smem + SM::oV);
   const uint16_t *kg = reinterpret_cast<const uint16_t *>(a.k) + (int64_t)k0 * a.k_row_stride + (int64_t)hk * a.k_head_stride;
   const uint16_t *vg = reinterpret_cast<const uint16_t *>(a.v) + (int64_t)k0 * a.v_row_stride + (int64_t)hk * a.v_head_stride;
-  int fl = lane;  // re-made opaque at every use: what is derived from it must not be kept in registers across steps
-  auto feed = [&](const uint16_t *g, uint32_t row_stride, uint32_t lds_ring, int stage, int t) {
-#if defined(__HIP_DEVICE_COMPILE__)
-    asm volatile("" : "+v"(fl));
-#endif
-    const int key0 = (sStep[min(t, nstep - 1)] & 0xffff) << 6;
-    const uint32_t dst = lds_ring + (uint32_t)__builtin_amdgcn_readfirstlane(stage * (int)SM::tile + wave * (64 / 8) * RB);
-    const int rl = fl / VPR, p = fl - rl * VPR;
+  // A lane's piece of row tr = wave * 8 + i * RPI + lane / VPR of a tile: its byte offset from the tile's first key, for K
+  // and for V.  A tile whose 64 keys all exist is fetched from a wave-uniform base plus these offsets (no vector
+  // instruction per load); the last tile of a sequence clamps the keys per lane.
+  uint32_t lofK[NI], lofV[NI];
+  {
+    const int rl = lane / VPR, p = lane - rl * VPR;
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int tr = wave * (64 / 8) + i * RPI + rl;  // row of the tile
+      const int tr = wave * (64 / 8) + i * RPI + rl;
       const uint32_t e = (uint32_t)min((p ^ tile_swz<HD>(tr)) * 8, D - 8);
-      const uint32_t key = (uint32_t)min(key0 + tr, Lk - 1);
-      global_to_lds16(g + ((uint64_t)key * row_stride + e), dst + (uint32_t)(i * RPI * RB));
+      lofK[i] = ((uint32_t)tr * (uint32_t)a.k_row_stride + e) * 2u;
+      lofV[i] = ((uint32_t)tr * (uint32_t)a.v_row_stride + e) * 2u;
+    }
+  }
+  auto feed = [&](const uint16_t *g, uint32_t row_stride, const uint32_t(&lof)[NI], uint32_t lds_ring, int stage, int t) {
+    const int key0 = __builtin_amdgcn_readfirstlane((sStep[min(t, nstep - 1)] & 0xffff) << 6);
+    const uint32_t dst = lds_ring + (uint32_t)__builtin_amdgcn_readfirstlane(stage * (int)SM::tile + wave * (64 / 8) * RB);
+    if (key0 + 64 <= Lk) {
+      const uint16_t *base = g + (uint64_t)(uint32_t)key0 * row_stride;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) global_to_lds16_sbase(lof[i], base, dst + (uint32_t)(i * RPI * RB));
+    } else {
+      const int rl = lane / VPR, p = lane - rl * VPR;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int tr = wave * (64 / 8) + i * RPI + rl;  // row of the tile
+        const uint32_t e = (uint32_t)min((p ^ tile_swz<HD>(tr)) * 8, D - 8);
+        const uint32_t key = (uint32_t)min(key0 + tr, Lk - 1);
+        global_to_lds16(g + ((uint64_t)key * row_stride + e), dst + (uint32_t)(i * RPI * RB));
+      }
     }
   };
-  auto feed_k = [&](int t) { feed(kg, (uint32_t)a.k_row_stride, ldsK, t % 3, t); };
-  auto feed_v = [&](int t) { feed(vg, (uint32_t)a.v_row_stride, ldsV, t & 3, t); };
+  auto feed_k = [&](int t) { feed(kg, (uint32_t)a.k_row_stride, lofK, ldsK, t % 3, t); };
+  auto feed_v = [&](int t) { feed(vg, (uint32_t)a.v_row_stride, lofV, ldsV, t & 3, t); };
   // the loads of a step, once per wave: the wait before the next barrier lets exactly these stay in flight
   constexpr int kLoadsPerStep = 2 * NI;
 
@@ -788,8 +806,8 @@ __global__ __launch_bounds__(512) void attn_fwd_rows8_kernel(fmoba_attn_fwd_args
 }
 
 template <typename T, int HD>
-static int launch_rows8(const fmoba_attn_fwd_args &a, const uint32_t *bm, int nw, hipStream_t s) {
-  auto kern = attn_fwd_rows8_kernel<T, HD>;
+static int launch_rows_eight(const fmoba_attn_fwd_args &a, const uint32_t *bm, int nw, hipStream_t s) {
+  auto kern = attn_fwd_rows_kernel<T, HD>;
   const size_t smem = FwdRows8Smem<HD>::bytes;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("attn_fwd: cannot reserve %zu bytes of LDS", smem);
@@ -805,8 +823,8 @@ static int launch_rows8(const fmoba_attn_fwd_args &a, const uint32_t *bm, int nw
 }
 
 template <typename T, int HD>
-static int launch_rows(const fmoba_attn_fwd_args &a, const uint32_t *bm, int nw, hipStream_t s) {
-  auto kern = attn_fwd_rows_kernel<T, HD>;
+static int launch_rows_loader(const fmoba_attn_fwd_args &a, const uint32_t *bm, int nw, hipStream_t s) {
+  auto kern = attn_fwd_rows_loader_kernel<T, HD>;
   const size_t smem = FwdRowsSmem<HD>::bytes;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("attn_fwd: cannot reserve %zu bytes of LDS", smem);
@@ -849,15 +867,16 @@ int run_fwd_rows(const fmoba_attn_fwd_args &a, int phases, hipStream_t s) {
     const bool bf = a.dtype == FMOBA_DTYPE_BF16;
     int rc;
     // eight compute waves when the rows' selection words fit the workgroup's LDS (up to 512 chunks per sequence)
-    const bool eight = nw <= kRows8Words;
+    // (and the rows of a tile lie within 32-bit byte offsets of its first key)
+    const bool eight = nw <= kRows8Words && a.k_row_stride < ((int64_t)1 << 24) && a.v_row_stride < ((int64_t)1 << 24);
     if (a.head_dim <= 64)
-      rc = eight ? (bf ? launch_rows8<bf16_t, 64>(a, bm, nw, s) : launch_rows8<f16_t, 64>(a, bm, nw, s))
-                 : (bf ? launch_rows<bf16_t, 64>(a, bm, nw, s) : launch_rows<f16_t, 64>(a, bm, nw, s));
+      rc = eight ? (bf ? launch_rows_eight<bf16_t, 64>(a, bm, nw, s) : launch_rows_eight<f16_t, 64>(a, bm, nw, s))
+                 : (bf ? launch_rows_loader<bf16_t, 64>(a, bm, nw, s) : launch_rows_loader<f16_t, 64>(a, bm, nw, s));
     else if (a.head_dim <= 128)
-      rc = eight ? (bf ? launch_rows8<bf16_t, 128>(a, bm, nw, s) : launch_rows8<f16_t, 128>(a, bm, nw, s))
-                 : (bf ? launch_rows<bf16_t, 128>(a, bm, nw, s) : launch_rows<f16_t, 128>(a, bm, nw, s));
+      rc = eight ? (bf ? launch_rows_eight<bf16_t, 128>(a, bm, nw, s) : launch_rows_eight<f16_t, 128>(a, bm, nw, s))
+                 : (bf ? launch_rows_loader<bf16_t, 128>(a, bm, nw, s) : launch_rows_loader<f16_t, 128>(a, bm, nw, s));
     else
-      rc = bf ? launch_rows<bf16_t, 256>(a, bm, nw, s) : launch_rows<f16_t, 256>(a, bm, nw, s);
+      rc = bf ? launch_rows_loader<bf16_t, 256>(a, bm, nw, s) : launch_rows_loader<f16_t, 256>(a, bm, nw, s);
     if (rc) return rc;
   }
   return 0;

@@ -491,6 +491,15 @@ __device__ __forceinline__ void global_to_lds16(const void *g, uint32_t lds_base
   (void)g, (void)lds_base;
 #endif
 }
+// The same load with the address split into a wave-uniform 64-bit base and a 32-bit byte offset per lane (unsigned):
+// a tile whose rows lie at a fixed stride costs no vector instruction per load.
+__device__ __forceinline__ void global_to_lds16_sbase(uint32_t lane_byte_off, const void *uniform_base, uint32_t lds_base) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_byte_off), "s"(uniform_base), "s"(lds_base) : "memory");
+#else
+  (void)lane_byte_off, (void)uniform_base, (void)lds_base;
+#endif
+}
 __device__ __forceinline__ void wait_all_loads() {
 #if defined(__HIP_DEVICE_COMPILE__)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -121,7 +121,7 @@ int fmoba_varlen_sort(const int64_t *seg_starts, const int64_t *seg_ends, int64_
  *   out (total_q, heads, head_dim) dtype, softmax_lse (heads, total_q) fp32.
  * Rows that see no key get out = 0, lse = +inf.
  * Two forms.  Row blocks (patterns in which a row selects a good part of the chunks it may see):
- * one workgroup per 128 query rows walks every chunk any of its rows selected, with the running
+ * one workgroup per 256 (or 128) query rows walks every chunk any of its rows selected, with the running
  * softmax state in registers; `workspace` then holds one selection bit per (row, head, chunk).
  * Columns (sparser patterns): every visit of a (query row, key block) pair leaves a
  * partial result in `workspace`, and a second launch merges the partials of each row.  A key
