@@ -103,9 +103,9 @@ def time_events(fn, iters, warmup=1):
 # same counter reads for a plain 1 GiB copy (the summaries of those runs are kept under profiles/, one per workload).
 # Counter runs cannot be made from inside this script, so the figures are the committed measurement.
 MEASURED_TRAFFIC_BYTES = {
-    ("headline", "attn_fwd_rows_kernel"): 1.497e9,
-    ("headline", "attn_bwd_dkdv_kernel"): 6.675e9,
-    ("headline", "attn_bwd_dq_kernel"): 5.011e9,
+    ("headline", "attn_fwd_rows_kernel"): 1.302e9,
+    ("headline", "attn_bwd_dkdv_kernel"): 6.678e9,
+    ("headline", "attn_bwd_dq_kernel"): 5.009e9,
     ("c2", "attn_fwd_col_kernel"): 4.727e8,
     ("c3", "attn_fwd_col_kernel"): 8.464e9,
     ("c3", "attn_bwd_dkdv_kernel"): 1.257e10,
