@@ -416,7 +416,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         *reinterpret_cast<uint2 *>(t + 16 * s2 + 4 * hh) = make_uint2(dsf[TS][s2].w[0], dsf[TS][s2].w[1]);
         *reinterpret_cast<uint2 *>(t + 16 * s2 + 8 + 4 * hh) = make_uint2(dsf[TS][s2].w[2], dsf[TS][s2].w[3]);
       }
-      if constexpr (!DQP) wave_lds_fence();  // (the partials form waits for both key halves at a workgroup barrier later)
+      if constexpr (!DQP) wave_lds_order();  // (the partials form waits for both key halves at a workgroup barrier later)
     };
     // dS form: the wave's 32 keys of every row go to the dS tile of the row's list entry
     int dsrow = -1;
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       dsrow = pRow[TS * 32 + (lane & 31)];
 #pragma unroll
       for (int s4 = 0; s4 < 2; ++s4) dsx[s4] = tr_frag8_at(trdS, 16 * s4 * LDS_, (16 * s4 + 4) * LDS_);
-      wave_lds_fence();
+      wave_lds_order();
     };
     auto ds_store = [&](int tile) {
       if (dsrow >= 0) {

@@ -232,6 +232,17 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// The same order for the compiler only.  The LDS executes the instructions of one wave in the order they were issued, so
+// a read that follows a write of another lane of the same wave needs no wait; the fence above also makes the wave wait
+// for every LDS read it has in flight, which a software-pipelined loop keeps issued well ahead of their use.
+__device__ __forceinline__ void wave_lds_order() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+  asm volatile("" ::: "memory");
+#endif
+}
+
 // Cross-half / cross-row exchanges on the VALU (gfx950 v_permlane32_swap / v_permlane16_swap)
 // instead of the LDS crossbar.  swap32(x): {x of lanes l%32, x of lanes 32 + l%32};
 // swap16(x): {x of the even 16-lane row of this row pair, x of the odd row}.
