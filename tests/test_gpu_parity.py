@@ -192,6 +192,14 @@ def test_gating_more_than_256_chunks_per_sequence(fm, topk, causal):
 
 
 @pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("topk", [5, 16, 40])
+def test_gating_more_than_256_chunks_len_q_ne_len_k(fm, topk, causal):
+    # fewer queries than keys (the queries are the last rows of the sequence), ragged batch, grouped heads
+    q, k, cuq, cuk = _gate_case(fm, 21, [700, 33, 0, 1500], [2600, 700, 90, 1500], 4, 2, 64, 4, topk, causal)
+    _check_gating(fm, q, k, cuq, cuk, 4, topk, causal)
+
+
+@pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("topk", [16, 33, 64])
 def test_gating_reference_grid_point_1024_chunks(fm, topk, causal):
     # (b, h, s) = (8, 2, 1024) with chunk size 1 of tests/test_fused_topk.py:115-122: 1024 chunks per sequence
