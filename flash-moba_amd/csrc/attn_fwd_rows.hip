@@ -434,8 +434,8 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
   constexpr int NTHR = 512;
   constexpr int RB = HD * 2;            // bytes of a tile row
   constexpr int RPI = 64 / VPR;         // tile rows per direct-to-LDS instruction (64 lanes x 16 bytes)
-  constexpr int NI = 64 / RPI / 8;      // such instructions per tile and wave
-  static_assert(NI >= 1, "eight waves share the loads of a tile");
+  constexpr int NI = 64 / RPI / 4;      // such instructions per tile and feeding wave
+  static_assert(NI >= 1, "four waves share the loads of a tile");
   extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
   int *sStep = reinterpret_cast<int *>(smem + SM::oStep);
   uint32_t *sUnion = reinterpret_cast<uint32_t *>(smem + SM::oUnion);
@@ -522,11 +522,13 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
     return;
   }
 
-  // ---- feeding the rings: this wave's share of a tile, rows wave * 8 .. wave * 8 + 7 ------------------------------
+  // ---- feeding the rings: the waves 0..3 fetch the tiles, rows wave * 16 .. wave * 16 + 15 each.  They reach the
+  // barrier of a step well before the waves 4..7 (which run a step's last part one step late and meet them on the
+  // matrix cores at the end of the step), so the loads are theirs ---------------------------------------------------
   const uint32_t ldsK = (uint32_t)(uintptr_t)(smem + SM::oK), ldsV = (uint32_t)(uintptr_t)(smem + SM::oV);
   const uint16_t *kg = reinterpret_cast<const uint16_t *>(a.k) + (int64_t)k0 * a.k_row_stride + (int64_t)hk * a.k_head_stride;
   const uint16_t *vg = reinterpret_cast<const uint16_t *>(a.v) + (int64_t)k0 * a.v_row_stride + (int64_t)hk * a.v_head_stride;
-  // A lane's piece of row tr = wave * 8 + i * RPI + lane / VPR of a tile: its byte offset from the tile's first key, for K
+  // A lane's piece of row tr = wave * 16 + i * RPI + lane / VPR of a tile: its byte offset from the tile's first key, for K
   // and for V.  A tile whose 64 keys all exist is fetched from a wave-uniform base plus these offsets (no vector
   // instruction per load); the last tile of a sequence clamps the keys per lane.
   uint32_t lofK[NI], lofV[NI];
@@ -534,15 +536,16 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
     const int rl = lane / VPR, p = lane - rl * VPR;
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int tr = wave * (64 / 8) + i * RPI + rl;
+      const int tr = (wave & 3) * (64 / 4) + i * RPI + rl;
       const uint32_t e = (uint32_t)min((p ^ tile_swz<HD>(tr)) * 8, D - 8);
       lofK[i] = ((uint32_t)tr * (uint32_t)a.k_row_stride + e) * 2u;
       lofV[i] = ((uint32_t)tr * (uint32_t)a.v_row_stride + e) * 2u;
     }
   }
   auto feed = [&](const uint16_t *g, uint32_t row_stride, const uint32_t(&lof)[NI], uint32_t lds_ring, int stage, int t) {
+    if (wave >= 4) return;
     const int key0 = __builtin_amdgcn_readfirstlane((sStep[min(t, nstep - 1)] & 0xffff) << 6);
-    const uint32_t dst = lds_ring + (uint32_t)__builtin_amdgcn_readfirstlane(stage * (int)SM::tile + wave * (64 / 8) * RB);
+    const uint32_t dst = lds_ring + (uint32_t)__builtin_amdgcn_readfirstlane(stage * (int)SM::tile + wave * (64 / 4) * RB);
     if (key0 + 64 <= Lk) {
       const uint16_t *base = g + (uint64_t)(uint32_t)key0 * row_stride;
 #pragma unroll
@@ -551,7 +554,7 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
       const int rl = lane / VPR, p = lane - rl * VPR;
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
-        const int tr = wave * (64 / 8) + i * RPI + rl;  // row of the tile
+        const int tr = wave * (64 / 4) + i * RPI + rl;  // row of the tile
         const uint32_t e = (uint32_t)min((p ^ tile_swz<HD>(tr)) * 8, D - 8);
         const uint32_t key = (uint32_t)min(key0 + tr, Lk - 1);
         global_to_lds16(g + ((uint64_t)key * row_stride + e), dst + (uint32_t)(i * RPI * RB));
@@ -560,7 +563,7 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
   };
   auto feed_k = [&](int t) { feed(kg, (uint32_t)a.k_row_stride, lofK, ldsK, t % 3, t); };
   auto feed_v = [&](int t) { feed(vg, (uint32_t)a.v_row_stride, lofV, ldsV, t & 3, t); };
-  // the loads of a step, once per wave: the wait before the next barrier lets exactly these stay in flight
+  // the loads of a step, once per feeding wave: the wait before the next barrier lets exactly these stay in flight
   constexpr int kLoadsPerStep = 2 * NI;
 
   const int lim = valid ? min(causal ? row + off : 0x7fffffff, Lk - 1) : -1;  // last visible key
@@ -736,13 +739,13 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
   };
   auto wait_older_loads = [&]() {  // all but the loads of the current step
 #if defined(__HIP_DEVICE_COMPILE__)
-    if constexpr (kLoadsPerStep == 4)
-      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    if constexpr (kLoadsPerStep == 8)
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else
-      asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
 #endif
   };
-  static_assert(kLoadsPerStep == 4 || kLoadsPerStep == 2, "wait_older_loads");
+  static_assert(kLoadsPerStep == 8 || kLoadsPerStep == 4, "wait_older_loads");
 
   // K(0), K(1), V(0) have to be there for the first step: the two youngest groups of loads (K(2), V(1)) may stay out
   wait_older_loads();
