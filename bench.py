@@ -103,14 +103,14 @@ def time_events(fn, iters, warmup=1):
 # same counter reads for a plain 1 GiB copy (the summaries of those runs are kept under profiles/, one per workload).
 # Counter runs cannot be made from inside this script, so the figures are the committed measurement.
 MEASURED_TRAFFIC_BYTES = {
-    ("headline", "attn_fwd_rows_kernel"): 1.302e9,
-    ("headline", "attn_bwd_dkdv_kernel"): 6.678e9,
-    ("headline", "attn_bwd_dq_kernel"): 5.009e9,
-    ("c2", "attn_fwd_col_kernel"): 4.727e8,
-    ("c3", "attn_fwd_col_kernel"): 8.464e9,
-    ("c3", "attn_bwd_dkdv_kernel"): 1.257e10,
+    ("headline", "attn_fwd_rows_kernel"): 1.293e9,
+    ("headline", "attn_bwd_dkdv_kernel"): 6.679e9,
+    ("headline", "attn_bwd_dq_kernel"): 5.012e9,
+    ("c2", "attn_fwd_col_kernel"): 4.726e8,
+    ("c3", "attn_fwd_col_kernel"): 8.441e9,
+    ("c3", "attn_bwd_dkdv_kernel"): 1.254e10,
     ("c5", "attn_fwd_col_kernel"): 3.976e10,
-    ("c5", "attn_bwd_dkdv_kernel"): 6.463e10,
+    ("c5", "attn_bwd_dkdv_kernel"): 6.464e10,
 }
 
 
