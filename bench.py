@@ -176,6 +176,42 @@ def dense_sdpa_ms(cfg, dev, iters=3):
     return time_events(step, iters)
 
 
+def graph_replay_ms(q, k, v, dout, cu, max_len, chunk, topk, backward, steps):
+    """The same step recorded once as a HIP graph (torch.cuda.CUDAGraph) and replayed `steps` times: what a serving or
+    training loop pays per step when it keeps the launches of the hot path in a graph.  Reported beside `ms_per_step`
+    (which stays the eager loop); None if the capture fails."""
+    import flash_moba
+
+    try:
+        qs, ks, vs = (t.detach().clone().requires_grad_(backward) for t in (q, k, v))
+
+        def once():
+            out = flash_moba.flash_moba_varlen_func(qs, ks, vs, cu, cu, max_len, max_len, chunk, topk, causal=True)
+            return (out,) + (torch.autograd.grad(out, (qs, ks, vs), dout) if backward else ())
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            once()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            keep = once()
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        del graph, keep
+        return ms
+    except Exception as e:  # the eager measurement does not depend on this one
+        print(f"bench.py: graph replay not measured: {e}", file=sys.stderr)
+        return None
+
+
 def run_config(name, steps, warmup, args, dev, cpu_budget_s):
     """Measures one configuration: K timed steps, then per-stage and per-kernel timings, the roofline object of its
     dominant kernel and (cpu_budget_s > 0) the CPU leg on a bounded sample of the same inputs."""
@@ -205,6 +241,7 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    graph_ms = graph_replay_ms(q, k, v, dout, cu, max_len, chunk, topk, backward, steps)
 
     # ---- algorithmic work -------------------------------------------------------------
     with torch.no_grad():
@@ -325,6 +362,7 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
         "steps": steps,
         "warmup": warmup,
         "ms_per_step": ms_per_step,
+        "graph_replay_ms_per_step": graph_ms,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -387,7 +425,7 @@ def main():
             r = run_config(name, k_steps, 2, args, dev, 0.0 if args.no_cpu else cpu_s)
             if name == "sweep16k":
                 r["dense_sdpa_fwd_bwd_ms"] = dense_sdpa_ms(CONFIGS[name], dev)  # the dense baseline of the reference's benchmark
-            keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "frac_of_bf16_mfma_peak", "pairs", "flops_per_step",
+            keep = ("metric", "value", "unit", "ms_per_step", "graph_replay_ms_per_step", "steps", "warmup", "frac_of_bf16_mfma_peak", "pairs", "flops_per_step",
                     "topk_csc_ms", "stages", "roofline", "cpu_baseline", "dense_sdpa_fwd_bwd_ms")
             entry = {"name": name, "workload": r["config"]["workload"]}
             entry.update({k: r[k] for k in keep if k in r})
