@@ -36,6 +36,29 @@ static inline int csc_seg_rows(int64_t batch, int64_t heads, int64_t max_seqlen_
   return seg_rows;
 }
 
+// n + (x0 > y) + (x1 > y) + (x2 > y) + (x3 > y): four compares into four scalar register pairs, then four adds with
+// carry, so that no add follows its compare at once (a vector instruction that reads a scalar register written by the
+// one before it has to wait; left alone, the compiler pairs every compare with its consumer and pads with idle slots)
+__device__ __forceinline__ int count4_gt(int n, float x0, float x1, float x2, float x3, float y) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  unsigned long long m0, m1, m2, m3;
+  asm("v_cmp_gt_f32_e64 %1, %5, %9\n\t"
+      "v_cmp_gt_f32_e64 %2, %6, %9\n\t"
+      "v_cmp_gt_f32_e64 %3, %7, %9\n\t"
+      "v_cmp_gt_f32_e64 %4, %8, %9\n\t"
+      "v_addc_co_u32_e64 %0, vcc, 0, %0, %1\n\t"
+      "v_addc_co_u32_e64 %0, vcc, 0, %0, %2\n\t"
+      "v_addc_co_u32_e64 %0, vcc, 0, %0, %3\n\t"
+      "v_addc_co_u32_e64 %0, vcc, 0, %0, %4"
+      : "+v"(n), "=&s"(m0), "=&s"(m1), "=&s"(m2), "=&s"(m3)
+      : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "v"(y)
+      : "vcc");
+  return n;
+#else
+  return n + (x0 > y) + (x1 > y) + (x2 > y) + (x3 > y);
+#endif
+}
+
 template <typename T, int HD, int NT>
 __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_kernel(TopkParams p) {
   constexpr int KS = HD / 16;
@@ -179,7 +202,7 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
       for (int t = 0; t < NT; ++t)
         if (t < n_tiles) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) cnt += (sc[t][i] > probe) ? 1 : 0;
+          for (int i = 0; i < 16; i += 4) cnt = count4_gt(cnt, sc[t][i], sc[t][i + 1], sc[t][i + 2], sc[t][i + 3], probe);
         }
       cnt = sum_xor32_i(cnt);
       if (open) {
