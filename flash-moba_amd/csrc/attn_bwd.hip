@@ -60,7 +60,7 @@ struct BwdWs {
   int32_t *pid;    // [total_q * heads * cap] key block id of each partial
   uint16_t *part;  // [total_q * heads * cap][head_dim] dQ partials (unscaled)
   int32_t cap;
-  uint16_t *ds;    // [row list entry][lg_block_n] dS tiles (row-stationary dQ form)
+  uint16_t *ds;    // dS tiles (row-stationary dQ form): [row list position / 32][key of the column / 8][position % 32][8 keys]
 };
 
 // DQP = true: dQ partials per visit (for the combine kernel); false: dS^T tiles to ws.ds (for the row-stationary dQ kernel).
@@ -429,9 +429,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     };
     auto ds_store = [&](int tile) {
       if (dsrow >= 0) {
-        uint16_t *wp = ws.ds + (lbase + start + tile * 32 + (lane & 31)) * Bn + koff + kq * 32;
+        // key groups koff / 8 + 4 kq + 2 s4 + hh of list position p: consecutive lanes write consecutive 16-byte pieces
+        const int64_t p = lbase + start + tile * 32 + (lane & 31);
+        uint16_t *wp = ws.ds + ds_piece_offset(p, (koff >> 3) + 4 * kq + hh, Bn >> 3);
 #pragma unroll
-        for (int s4 = 0; s4 < 2; ++s4) *reinterpret_cast<Pack8 *>(wp + 16 * s4 + 8 * hh) = dsx[s4];
+        for (int s4 = 0; s4 < 2; ++s4) *reinterpret_cast<Pack8 *>(wp + s4 * 512) = dsx[s4];
       }
     };
     auto dq_load = [&](auto tsc) {
@@ -642,33 +644,44 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 }
 
 // ------------------------------------------------------------------------------------
-// dQ, first form: row blocks.  One workgroup owns 128 consecutive query rows of one (sequence, head) and walks the
-// 64-key blocks of every column in which one of its rows appears.  The dS rows of a step (written by the dK/dV
-// pass in list order) go from global memory straight into the registers of the lane that owns the query row; rows
-// that are absent contribute zeros, so every compute wave multiplies its own 32 rows and keeps dQ in registers for
-// the whole walk.  Registers (128) and LDS (about 52 KB) leave room for two workgroups per compute unit: one
-// workgroup's waits at barriers and on LDS are covered by the other.
+// dQ, first form: row blocks.  One workgroup owns 256 or 512 consecutive query rows of one (sequence, head) and
+// walks the 64-key blocks of every column in which one of its rows appears.  The dS rows of a step (written by the
+// dK/dV pass in list order) go from global memory straight into the registers of the lane that owns the query row;
+// rows that are absent contribute zeros, so every wave multiplies its own 32-row tiles and keeps dQ in registers
+// for the whole walk.  All eight waves compute, two per SIMD, and nothing in the workgroup only moves data.  What a
+// step needs from other threads -- its K tile (global memory straight into LDS, global_load_lds, every wave a share
+// of the tile, swizzled rows of exactly head_dim elements) and the list positions of its rows (scattered into LDS by
+// the thread whose index is the row's place in the step's run) -- is prepared for a whole group of G steps at once,
+// one group ahead, so the workgroup meets at a barrier once per group: inside a group every wave runs at its own
+// pace, and a wave's chain of dependent steps (where are my rows in this column's list -> fetch them -> multiply)
+// is covered by the products of the other wave of its SIMD.
 // ------------------------------------------------------------------------------------
-constexpr int kDqRows = 128;
+constexpr int kDqWaves = 8;
 constexpr int kDqColBatch = 256;
 constexpr int kDqMaxSteps = 512;
-constexpr int kDqRing = 4;   // K tiles the loaders keep in flight
-constexpr int kDqRows2 = 2;  // dS rows in flight per compute lane (16 registers each)
 
-template <int HD>
+template <int HD, int RT>
 struct DqSmem {
-  static constexpr int LDQ = HD + 16;  // elements, K tile
+  static constexpr int ROWS = kDqWaves * 32 * RT;
+  static constexpr int G = HD == 128 ? 4 : 2;  // steps per group (one workgroup barrier per group)
+  static constexpr int NS = 2 * G;              // K tiles / position slots in LDS: the group in use and the next one
   static constexpr int LDO = HD + 8;   // elements, per-wave output tile [32 rows][LDO] (reuses the K tiles at the end)
-  static constexpr size_t oK = 0;                                   // [2][64][LDQ]
-  static constexpr size_t oTag = oK + (size_t)2 * 64 * LDQ * 2;    // int[3][rows of the block, at most 256]: (step tag << 8) | list position of the row in that step
-  static constexpr size_t oLo = oTag + 3 * 2 * kDqRows * 4;
+  static constexpr size_t tileBytes = (size_t)64 * HD * 2;
+  static constexpr size_t outBytes = (size_t)kDqWaves * 32 * LDO * 2;
+  static constexpr size_t prepBytes = (size_t)kDqColBatch * 16 + (size_t)kDqMaxSteps * 4;
+  static constexpr size_t oK = 0;                                   // [NS][64 keys][HD], swizzled; later the output tiles
+  static constexpr size_t ringBytes = NS * tileBytes > outBytes ? NS * tileBytes : outBytes;
+  static_assert(prepBytes <= ringBytes, "the preparation arrays lie over the K tiles");
+  static constexpr size_t oTag = oK + ringBytes;                   // int[NS][ROWS]: (step tag << 10) | list position of the row in that step
+  static constexpr size_t oInfo = oTag + (size_t)NS * ROWS * 4;    // int4[kDqMaxSteps]: key0, rows, list position (lo, hi)
+  static constexpr size_t oMisc = oInfo + (size_t)kDqMaxSteps * 16;
+  static constexpr size_t bytes = oMisc + 64;
+  // what only the preparation of a batch of columns uses (no tile is in use or on its way then)
+  static constexpr size_t oOff = oK;                                // int64[kDqColBatch]
+  static constexpr size_t oLo = oOff + kDqColBatch * 8;
   static constexpr size_t oCnt = oLo + kDqColBatch * 4;
   static constexpr size_t oStep = oCnt + kDqColBatch * 4;
-  static constexpr size_t oOff = oStep + kDqMaxSteps * 4;          // int64[kDqColBatch]
-  static constexpr size_t oInfo = oOff + kDqColBatch * 8;          // int4[kDqMaxSteps]: key0, rows, list position (lo, hi)
-  static constexpr size_t oMisc = oInfo + kDqMaxSteps * 16;
-  static constexpr size_t bytes = oMisc + 64;
-  static_assert((size_t)4 * 32 * LDO * 2 <= (size_t)2 * 64 * LDQ * 2, "output tiles must fit the K tiles");
+  static_assert(bytes <= 160 * 1024, "LDS of one compute unit");
 };
 
 struct DqItem {
@@ -683,16 +696,26 @@ __device__ __forceinline__ DqItem dq_decode_item(int id, int npairs, int nsb_max
   return w;
 }
 
-// RT: 32-row tiles per compute wave.  With two, a workgroup owns 256 rows and every K^T operand read from LDS feeds two
-// MFMAs; the accumulators then take 128 registers, and one workgroup fits a compute unit instead of two.
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {  // until at most N of the wave's vector memory loads are outstanding
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+#endif
+}
+
+// RT: 32-row tiles per wave.  With two, a workgroup owns 512 rows and every K^T operand read from LDS feeds two MFMAs.
 template <typename T, int HD, int RT>
 __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq_kernel(fmoba_attn_bwd_args a, const uint16_t *ds_ws, int nsb_max) {
-  typedef DqSmem<HD> SM;
-  constexpr int ROWS = kDqRows * RT;  // query rows of the workgroup
-  constexpr int LDQ = SM::LDQ, LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
-  constexpr int KVV = 64 * VPR / 256;  // K-tile vectors per loader thread
+  typedef DqSmem<HD, RT> SM;
+  constexpr int ROWS = SM::ROWS;  // query rows of the workgroup
+  constexpr int LDO = SM::LDO, NDT = HD / 32, VPR = HD / 8;
+  constexpr int RB = HD * 2;                       // bytes of a K tile row
+  constexpr uint32_t TB = (uint32_t)SM::tileBytes;
+  constexpr int RPI = 64 / VPR;                    // K rows per load instruction
+  constexpr int NKI = 64 / RPI / kDqWaves;         // K load instructions per wave and tile
+  static_assert(NKI >= 1 && NKI * RPI * kDqWaves == 64, "the waves share a K tile evenly");
+  constexpr int NS = SM::NS, G = SM::G;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint16_t *sK = reinterpret_cast<uint16_t *>(smem + SM::oK);
   int *sPos = reinterpret_cast<int *>(smem + SM::oTag);
   int *sLo = reinterpret_cast<int *>(smem + SM::oLo);
   int *sCnt = reinterpret_cast<int *>(smem + SM::oCnt);
@@ -700,6 +723,7 @@ __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq
   int64_t *sOff = reinterpret_cast<int64_t *>(smem + SM::oOff);
   int4 *sInfo = reinterpret_cast<int4 *>(smem + SM::oInfo);
   int *sMisc = reinterpret_cast<int *>(smem + SM::oMisc);
+  const uint32_t ldsK = (uint32_t)(uintptr_t)(smem + SM::oK);
 
   const DqItem wi = dq_decode_item(blockIdx.x, a.heads * a.batch, nsb_max);
   if (wi.pair < 0) return;
@@ -713,12 +737,11 @@ __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq
   const int D = a.head_dim;
   const int hk = h / (a.heads / a.heads_k);
   const int Bn = a.lg_block_n, nsub = Bn / 64;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
-  const bool is_loader = tid >= 256;
-  const int ltid = tid & 255;
+  const int tid = threadIdx.x, lane = tid & 63, hh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool causal = a.is_causal != 0;
 
-  for (int v = tid; v < 3 * ROWS; v += 512) sPos[v] = 0;  // step tags start at 1
+  for (int v = tid; v < NS * ROWS; v += 512) sPos[v] = 0;  // step tags start at 1
 
   int ncols = min((Lk + Bn - 1) / Bn, a.max_cols);
   const int last_rowpos = m0 + rows_sb - 1 + off;
@@ -729,7 +752,8 @@ __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq
   const int cols_per_batch = min(kDqColBatch, kDqMaxSteps / nsub);
 
   // The steps of one batch of columns: for every column the part of its list that falls into this row block, then
-  // one record per (column, 64-key block) that has rows and visible keys.  Both roles run it (same barriers).
+  // one record per (column, 64-key block) that has rows and visible keys.  Its scratch arrays lie over the K tiles:
+  // no tile is in use or on its way when the workgroup comes here.
   auto prepare_batch = [&](int cb, int cend) {
     __syncthreads();
     for (int c = cb + tid; c < cend; c += 512) {
@@ -765,214 +789,214 @@ __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq
       if (lane == 0) sMisc[0] = nst;
     }
     __syncthreads();
-    const int nsteps = sMisc[0];
-    // one record per step, so that a loader needs a single LDS read before it can issue its loads
+    const int nsteps = __builtin_amdgcn_readfirstlane(sMisc[0]);
+    // one record per step
     for (int st = tid; st < nsteps; st += 512) {
       const int code = sStep[st];
       const int cl = code >> 8, kb = code & 255;
       const int64_t pos0 = sOff[cl];
       sInfo[st] = make_int4((cb + cl) * Bn + kb * 64, sCnt[cl], (int)(uint32_t)(pos0 & 0xffffffffll), (int)(pos0 >> 32));
     }
-    __syncthreads();
+    __syncthreads();  // (also: everyone has read the scratch arrays before the first tile loads overwrite them)
     return nsteps;
   };
 
-  typedef std::integral_constant<int, 0> P0;
-  // The K tiles are double buffered in LDS by step parity: while the compute waves work on step s the loaders put
-  // step s+1 into the other buffer and then fetch step s+1+RK into the ring entry that this frees.  The loaders also
-  // tell every query row of the block where its dS row of a step lies (position in the step's list segment, tagged
-  // with the step number), NR steps ahead; a compute lane fetches the 128 bytes of its row (one half per lane of the
-  // pair that holds the row) NR-1 steps ahead of their use.  Rows that are not in a step keep a stale tag.
-  // The two roles run separate code with the same barrier sequence.  Every load is issued unconditionally and no
-  // control flow joins a path between a load and its use: the compiler sizes each wait by the smallest number of
-  // younger loads over all paths that reach it, and a path without loads would make every use wait for the whole ring.
-  constexpr int RK = kDqRing;  // ring of the K tiles (and of the row ids, which run NR - 1 steps ahead of them)
-  constexpr int NR = kDqRows2;
-  constexpr int PADTO = (NR % 4 == 0) ? NR : ((NR % 2 == 0) ? 2 * NR : 4 * NR);
-  if (is_loader) {
-    Pack8 pk[RK][KVV];
-    int prid[RK];
-    int tag_base = 0;
-    uint32_t kvo[KVV];
+  f32x16 acc[RT][NDT];
 #pragma unroll
-    for (int i = 0; i < KVV; ++i) kvo[i] = (uint32_t)((ltid / VPR + i * (256 / VPR)) * (int)a.k_row_stride + min((ltid % VPR) * 8, D - 8));
-    const int klo = (ltid / VPR) * LDQ + (ltid % VPR) * 8;
-    for (int cb = 0; cb < ncols; cb += cols_per_batch) {
-      const int nsteps = prepare_batch(cb, min(ncols, cb + cols_per_batch));
-      if (nsteps == 0) continue;
-      auto row_id = [&](int step) {  // row of list position ltid of the step (clamped), for the threads that write positions
-        const int4 info = sInfo[min(step, nsteps - 1)];
-        const int n = __builtin_amdgcn_readfirstlane(info.y);
-        const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
-        return a.row_indices[pos0 + min(ltid & (ROWS - 1), n - 1)];
-      };
-      auto put_pos = [&](int step, int rr) {  // positions of the rows of `step`
-        if (step < nsteps && ltid < ROWS) {
-          const int4 info = sInfo[step];
-          const int key0 = info.x, n = info.y;
-          const int first_rel = causal ? key0 - off - m0 : -0x40000000;  // rows before it see no key of the block
-          const int rel = rr - m0;
-          if ((ltid < n) & ((uint32_t)rel < (uint32_t)rows_sb) & (rel >= first_rel)) sPos[(step % 3) * ROWS + rel] = ((tag_base + step + 1) << 8) | ltid;
-        }
-      };
-      // K of `step`, row ids of `step + 2`
-      auto load_step = [&](auto par, int step) {
-        constexpr int P = decltype(par)::value;
-        const int key0 = __builtin_amdgcn_readfirstlane(sInfo[min(step, nsteps - 1)].x);
-        if (key0 + 64 <= Lk) {
-          const uint16_t *kb0 = kp + (int64_t)key0 * a.k_row_stride;
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-          for (int i = 0; i < KVV; ++i) pk[P][i] = ld_global16(kb0 + kvo[i]);
-        } else {
+    for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
-          for (int i = 0; i < KVV; ++i) {
-            const int v = ltid + i * 256;
-            const int key = min(key0 + v / VPR, Lk - 1), e = min((v % VPR) * 8, D - 8);
-            pk[P][i] = ld_global16(kp + (int64_t)key * a.k_row_stride + e);
-          }
-        }
-        prid[P] = row_id(step + NR - 1);
-      };
-      auto store_step = [&](auto par, int step) {
-        constexpr int P = decltype(par)::value;
-        const int key0 = __builtin_amdgcn_readfirstlane(sInfo[step].x);
-        uint16_t *tK = sK + (size_t)(step & 1) * 64 * LDQ;
-        if (D == HD && key0 + 64 <= Lk) {
+      for (int i = 0; i < 16; ++i) acc[rt][dt][i] = 0.f;
+  int myrow[RT];
 #pragma unroll
-          for (int i = 0; i < KVV; ++i) *reinterpret_cast<Pack8 *>(tK + klo + i * (256 / VPR) * LDQ) = pk[P][i];
-        } else {
+  for (int rt = 0; rt < RT; ++rt) myrow[rt] = (wave * RT + rt) * 32 + (lane & 31);
+
+  // K tile loads of this wave: instruction i brings tile rows (wave * NKI + i) * RPI .. + RPI - 1, lane -> row rl, piece p;
+  // piece c of tile row r is stored at piece c ^ tile_swz<HD>(r)
+  const int krl = lane / VPR, kpp = lane - krl * VPR;
+  uint32_t ksrc[NKI];  // element offset of this lane's piece inside a tile that exists completely
 #pragma unroll
-          for (int i = 0; i < KVV; ++i) {
-            const int v = ltid + i * 256;
-            const int key = v / VPR, e = (v - key * VPR) * 8;
-            const bool ok = (key0 + key < Lk) & (e < D);
-            Pack8 x = pk[P][i];
-#pragma unroll
-            for (int w = 0; w < 4; ++w) x.w[w] = ok ? x.w[w] : 0u;
-            *reinterpret_cast<Pack8 *>(tK + key * LDQ + e) = x;
-          }
-        }
-        put_pos(step + NR - 1, prid[P]);
-      };
-      static_for<RK>([&](auto e) { load_step(e, decltype(e)::value); });
-      for (int t = 0; t < NR - 1; ++t) put_pos(t, row_id(t));
-      store_step(P0{}, 0);
-      load_step(P0{}, RK);
-      __syncthreads();  // the positions of steps 0, 1, 2 are in LDS
-      auto loader_step = [&](auto par, int step) {  // par: ring entry of step + 1, stored during step
-        __syncthreads();
-        if (step + 1 < nsteps) store_step(par, step + 1);
-        load_step(par, step + 1 + RK);
-      };
-      const int nsteps_pad = (nsteps + PADTO - 1) / PADTO * PADTO;
-      for (int step = 0; step < nsteps_pad; step += RK)
-        static_for<RK>([&](auto e) { loader_step(std::integral_constant<int, (decltype(e)::value + 1) % RK>{}, step + decltype(e)::value); });
-      tag_base += nsteps;
-    }
-    __syncthreads();  // the compute waves are done with the K tiles
-  } else {
-    f32x16 acc[RT][NDT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[rt][dt][i] = 0.f;
-    int myrow[RT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) myrow[rt] = (wave * RT + rt) * 32 + (lane & 31);
-    int tag_base = 0;
-    Pack8 df[NR][RT][4];   // this lane's dS rows of NR consecutive steps (B operands)
-    bool dfp[NR][RT];
-    for (int cb = 0; cb < ncols; cb += cols_per_batch) {
-      const int nsteps = prepare_batch(cb, min(ncols, cb + cols_per_batch));
-      if (nsteps == 0) continue;
-      // fetch this lane's dS rows of `step` into ring entry R (unconditional: an absent row reads position 0)
-      auto fetch = [&](auto rc, int step) {
-        constexpr int R = decltype(rc)::value;
-        const int sc_ = min(step, nsteps - 1);
-        const int4 info = sInfo[sc_];
-        const int key0 = __builtin_amdgcn_readfirstlane(info.x);
-        const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
-        const int koff = key0 - (key0 / Bn) * Bn;
-        const uint16_t *rp = ds_ws + pos0 * Bn + koff + 8 * hh;
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          const int v = sPos[(sc_ % 3) * ROWS + myrow[rt]];
-          const bool pres = (step < nsteps) & ((v >> 8) == tag_base + sc_ + 1);
-          const uint32_t j = pres ? (uint32_t)(v & 255) : 0u;
-#pragma unroll
-          for (int s4 = 0; s4 < 4; ++s4) df[R][rt][s4] = ld_global16(rp + j * (uint32_t)Bn + 16 * s4);
-          dfp[R][rt] = pres;
-        }
-      };
-      auto compute = [&](auto rc, int step) {
-        constexpr int R = decltype(rc)::value;
-        bool anyp = false;
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) anyp |= dfp[R][rt];
-        if (!__any(anyp)) return;
-        Pack8 dz[RT][4];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-          for (int s4 = 0; s4 < 4; ++s4)
-#pragma unroll
-            for (int w = 0; w < 4; ++w) dz[rt][s4].w[w] = dfp[R][rt] ? df[R][rt][s4].w[w] : 0u;
-        lds_cu16 *trK = tr_lane_base(sK + (size_t)(step & 1) * 64 * LDQ, LDQ, lane) + 8 * hh * LDQ;
-        // K^T operands half a feature tile (two products per row tile) ahead of their use
-        Pack8 kf[2][2];
-        auto kread = [&](int u, Pack8 (&dst)[2]) {  // unit u: feature tile u / 2, keys 32 (u % 2) .. + 31
-          const int dt = u >> 1, sb = 2 * (u & 1);
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) dst[s2] = tr_frag8_at(trK, 16 * (sb + s2) * LDQ + dt * 32, (16 * (sb + s2) + 4) * LDQ + dt * 32);
-        };
-        kread(0, kf[0]);
-#pragma unroll
-        for (int u = 0; u < 2 * NDT; ++u) {
-          if (u + 1 < 2 * NDT) kread(u + 1, kf[(u + 1) & 1]);
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt) acc[rt][u >> 1] = mfma32<T>(kf[u & 1][s2], dz[rt][2 * (u & 1) + s2], acc[rt][u >> 1]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      };
-      __syncthreads();  // the positions of the first steps are in LDS
-      static_for<NR - 1>([&](auto e) { fetch(e, decltype(e)::value); });
-      const int nsteps_pad = (nsteps + PADTO - 1) / PADTO * PADTO;
-      for (int step = 0; step < nsteps_pad; step += NR)
-        static_for<NR>([&](auto e) {
-          constexpr int E = decltype(e)::value;
-          __syncthreads();
-          fetch(std::integral_constant<int, (E + NR - 1) % NR>{}, step + E + NR - 1);
-          if (step + E < nsteps) compute(e, step + E);
-        });
-      tag_base += nsteps;
-    }
-    __syncthreads();  // every wave is done with the K tiles: they now hold the output tiles (one 32-row tile per wave)
-    uint16_t *sOut = reinterpret_cast<uint16_t *>(smem + SM::oK) + (size_t)wave * 32 * LDO;
-    uint16_t *op = reinterpret_cast<uint16_t *>(a.dq) + (int64_t)(q0 + m0) * a.dq_row_stride + (int64_t)h * a.dq_head_stride;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-          *reinterpret_cast<uint2 *>(sOut + (lane & 31) * LDO + dt * 32 + 8 * g + 4 * hh) =
-              make_uint2(pack2<T>(acc[rt][dt][4 * g] * a.softmax_scale, acc[rt][dt][4 * g + 1] * a.softmax_scale),
-                         pack2<T>(acc[rt][dt][4 * g + 2] * a.softmax_scale, acc[rt][dt][4 * g + 3] * a.softmax_scale));
-      wave_lds_fence();
-      // rows leave as 16-byte pieces, VPR of them per row, consecutive lanes taking consecutive pieces
-#pragma unroll
-      for (int v0 = 0; v0 < 32 * VPR; v0 += 64) {
-        const int v = v0 + lane, rl = v / VPR, e = (v - rl * VPR) * 8;
-        const int r2 = (wave * RT + rt) * 32 + rl;
-        if (r2 < rows_sb && e < D)
-          *reinterpret_cast<Pack8 *>(op + (int64_t)r2 * a.dq_row_stride + e) = *reinterpret_cast<const Pack8 *>(sOut + rl * LDO + e);
+  for (int i = 0; i < NKI; ++i) {
+    const int r = (wave * NKI + i) * RPI + krl;
+    ksrc[i] = (uint32_t)(r * (int)a.k_row_stride + min((kpp ^ tile_swz<HD>(r)) * 8, D - 8));
+  }
+  // K^T operands (transposing reads): lane l (i = l % 16) supplies the address of key 8 hh + i / 4 (+ 4 for the
+  // second read) of a 16-key group, features 16 ((l / 16) % 2) + 4 (i % 4) .. of a 32-feature tile
+  const int li = lane & 15;
+  const int kk0 = 8 * hh + (li >> 2);
+  const int low2 = ((lane >> 4) & 1) * 2 + ((li & 3) >> 1);
+  const uint32_t tlo = (uint32_t)(kk0 * RB + ((low2 ^ tile_swz<HD>(kk0)) * 16) + (li & 1) * 8);
+  const uint32_t thi = (uint32_t)((kk0 + 4) * RB + ((low2 ^ tile_swz<HD>(kk0 + 4)) * 16) + (li & 1) * 8);
+
+  int tag_base = 0;
+  Pack8 df[2][RT][4];  // this lane's dS rows of two consecutive steps (B operands)
+  bool dfp[2][RT];
+  int rid[G];
+  for (int cb = 0; cb < ncols; cb += cols_per_batch) {
+    const int nsteps = prepare_batch(cb, min(ncols, cb + cols_per_batch));
+    if (nsteps == 0) continue;
+    auto row_id = [&](int step) {  // row of list position tid of the step (clamped)
+      const int4 info = sInfo[min(step, nsteps - 1)];
+      const int n = __builtin_amdgcn_readfirstlane(info.y);
+      const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
+      return a.row_indices[pos0 + min(tid & (ROWS - 1), n - 1)];
+    };
+    auto put_pos = [&](int step, int rr) {  // thread t tells row rr, the t-th of the step's run, where it is
+      if (step < nsteps && tid < ROWS) {
+        const int4 info = sInfo[step];
+        const int key0 = info.x, n = info.y;
+        const int first_rel = causal ? key0 - off - m0 : -0x40000000;  // rows before it see no key of the block
+        const int rel = rr - m0;
+        if ((tid < n) & ((uint32_t)rel < (uint32_t)rows_sb) & (rel >= first_rel)) sPos[(step % NS) * ROWS + rel] = ((tag_base + step + 1) << 10) | tid;
       }
-      wave_lds_fence();
+    };
+    auto k_issue = [&](int step) {  // this wave's share of the K tile of `step`
+      const int key0 = __builtin_amdgcn_readfirstlane(sInfo[min(step, nsteps - 1)].x);
+      const uint32_t dst = ldsK + (uint32_t)__builtin_amdgcn_readfirstlane(step % NS) * TB + (uint32_t)(wave * NKI) * 1024u;
+      if (key0 + 64 <= Lk) {
+        const uint16_t *kb0 = kp + (int64_t)key0 * a.k_row_stride;
+#pragma unroll
+        for (int i = 0; i < NKI; ++i) global_to_lds16_sbase(ksrc[i] * 2u, kb0, dst + (uint32_t)i * 1024u);
+      } else {  // keys past the end of the sequence: the last key's data, which meets dS = 0
+#pragma unroll
+        for (int i = 0; i < NKI; ++i) {
+          const int r = (wave * NKI + i) * RPI + krl;
+          const int key = min(key0 + r, Lk - 1), e = min((kpp ^ tile_swz<HD>(r)) * 8, D - 8);
+          global_to_lds16(kp + (int64_t)key * a.k_row_stride + e, dst + (uint32_t)i * 1024u);
+        }
+      }
+    };
+    // fetch this lane's dS rows of `step` into ring entry R (unconditional: an absent row reads a piece near its neighbours')
+    auto fetch = [&](auto rc, int step) {
+      constexpr int R = decltype(rc)::value;
+      const int sc_ = min(step, nsteps - 1);
+      // (all LDS reads first: one wait)
+      const int4 info = sInfo[sc_];
+      int v[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) v[rt] = sPos[(sc_ % NS) * ROWS + myrow[rt]];
+      const int key0 = __builtin_amdgcn_readfirstlane(info.x);
+      const int n = __builtin_amdgcn_readfirstlane(info.y);
+      const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
+      const int koff = key0 - (key0 / Bn) * Bn;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const bool pres = (step < nsteps) & ((v[rt] >> 10) == tag_base + sc_ + 1);
+        const uint32_t j = pres ? (uint32_t)(v[rt] & 1023) : (uint32_t)(myrow[rt] * n) / (uint32_t)ROWS;
+        const uint16_t *rp = ds_ws + ds_piece_offset(pos0 + j, (koff >> 3) + hh, Bn >> 3);
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) df[R][rt][s4] = ld_global16(rp + 512 * s4);
+        dfp[R][rt] = pres;
+      }
+    };
+    // the products of `step`; `between` runs after the first group of them (the tile loads of a later step: issued
+    // there, they are younger than every load this step has waited for)
+    auto compute = [&](auto rc, int step, auto &&between) {
+      constexpr int R = decltype(rc)::value;
+      bool anyp = false;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) anyp |= dfp[R][rt];
+      if (!__any(anyp) || step >= nsteps) {
+        between();
+        return;
+      }
+      Pack8 dz[RT][4];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) dz[rt][s4].w[w] = dfp[R][rt] ? df[R][rt][s4].w[w] : 0u;
+      const uint32_t stage = ldsK + (uint32_t)__builtin_amdgcn_readfirstlane(step % NS) * TB;
+      const uint32_t alo = tlo + stage, ahi = thi + stage;
+      // K^T operands half a feature tile (two products per row tile) ahead of their use
+      Pack8 kf[2][2];
+      auto kread = [&](int u, Pack8 (&dst)[2]) {  // unit u: feature tile u / 2, keys 32 (u % 2) .. + 31
+        const uint32_t x = (uint32_t)((u >> 1) * 64);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const uint32_t o = (uint32_t)(16 * (2 * (u & 1) + s2) * RB);
+          dst[s2] = lds_tr8((alo ^ x) + o, (ahi ^ x) + o);
+        }
+      };
+      kread(0, kf[0]);
+#pragma unroll
+      for (int u = 0; u < 2 * NDT; ++u) {
+        if (u + 1 < 2 * NDT) kread(u + 1, kf[(u + 1) & 1]);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) acc[rt][u >> 1] = mfma32<T>(kf[u & 1][s2], dz[rt][2 * (u & 1) + s2], acc[rt][u >> 1]);
+        if (u == 0) between();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // before the loop: positions of steps 0 .. G, row ids of steps G + 1 .. 2 G, K tiles of steps 0 .. G - 1, dS rows of step 0
+    {
+      int r0[G + 1];
+#pragma unroll
+      for (int g = 0; g <= G; ++g) r0[g] = row_id(g);
+#pragma unroll
+      for (int g = 0; g < G; ++g) rid[g] = row_id(G + 1 + g);
+#pragma unroll
+      for (int g = 0; g <= G; ++g) put_pos(g, r0[g]);
     }
+#pragma unroll
+    for (int g = 0; g < G; ++g) k_issue(g);
+    __syncthreads();
+    fetch(std::integral_constant<int, 0>{}, 0);
+    wait_all_loads();
+    // group of steps s0 .. s0 + G - 1: positions of steps s0 + G + 1 .. s0 + 2 G into LDS, row ids of the G steps after
+    // those, then per step the dS rows of the next step and the products of this one; the K tile loads of the next
+    // group are issued among the products of the group's first step
+    const int nsteps_pad = (nsteps + G - 1) / G * G;
+    for (int s0 = 0; s0 < nsteps_pad; s0 += G) {
+      __syncthreads();  // the K tiles of this group and the positions up to step s0 + G are in LDS; everyone is done with the group before
+#pragma unroll
+      for (int g = 0; g < G; ++g) put_pos(s0 + G + 1 + g, rid[g]);
+#pragma unroll
+      for (int g = 0; g < G; ++g) rid[g] = row_id(s0 + 2 * G + 1 + g);
+      static_for<G>([&](auto e) {
+        constexpr int E = decltype(e)::value;
+        const int s = s0 + E;
+        fetch(std::integral_constant<int, (E + 1) & 1>{}, s + 1);
+        compute(std::integral_constant<int, E & 1>{}, s, [&]() {
+          if constexpr (E == 0) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) k_issue(s0 + G + g);
+          }
+        });
+      });
+      // this wave's share of the next group's K tiles has to be in LDS at the barrier: everything but the dS rows
+      // fetched after it was issued
+      wait_loads_but<(G - 1) * 4 * RT>();
+    }
+    tag_base += nsteps;
+    wait_all_loads();
+  }
+  __syncthreads();  // every wave is done with the K tiles: they now hold the output tiles (one 32-row tile per wave)
+  uint16_t *sOut = reinterpret_cast<uint16_t *>(smem + SM::oK) + (size_t)wave * 32 * LDO;
+  uint16_t *op = reinterpret_cast<uint16_t *>(a.dq) + (int64_t)(q0 + m0) * a.dq_row_stride + (int64_t)h * a.dq_head_stride;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<uint2 *>(sOut + (lane & 31) * LDO + dt * 32 + 8 * g + 4 * hh) =
+            make_uint2(pack2<T>(acc[rt][dt][4 * g] * a.softmax_scale, acc[rt][dt][4 * g + 1] * a.softmax_scale),
+                       pack2<T>(acc[rt][dt][4 * g + 2] * a.softmax_scale, acc[rt][dt][4 * g + 3] * a.softmax_scale));
+    wave_lds_fence();
+    // rows leave as 16-byte pieces, VPR of them per row, consecutive lanes taking consecutive pieces
+#pragma unroll
+    for (int v0 = 0; v0 < 32 * VPR; v0 += 64) {
+      const int v = v0 + lane, rl = v / VPR, e = (v - rl * VPR) * 8;
+      const int r2 = (wave * RT + rt) * 32 + rl;
+      if (r2 < rows_sb && e < D)
+        *reinterpret_cast<Pack8 *>(op + (int64_t)r2 * a.dq_row_stride + e) = *reinterpret_cast<const Pack8 *>(sOut + rl * LDO + e);
+    }
+    wave_lds_fence();
   }
 }
 
@@ -1101,12 +1125,12 @@ static int launch_dkdv(const fmoba_attn_bwd_args &a, const BwdWs &ws, hipStream_
 template <typename T, int HD, int RT>
 static int launch_dq(const fmoba_attn_bwd_args &a, const uint16_t *ws, hipStream_t s) {
   auto kern = attn_bwd_dq_kernel<T, HD, RT>;
-  const size_t smem = DqSmem<HD>::bytes;
+  const size_t smem = DqSmem<HD, RT>::bytes;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("attn_bwd: cannot reserve %zu bytes of LDS", smem);
     return 2;
   }
-  const int nsb_max = ceil_div(a.max_seqlen_q, kDqRows * RT);
+  const int nsb_max = ceil_div(a.max_seqlen_q, DqSmem<HD, RT>::ROWS);
   const int64_t items = (int64_t)a.heads * a.batch * nsb_max;
   if (items >= ((int64_t)1 << 31)) {
     set_error("attn_bwd: too many (sequence, head, superblock) work items");
@@ -1203,7 +1227,7 @@ extern "C" int32_t fmoba_attn_bwd_uses_partials(const fmoba_attn_bwd_args *a) {
 extern "C" size_t fmoba_attn_bwd_workspace_bytes(const fmoba_attn_bwd_args *a) {
   using namespace fmoba;
   if (a == nullptr || a->total_q <= 0 || a->heads <= 0 || a->head_dim <= 0 || a->batch <= 0 || a->lg_block_n <= 0) return 256;
-  if (!bwd_dq_partials(*a)) return (size_t)(a->num_row_indices > 0 ? a->num_row_indices : 0) * a->lg_block_n * 2 + 256;
+  if (!bwd_dq_partials(*a)) return ds_workspace_tiles(a->num_row_indices) * (size_t)a->lg_block_n * 64 + 256;
   const size_t rows = (size_t)a->total_q * a->heads, cap = (size_t)bwd_partial_cap(*a);
   // one spare partial row / block id at the end takes the writes of absent rows
   return bwd_align256(rows * 4) + bwd_align256((rows * cap + 1) * 4) + bwd_align256((rows * cap + 1) * a->head_dim * 2) + 256;

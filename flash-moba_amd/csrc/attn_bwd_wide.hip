@@ -179,12 +179,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_wide_kernel(fmoba_attn_bwd_
         dv[dt] = mfma32<T>(dot, pf[s2], dv[dt]);
         dk[dt] = mfma32<T>(qt, dsf[s2], dk[dt]);
       }
-    // the dS tile leaves as rows of 64 keys, 16 bytes per thread, to the row's list entry
+    // the dS tile leaves in 16-byte pieces (8 keys of one list entry), one per thread
     if (ds_ws != nullptr) {
       __syncthreads();
-      const int rl = tid >> 3, piece = tid & 7;
+      const int rl = tid & 31, piece = tid >> 5;  // consecutive threads: consecutive list positions of one key group
       if (sRow[rl] >= 0)
-        *reinterpret_cast<Pack8 *>(ds_ws + (lbase + start + tile * 32 + rl) * Bn + koff + piece * 8) = *reinterpret_cast<const Pack8 *>(sdS + rl * LDX + piece * 8);
+        *reinterpret_cast<Pack8 *>(ds_ws + ds_piece_offset(lbase + start + tile * 32 + rl, (koff >> 3) + piece, Bn >> 3)) = *reinterpret_cast<const Pack8 *>(sdS + rl * LDX + piece * 8);
     }
   }
 
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_wide_kernel(fmoba_attn_bwd_
   }
 }
 
-// dK / dV and the dS tiles for head dimensions above 128 (ds_ws: [row list entry][lg_block_n] 16-bit)
+// dK / dV and the dS tiles for head dimensions above 128 (ds_ws: the dS workspace, laid out by ds_piece_offset)
 int run_bwd_dkdv_wide(const fmoba_attn_bwd_args &a, uint16_t *ds_ws, hipStream_t s) {
   const size_t smem = BwdWideSmem::bytes;
   const dim3 grid(ceil_div(a.max_seqlen_k, 64), a.heads, a.batch);

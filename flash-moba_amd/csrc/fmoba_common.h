@@ -494,7 +494,8 @@ __device__ __forceinline__ Pack8 lds_tr8(uint32_t addr_lo, uint32_t addr_hi) {
 // 64 lanes x 16 bytes from each lane's own global address to LDS bytes [lds_base, lds_base + 1024), lane order;
 // lds_base is the same for the whole wave.  Written as assembly because the compiler makes every later LDS read wait
 // for a load that it knows to write LDS, and these are meant to stay in flight for a whole round: the kernel waits for
-// them itself (wait_all_loads) before the barrier that hands the tiles over.  Nothing else in the kernel uses m0.
+// them itself (wait_all_loads) before the barrier that hands the tiles over.  m0 is not in the clobber list: the compiler reserves it, warns that such a
+// clobber may not be honoured, and sets it itself right before each of its own instructions that read it.
 __device__ __forceinline__ void global_to_lds16(const void *g, uint32_t lds_base) {
 #if defined(__HIP_DEVICE_COMPILE__)
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base) : "memory");
@@ -516,6 +517,15 @@ __device__ __forceinline__ void wait_all_loads() {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #endif
 }
+// The dS workspace of the backward (16-bit): tiles of 32 consecutive positions of the row-index array; inside a tile
+// the 16-byte pieces (8 keys) of one key group of all 32 entries are contiguous:
+//   [position / 32][key of the column / 8][position % 32][8 keys].
+// The dK/dV pass writes a gathered tile (32 consecutive positions) in runs of consecutive pieces, and the dQ pass
+// brings a run of positions into LDS one contiguous kilobyte (two key groups of a tile) per load instruction.
+// Returns the element offset of piece (position p, key group kg); kgs = key groups per entry (column width / 8).
+__host__ __device__ __forceinline__ int64_t ds_piece_offset(int64_t p, int kg, int kgs) { return ((((p >> 5) * kgs + kg) << 5) + (p & 31)) << 3; }
+static inline size_t ds_workspace_tiles(int64_t positions) { return (size_t)((positions > 0 ? positions : 0) + 31) / 32 + 1; }
+
 // Row id of a gathered tile row as it is kept in LDS: r itself if the entry is present and the row exists, else
 // negative with a row that exists in the low 31 bits (the entry's own if it exists: past the end of a list that is the
 // list's last row, whose data the column meets anyway; else row 0).  The tile loads fetch that row unconditionally, the
