@@ -2,11 +2,12 @@
 
 Mirrors the reference's benchmarks/bench_flash_moba.py (batch 2, 16 heads of 128, fp16, causal,
 chunk 128, top-k 8, sequence lengths 4K ... 512K, forward and backward timed separately, TFLOP/s
-counted on the DENSE causal work of the same shape so that the two methods share one axis).  The
+counted on the DENSE causal work of the same shape so that the two methods share one axis) and its
+benchmarks/bench_flash_moba_memory.py (peak device memory of one forward + backward per point).  The
 dense baseline is torch's scaled_dot_product_attention (its flash kernel on ROCm) where the
 reference uses flash_attn_varlen_func.
 
-    python flash-moba_amd/benchmarks/bench_flash_moba.py [--max-seqlen 262144] [--dense-max-seqlen 65536]
+    python flash-moba_amd/benchmarks/bench_flash_moba.py [--max-seqlen 524288] [--dense-max-seqlen 65536]
 
 Prints one line per (method, sequence length) and a JSON line per sequence length.
 """
@@ -49,9 +50,25 @@ def time_fwd_bwd(fn, inputs, repeats):
     return tf / repeats, tb / repeats
 
 
+def peak_memory_mb(fn, inputs):
+    """Peak device memory (MiB, torch.cuda.max_memory_allocated) of one forward + backward after one warm-up pass, as
+    the reference's benchmarks/bench_flash_moba_memory.py:104-143 measures it: inputs and the upstream gradient included."""
+    out = fn()
+    grad = torch.randn_like(out)
+    torch.autograd.grad(out, inputs, grad)
+    del out
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    out = fn()
+    torch.autograd.grad(out, inputs, grad)
+    torch.cuda.synchronize()
+    return torch.cuda.max_memory_allocated() / 1024 ** 2
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--max-seqlen", type=int, default=262144)
+    ap.add_argument("--max-seqlen", type=int, default=524288)
     ap.add_argument("--dense-max-seqlen", type=int, default=65536, help="longest sequence the dense baseline is timed on")
     ap.add_argument("--chunk", type=int, default=128)
     ap.add_argument("--topk", type=int, default=8)
@@ -76,11 +93,14 @@ def main():
         f, b = time_fwd_bwd(lambda: flash_moba_varlen_func(q, k, v, cu, cu, seqlen, seqlen, args.chunk, args.topk, causal=causal),
                             (q, k, v), repeats)
         row["FlashMoBA"] = {"fwd_ms": f, "bwd_ms": b}
+        row["FlashMoBA"]["peak_mb"] = peak_memory_mb(
+            lambda: flash_moba_varlen_func(q, k, v, cu, cu, seqlen, seqlen, args.chunk, args.topk, causal=causal), (q, k, v))
         if seqlen <= args.dense_max_seqlen:
             qd, kd, vd = (t.detach().view(batch, seqlen, nheads, headdim).transpose(1, 2).requires_grad_(True) for t in (q, k, v))
             f2, b2 = time_fwd_bwd(lambda: torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, is_causal=causal),
                                   (qd, kd, vd), repeats)
             row["SDPA"] = {"fwd_ms": f2, "bwd_ms": b2}
+            row["SDPA"]["peak_mb"] = peak_memory_mb(lambda: torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, is_causal=causal), (qd, kd, vd))
         print(f"### causal={causal}, headdim={headdim}, batch_size={batch}, seqlen={seqlen} ###")
         for method in ("FlashMoBA", "SDPA"):
             if method not in row:
@@ -88,7 +108,7 @@ def main():
             tf, tb = row[method]["fwd_ms"], row[method]["bwd_ms"]
             eff = lambda mode, ms: dense_flops(batch, seqlen, headdim, nheads, causal, mode) / (ms * 1e-3) / 1e12
             print(f"{method} fwd: {eff('fwd', tf):.2f} TFLOPs/s, time: {tf:.2f} ms, bwd: {eff('bwd', tb):.2f} TFLOPs/s, time: {tb:.2f} ms, "
-                  f"fwd + bwd: {eff('fwd_bwd', tf + tb):.2f} TFLOPs/s, time: {tf + tb:.2f} ms")
+                  f"fwd + bwd: {eff('fwd_bwd', tf + tb):.2f} TFLOPs/s, time: {tf + tb:.2f} ms, peak memory: {row[method]['peak_mb'] / 1024:.2f} GiB")
         if "SDPA" in row:
             row["speedup_fwd_bwd"] = (row["SDPA"]["fwd_ms"] + row["SDPA"]["bwd_ms"]) / (f + b)
         print(json.dumps(row), flush=True)
