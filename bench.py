@@ -38,10 +38,12 @@ CONFIGS = {
     "c2": ([8192], 16, 128, 128, 8, False),
     "c3": ([32768], 32, 128, 128, 16, True),
     "c5": ([262144], 16, 128, 128, 16, True),
-    # two points of the reference's own sequence-length sweep (benchmarks/bench_flash_moba.py): batch 2, chunk 128, top-k 8
+    # two points of the reference's own sequence-length sweep (benchmarks/bench_flash_moba.py): batch 2, chunk 128, top-k 8, fp16
     "sweep16k": ([16384, 16384], 16, 128, 128, 8, True),
     "sweep64k": ([65536, 65536], 16, 128, 128, 8, True),
 }
+# the arithmetic type of the 16-bit inputs: bf16 as BASELINE.json's configs say, fp16 where the reference's own sweep uses it
+CONFIG_DTYPE = {"sweep16k": "fp16", "sweep64k": "fp16"}
 
 
 def headline_seqlens(seed=1004, n=8, total=65536, lo=2048, hi=14336, mult=64):
@@ -54,7 +56,7 @@ def headline_seqlens(seed=1004, n=8, total=65536, lo=2048, hi=14336, mult=64):
     return lens
 
 
-def make_inputs(seqlens, H, D, chunk, seed, device):
+def make_inputs(seqlens, H, D, chunk, seed, device, dtype=torch.bfloat16):
     """q, v, dout ~ N(0,1); k = N(0,1) + per-(sequence, chunk, head) bias ~ N(0, 0.5)."""
     g = torch.Generator(device=device).manual_seed(seed)
     T = sum(seqlens)
@@ -69,8 +71,7 @@ def make_inputs(seqlens, H, D, chunk, seed, device):
         k[pos:pos + L] += bias.repeat_interleave(chunk, dim=0)[:L]
         pos += L
     cu = torch.tensor([0] + list(np.cumsum(seqlens)), dtype=torch.int32, device=device)
-    bf = torch.bfloat16
-    return q.to(bf), k.to(bf), v.to(bf), dout.to(bf), cu
+    return q.to(dtype), k.to(dtype), v.to(dtype), dout.to(dtype), cu
 
 
 def count_pairs(seqlens, col_nnz, chunk, H):
@@ -162,12 +163,12 @@ def cpu_baseline(q, k, v, cu, seqlens, chunk, topk, budget_s=12.0):
 
 
 def dense_sdpa_ms(cfg, dev, iters=3):
-    """Forward + backward of dense causal attention (torch scaled_dot_product_attention, bf16) on a sweep shape: the
+    """Forward + backward of dense causal attention (torch scaled_dot_product_attention, fp16) on a sweep shape: the
     baseline benchmarks/bench_flash_moba.py of the reference compares with."""
     seqlens, H, D, _, _, _ = cfg
     B, L = len(seqlens), seqlens[0]
-    q, k, v = (torch.randn((B, H, L, D), device=dev, dtype=torch.bfloat16, requires_grad=True) for _ in range(3))
-    g = torch.randn((B, H, L, D), device=dev, dtype=torch.bfloat16)
+    q, k, v = (torch.randn((B, H, L, D), device=dev, dtype=torch.float16, requires_grad=True) for _ in range(3))
+    g = torch.randn((B, H, L, D), device=dev, dtype=torch.float16)
 
     def step():
         q.grad = k.grad = v.grad = None
@@ -223,7 +224,9 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
     if seqlens is None:
         seqlens = headline_seqlens()
     T, nb, max_len = sum(seqlens), len(seqlens), max(seqlens)
-    q, k, v, dout, cu = make_inputs(seqlens, H, D, chunk, 1000 + len(seqlens), dev)
+    dtype_name = CONFIG_DTYPE.get(name, "bf16")
+    q, k, v, dout, cu = make_inputs(seqlens, H, D, chunk, 1000 + len(seqlens), dev,
+                                    torch.float16 if dtype_name == "fp16" else torch.bfloat16)
     q.requires_grad_(backward), k.requires_grad_(backward), v.requires_grad_(backward)
 
     def step():
@@ -294,16 +297,20 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
         "attn_fwd": {"ms": t_fwd, "TFLOPs": fwd_flops / t_fwd / 1e9, "frac_mfma": fwd_flops / t_fwd / 1e9 / PEAK_BF16_TFLOPS,
                      "phases_ms": fwd_phase_ms},
     }
-    # Compulsory HBM bytes of a launch: every tensor once, plus what the form of the kernel writes or reads per list
-    # entry (partial results, dS tiles); rows that a kernel gathers again per visit count once.
+    # Compulsory HBM bytes of a launch: the tensors it has to read and write, once each (q, k, v, out, dout, dq, dk, dv of
+    # T*H*D*2 bytes, the selection bits or the CSC lists); rows that a kernel gathers again per visit count once.  What a
+    # form of a kernel writes or reads per list entry on top of that (partial results, dS tiles) is the implementation's
+    # own scratch traffic and is reported beside it, not inside it.
     entries = int(cn.sum().item())
     qkv_once = T * H * D * 2
+    list_bytes = entries * 4
     fwd_visits = entries * (chunk // hip.fwd_key_block(chunk))
+    # kernels[name] = (ms, FLOP, compulsory bytes, scratch bytes)
     # one kernel runs both forward GEMMs: the row-block pass, or the column pass (its combine only merges partial rows)
     if row_blocks:
-        kernels = {"attn_fwd_rows_kernel": (fwd_phase_ms["row_blocks"], fwd_flops, 4 * qkv_once + T * H * ((maxC + 31) // 32) * 4)}
+        kernels = {"attn_fwd_rows_kernel": (fwd_phase_ms["row_blocks"], fwd_flops, 4 * qkv_once + T * H * ((maxC + 31) // 32) * 4, 0)}
     else:
-        kernels = {"attn_fwd_col_kernel": (fwd_phase_ms["columns"], fwd_flops, 3 * qkv_once + fwd_visits * (D * 2 + 16))}
+        kernels = {"attn_fwd_col_kernel": (fwd_phase_ms["columns"], fwd_flops, 3 * qkv_once + list_bytes, fwd_visits * (D * 2 + 16))}
     if backward:
         dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
         phase_ms = {}
@@ -329,10 +336,10 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
         # it writes one dQ partial row per visit instead
         if hip.last_bwd_partials():
             bwd_kb = 128 if (chunk % 128 == 0 and D > 64) else 64
-            kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 10.0 * D * pairs, 6 * qkv_once + entries * (chunk // bwd_kb) * (D * 2 + 4))
+            kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 10.0 * D * pairs, 6 * qkv_once + list_bytes, entries * (chunk // bwd_kb) * (D * 2 + 4))
         else:
-            kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 8.0 * D * pairs, 6 * qkv_once + entries * chunk * 2)
-            kernels["attn_bwd_dq_kernel"] = (phase_ms["dq"], 2.0 * D * pairs, 2 * qkv_once + entries * chunk * 2)
+            kernels["attn_bwd_dkdv_kernel"] = (phase_ms["dkdv"], 8.0 * D * pairs, 6 * qkv_once + list_bytes, entries * chunk * 2)
+            kernels["attn_bwd_dq_kernel"] = (phase_ms["dq"], 2.0 * D * pairs, 2 * qkv_once + list_bytes, entries * chunk * 2)
     # sort alone, on the CSC the gating produced (already sorted input; same traffic)
     t_sort = time_events(lambda: torch.ops.flash_moba._varlen_sort(co, cn, ind), it)
     sort_bytes = 2 * int(cn.sum().item()) * 4 + 2 * cn.numel() * 8
@@ -341,7 +348,7 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
     # ---- roofline of the dominant kernel ---------------------------------------------------
     # The bound is the roof that lies lower for this launch: the larger of flops / MFMA peak and bytes / HBM peak.
     dom = max(kernels, key=lambda n: kernels[n][0])
-    d_ms, d_flops, d_bytes = kernels[dom]
+    d_ms, d_flops, d_bytes, d_scratch = kernels[dom]
     t_mfma_ms = d_flops / (PEAK_BF16_TFLOPS * 1e9)
     t_hbm_ms = d_bytes / (PEAK_HBM_GBS * 1e6)
     if t_hbm_ms > t_mfma_ms:
@@ -351,7 +358,7 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
         roofline = {"kernel": dom, "bound": "mfma", "achieved": d_flops / d_ms / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                     "frac": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS}
     roofline.update({"traffic": MEASURED_TRAFFIC_BYTES.get((name, dom)), "traffic_unit": "bytes/launch", "avg_launch_ms": d_ms,
-                     "flops_per_launch": d_flops, "bytes_per_launch": d_bytes,
+                     "flops_per_launch": d_flops, "bytes_per_launch": d_bytes, "scratch_bytes_per_launch": d_scratch,
                      "frac_mfma": d_flops / d_ms / 1e9 / PEAK_BF16_TFLOPS, "frac_hbm": d_bytes / d_ms / 1e6 / PEAK_HBM_GBS})
 
     result = {
@@ -366,7 +373,7 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": dtype_name,
         "data": "synthetic",
         "config": {"workload": f"{name}: varlen packed batch, {nb} sequences totalling {T} tokens "
                                f"(lengths {seqlens}), causal, {H} heads, head_dim {D}, chunk {chunk}, top-k {topk}, "
@@ -382,6 +389,27 @@ def run_config(name, steps, warmup, args, dev, cpu_budget_s):
     if cpu_budget_s > 0:
         result["cpu_baseline"] = cpu_baseline(qd, kd, vd, cu, seqlens, chunk, topk, budget_s=cpu_budget_s)
     return result
+
+
+def stage_summary(r):
+    """The per-stage and per-kernel milliseconds of one configuration as one flat object (what a reader of the tail of
+    the line looks for first)."""
+    st = r["stages"]
+    out = {"workload": r["config"]["workload"].split(":")[0], "dtype": r["dtype"], "ms_per_step": round(r["ms_per_step"], 4),
+           "effective_sparse_tflops": round(r["value"], 1), "frac_of_bf16_mfma_peak": round(r["frac_of_bf16_mfma_peak"], 4),
+           "mean_pool_ms": round(st["mean_pool"]["ms"], 4), "mean_pool_frac_hbm": round(st["mean_pool"]["frac_hbm"], 4),
+           "topk_csc_ms": round(st["topk_csc"]["ms"], 4), "topk_csc_frac_hbm": round(st["topk_csc"]["frac_hbm"], 4),
+           "attn_fwd_ms": round(st["attn_fwd"]["ms"], 4), "attn_fwd_frac_mfma": round(st["attn_fwd"]["frac_mfma"], 4)}
+    for k, v in st["attn_fwd"]["phases_ms"].items():
+        out["fwd_" + k + "_ms"] = round(v, 4)
+    if "attn_bwd" in st:
+        out["attn_bwd_ms"] = round(st["attn_bwd"]["ms"], 4)
+        out["attn_bwd_frac_mfma"] = round(st["attn_bwd"]["frac_mfma"], 4)
+        for k, v in st["attn_bwd"]["phases_ms"].items():
+            out["bwd_" + k + "_ms"] = round(v, 4)
+    out["varlen_sort_ms"] = round(st["varlen_sort"]["ms"], 4)
+    out["varlen_sort_frac_hbm"] = round(st["varlen_sort"]["frac_hbm"], 4)
+    return out
 
 
 
@@ -425,11 +453,16 @@ def main():
             r = run_config(name, k_steps, 2, args, dev, 0.0 if args.no_cpu else cpu_s)
             if name == "sweep16k":
                 r["dense_sdpa_fwd_bwd_ms"] = dense_sdpa_ms(CONFIGS[name], dev)  # the dense baseline of the reference's benchmark
-            keep = ("metric", "value", "unit", "ms_per_step", "graph_replay_ms_per_step", "steps", "warmup", "frac_of_bf16_mfma_peak", "pairs", "flops_per_step",
+            keep = ("metric", "value", "unit", "dtype", "ms_per_step", "graph_replay_ms_per_step", "steps", "warmup", "frac_of_bf16_mfma_peak", "pairs", "flops_per_step",
                     "topk_csc_ms", "stages", "roofline", "cpu_baseline", "dense_sdpa_fwd_bwd_ms")
             entry = {"name": name, "workload": r["config"]["workload"]}
             entry.update({k: r[k] for k in keep if k in r})
             result["configs"].append(entry)
+    # last keys of the line: the other configurations' stage and kernel times as flat objects, then those of the configuration that was asked for
+    if "configs" in result:
+        result["configs_stages_flat"] = [stage_summary({**c, "config": {"workload": c["name"] + ":"}}) for c in result["configs"]]
+    result["stages_flat"] = stage_summary(result)
+    result["topk_csc_ms"] = result.pop("topk_csc_ms")
     print(json.dumps(result))
 
 

@@ -316,12 +316,12 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
   constexpr int PL = CAP / 2;    // previous winners held per lane (two lanes per row)
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint16_t *sKm = reinterpret_cast<uint16_t *>(smem);
-  uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [W][128], reuses the chunk-mean tile after the last group
+  uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [word columns of a pass][128], reuses the chunk-mean tile after the last group
   float *sVal = reinterpret_cast<float *>(smem + (size_t)GC * LD * 2);   // [NLIST][128][CAP]
   int *sIdx = reinterpret_cast<int *>(sVal + NLIST * kGateRows * CAP);   // [NLIST][128][CAP]
   int *sCnt = sIdx + NLIST * kGateRows * CAP;                            // [2][128]
-  int *sHist = sCnt + 2 * kGateRows;                                     // [max_cols]
-  int *sTrash = sHist + p.max_cols;                                      // [256]: takes the stores of lanes that have nothing to store
+  int *sHist = sCnt + 2 * kGateRows;                                     // [32 chunks per word column the tile holds as selection words]
+  int *sTrash = sHist + (size_t)GC * LD * 2 / (kGateRows * 4) * 32;      // [256]: takes the stores of lanes that have nothing to store
 
   const fmoba_fused_topk_args &a = p.a;
   const int mb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -655,38 +655,48 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
   }
   __syncthreads();
 
-  // selection words and per-chunk counts of the block, assembled in LDS
-  for (int v = tid; v < p.W * kGateRows; v += 256) sSel[v] = 0u;
-  for (int c = tid; c < p.max_cols; c += 256) sHist[c] = 0;
-  __syncthreads();
-  if (valid) {
-    const int m = min(sCnt[cur * kGateRows + rs], CAP);
-#pragma unroll
-    for (int j = 0; j < PL; ++j) {
-      const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
-      if (e < m) {
-        const int c = sIdx[((TWO_LISTS ? cur : 0) * kGateRows + rs) * CAP + e];
-        atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
-        atomicAdd(&sHist[c], 1);
-      }
-    }
-    if (hh == 0 && a.is_causal && rp >= 0) {
-      const int c = rp / B;  // the own chunk is always selected
-      if (c < p.max_cols) {
-        atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
-        atomicAdd(&sHist[c], 1);
-      }
-    }
-  }
-  __syncthreads();
-  for (int v = tid; v < p.W * kGateRows; v += 256) {
-    const int t = v / kGateRows, slot_r = v - t * kGateRows;
-    if (m0 + slot_r < Lq) p.sel[((int64_t)h * p.W + t) * a.total_q + q0 + m0 + slot_r] = sSel[v];
-  }
+  // selection words and per-chunk counts of the block, assembled in LDS and written out in passes of WP word columns
+  // (what the chunk-mean tile holds), so that a sequence may have any number of chunks
+  const int WP = min(p.W, (int)((size_t)GC * LD * 2 / (kGateRows * 4)));
+  const int m_fin = valid ? min(sCnt[cur * kGateRows + rs], CAP) : 0;
   const int seg = m0 / p.seg_rows;
-  for (int c = tid; c < p.max_cols; c += 256) {
-    const int v = sHist[c];
-    if (v) atomicAdd(&p.segcnt[(((int64_t)b * a.heads + h) * p.nseg + seg) * p.max_cols + c], v);
+  for (int w0 = 0; w0 < p.W; w0 += WP) {
+    const int wn = min(WP, p.W - w0);
+    __syncthreads();  // the pass before has been written out
+    for (int v = tid; v < wn * kGateRows; v += 256) sSel[v] = 0u;
+    for (int c = tid; c < wn * 32; c += 256) sHist[c] = 0;
+    __syncthreads();
+    if (valid) {
+#pragma unroll
+      for (int j = 0; j < PL; ++j) {
+        const int e = 2 * j + hh;  // the two lanes of a row hold alternate entries of its list
+        if (e < m_fin) {
+          const int c = sIdx[((TWO_LISTS ? cur : 0) * kGateRows + rs) * CAP + e];
+          const int cw = (c >> 5) - w0;
+          if ((uint32_t)cw < (uint32_t)wn) {
+            atomicOr(&sSel[cw * kGateRows + rs], 1u << (c & 31));
+            atomicAdd(&sHist[c - 32 * w0], 1);
+          }
+        }
+      }
+      if (hh == 0 && a.is_causal && rp >= 0) {
+        const int c = rp / B;  // the own chunk is always selected
+        const int cw = (c >> 5) - w0;
+        if (c < p.max_cols && (uint32_t)cw < (uint32_t)wn) {
+          atomicOr(&sSel[cw * kGateRows + rs], 1u << (c & 31));
+          atomicAdd(&sHist[c - 32 * w0], 1);
+        }
+      }
+    }
+    __syncthreads();
+    for (int v = tid; v < wn * kGateRows; v += 256) {
+      const int t = v / kGateRows, slot_r = v - t * kGateRows;
+      if (m0 + slot_r < Lq) p.sel[((int64_t)h * p.W + w0 + t) * a.total_q + q0 + m0 + slot_r] = sSel[v];
+    }
+    for (int c = tid; c < wn * 32; c += 256) {
+      const int v = sHist[c];
+      if (v) atomicAdd(&p.segcnt[(((int64_t)b * a.heads + h) * p.nseg + seg) * p.max_cols + 32 * w0 + c], v);
+    }
   }
 }
 
@@ -703,9 +713,9 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
 //    beats it.  More than 16 entrants in some row of a wave, the first group, and rows whose list is not full yet
 //    take the bisection over this group's scores and the winners.
 // ------------------------------------------------------------------------------------
-// A winner is ONE double: order key of its score * 8192 + chunk (exact: below 2^45), so that the order "score
+// A winner is ONE double: order key of its score * 65536 + chunk (exact: below 2^48), so that the order "score
 // descending, chunk descending" is the order of the doubles and minimum / maximum are single instructions.
-constexpr double kChunkSpan = 8192.0;   // more chunks per sequence than the LDS of these kernels can hold anyway
+constexpr double kChunkSpan = 65536.0;  // chunk indices stay below it (checked on the host before the launch)
 constexpr double kSlotFiller = INFINITY;  // unused slot of a complete list: above every winner, never the weakest
 constexpr double kSlotEmpty = -1.0;       // unused slot of a list that is still filling: below every winner
 
@@ -755,10 +765,10 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
   constexpr int EW = kGateRows * LS + 256;    // words of an entrant array: the lists, then a trash word per thread
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint16_t *sKm = reinterpret_cast<uint16_t *>(smem);
-  uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [W][128], reuses the tile and the lists after the last group
+  uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [word columns of a pass][128], reuses the tile and the lists after the last group
   float *sEv = reinterpret_cast<float *>(smem + (size_t)GC * LD * 2);  // [EW] scores of the entrants
-  const size_t head = max((size_t)GC * LD * 2 + (size_t)2 * EW * 4, (size_t)p.W * kGateRows * 4);
-  int *sHist = reinterpret_cast<int *>(smem + head);                   // [max_cols]
+  constexpr size_t head = (size_t)GC * LD * 2 + (size_t)2 * EW * 4;
+  int *sHist = reinterpret_cast<int *>(smem + head);                   // [32 chunks per word column of a pass]
 
   const fmoba_fused_topk_args &a = p.a;
   const int mb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -1108,36 +1118,46 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
   }
   __syncthreads();
 
-  // selection words and per-chunk counts of the block, assembled in LDS
-  for (int v = tid; v < p.W * kGateRows; v += 256) sSel[v] = 0u;
-  for (int c = tid; c < p.max_cols; c += 256) sHist[c] = 0;
-  __syncthreads();
-  if (valid) {
-#pragma unroll
-    for (int j = 0; j < PL; ++j) {
-      if (winner_real(win[j])) {
-        const uint32_t c = (uint32_t)winner_chunk(win[j]);
-        atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
-        atomicAdd(&sHist[c], 1);
-      }
-    }
-    if (hh == 0 && a.is_causal && rp >= 0) {
-      const int c = rp / B;  // the own chunk is always selected
-      if (c < p.max_cols) {
-        atomicOr(&sSel[(c >> 5) * kGateRows + rs], 1u << (c & 31));
-        atomicAdd(&sHist[c], 1);
-      }
-    }
-  }
-  __syncthreads();
-  for (int v = tid; v < p.W * kGateRows; v += 256) {
-    const int t = v / kGateRows, slot_r = v - t * kGateRows;
-    if (m0 + slot_r < Lq) p.sel[((int64_t)h * p.W + t) * a.total_q + q0 + m0 + slot_r] = sSel[v];
-  }
+  // selection words and per-chunk counts of the block, assembled in LDS and written out in passes of WP word columns
+  // (what the tile and the lists hold), so that a sequence may have any number of chunks
+  const int WP = min(p.W, (int)(head / (kGateRows * 4)));
   const int seg = m0 / p.seg_rows;
-  for (int c = tid; c < p.max_cols; c += 256) {
-    const int v = sHist[c];
-    if (v) atomicAdd(&p.segcnt[(((int64_t)b * a.heads + h) * p.nseg + seg) * p.max_cols + c], v);
+  for (int w0 = 0; w0 < p.W; w0 += WP) {
+    const int wn = min(WP, p.W - w0);
+    __syncthreads();  // the pass before has been written out
+    for (int v = tid; v < wn * kGateRows; v += 256) sSel[v] = 0u;
+    for (int c = tid; c < wn * 32; c += 256) sHist[c] = 0;
+    __syncthreads();
+    if (valid) {
+#pragma unroll
+      for (int j = 0; j < PL; ++j) {
+        if (winner_real(win[j])) {
+          const int c = winner_chunk(win[j]);
+          const int cw = (c >> 5) - w0;
+          if ((uint32_t)cw < (uint32_t)wn) {
+            atomicOr(&sSel[cw * kGateRows + rs], 1u << (c & 31));
+            atomicAdd(&sHist[c - 32 * w0], 1);
+          }
+        }
+      }
+      if (hh == 0 && a.is_causal && rp >= 0) {
+        const int c = rp / B;  // the own chunk is always selected
+        const int cw = (c >> 5) - w0;
+        if (c < p.max_cols && (uint32_t)cw < (uint32_t)wn) {
+          atomicOr(&sSel[cw * kGateRows + rs], 1u << (c & 31));
+          atomicAdd(&sHist[c - 32 * w0], 1);
+        }
+      }
+    }
+    __syncthreads();
+    for (int v = tid; v < wn * kGateRows; v += 256) {
+      const int t = v / kGateRows, slot_r = v - t * kGateRows;
+      if (m0 + slot_r < Lq) p.sel[((int64_t)h * p.W + w0 + t) * a.total_q + q0 + m0 + slot_r] = sSel[v];
+    }
+    for (int c = tid; c < wn * 32; c += 256) {
+      const int v = sHist[c];
+      if (v) atomicAdd(&p.segcnt[(((int64_t)b * a.heads + h) * p.nseg + seg) * p.max_cols + 32 * w0 + c], v);
+    }
   }
 }
 
@@ -1359,18 +1379,17 @@ static int launch_gate_nt(const TopkParams &p, dim3 grid, hipStream_t s) {
   return launch_gate<T, HD, 8>(p, grid, s);
 }
 template <int HD, int NT, int CAP>
-static size_t gate_big_smem(const TopkParams &p) {
-  const size_t tile = (size_t)NT * 32 * (HD + 16) * 2;
-  if ((size_t)p.W * kGateRows * 4 > tile) return (size_t)1 << 30;  // the selection words reuse the tile
-  return tile + (size_t)(CAP <= kBigCap ? 2 : 1) * kGateRows * CAP * 8 + (size_t)2 * kGateRows * 4 + (size_t)p.max_cols * 4 + 256 * 4;
+static constexpr size_t gate_big_smem() {
+  const size_t tile = (size_t)NT * 32 * (HD + 16) * 2;  // chunk means of a group; later the selection words of a pass
+  const size_t hist = tile / (kGateRows * 4) * 32 * 4;   // counts of the chunks of a pass
+  return tile + (size_t)(CAP <= kBigCap ? 2 : 1) * kGateRows * CAP * 8 + (size_t)2 * kGateRows * 4 + hist + 256 * 4;
 }
+// chunk indices are 16-bit fields of the running winners (topk_gate_stream_kernel) and the forward's step lists
+constexpr int kMaxChunksPerSequence = 65535;
 template <typename T, int HD, int NT, int CAP>
 static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
-  const size_t smem = gate_big_smem<HD, NT, CAP>(p);
-  if (smem > 160 * 1024) {
-    set_error("fused_topk: %d key chunks per sequence exceed what the LDS of this build holds", p.max_cols);
-    return 1;
-  }
+  const size_t smem = gate_big_smem<HD, NT, CAP>();
+  static_assert(gate_big_smem<HD, NT, CAP>() <= 160 * 1024, "LDS of one compute unit");
   auto kern = topk_gate_big_kernel<T, HD, NT, CAP>;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("fused_topk: cannot reserve %zu bytes of LDS", smem);
@@ -1380,17 +1399,13 @@ static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
   return 0;
 }
 template <int HD, int NT>
-static size_t gate_stream_smem(const TopkParams &p) {
-  const size_t lists = (size_t)2 * (kGateRows * 18 + 256) * 4;
-  return std::max((size_t)NT * 32 * (HD + 16) * 2 + lists, (size_t)p.W * kGateRows * 4) + (size_t)p.max_cols * 4;
+static constexpr size_t gate_stream_smem() {
+  const size_t head = (size_t)NT * 32 * (HD + 16) * 2 + (size_t)2 * (kGateRows * 18 + 256) * 4;  // tile and lists; later the selection words of a pass
+  return head + head / (kGateRows * 4) * 32 * 4;
 }
 template <typename T, int HD, int NT>
 static int launch_gate_stream(const TopkParams &p, dim3 grid, hipStream_t s) {
-  const size_t smem = gate_stream_smem<HD, NT>(p);
-  if (smem > 160 * 1024 || p.max_cols > (int)kChunkSpan) {  // (the second follows from the first; the winners' encoding relies on it)
-    set_error("fused_topk: %d key chunks per sequence exceed what the LDS of this build holds", p.max_cols);
-    return 1;
-  }
+  const size_t smem = gate_stream_smem<HD, NT>();
   auto kern = topk_gate_stream_kernel<T, HD, NT>;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("fused_topk: cannot reserve %zu bytes of LDS", smem);
@@ -1460,6 +1475,7 @@ static int fused_topk_run(const fmoba_fused_topk_args *a, void *workspace, size_
     return 0;
   }
   const bool big = max_cols > 256;  // more chunks than the register-resident gate holds: grouped gate
+  FMOBA_REQUIRE(max_cols <= kMaxChunksPerSequence, "fused_topk: %d key chunks per sequence; at most %d are supported", max_cols, kMaxChunksPerSequence);
   FMOBA_REQUIRE(a->q && a->km, "fused_topk: null q/km pointer");
   FMOBA_REQUIRE(a->q_row_stride % 8 == 0 && a->q_head_stride % 8 == 0 && a->km_row_stride % 8 == 0 && a->km_head_stride % 8 == 0,
                 "fused_topk: strides must be multiples of 8 elements");

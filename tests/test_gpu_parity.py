@@ -233,6 +233,35 @@ def test_gating_more_than_256_chunks_exact_ties_long_lists(fm, causal):
     _check_gating(fm, q, k, cuq, cuk, 4, 50, causal, integer=True)
 
 
+@pytest.mark.parametrize("topk", [8, 33, 64])
+@pytest.mark.parametrize("lens", [[4096], [4500, 300], [8192]])
+def test_gating_4096_to_8192_chunks_exact_ties(fm, topk, lens):
+    # the chunk counts of the reference's own 2 x 524288-token benchmark point (4096) and beyond: the grouped gates
+    # write their selection words and counts out in several passes; top-k 8 keeps a row's winners in registers, 33 and
+    # 64 take the variants with 32 and 64 running winners per row
+    q, k, cuq, cuk = _gate_case(fm, 31, lens, lens, 2, 1, 64, 1, topk, True, integer=True)
+    _check_gating(fm, q, k, cuq, cuk, 1, topk, True, integer=True)
+
+
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("topk", [40, 64])
+def test_gating_long_lists_3000_chunks_every_head_dim(fm, D, topk):
+    # 64 running winners per row with thousands of chunks, at every width of the chunk-mean tile
+    q, k, cuq, cuk = _gate_case(fm, 32, [3000], [3000], 2, 2, D, 1, topk, True, integer=True)
+    _check_gating(fm, q, k, cuq, cuk, 1, topk, True, integer=True)
+    q, k, cuq, cuk = _gate_case(fm, 33, [2900, 200], [2900, 200], 2, 1, D, 1, topk, False, torch.float16)
+    _check_gating(fm, q, k, cuq, cuk, 1, topk, False)
+
+
+def test_gating_rejects_more_chunks_than_supported(fm):
+    # chunk indices are 16-bit fields inside the kernels: the call fails on the host, before anything is launched
+    T = 65536 + 8
+    q = torch.zeros((T, 1, 8), dtype=torch.bfloat16).cuda()
+    cu = torch.tensor([0, T], dtype=torch.int32).cuda()
+    with pytest.raises(RuntimeError, match="at most 65535 are supported"):
+        fm.hip.moba_fused_topk(q, q, cu, cu, cu, T, T, 4, 1, True, return_raw=False)
+
+
 def test_gating_no_keys(fm):
     q = torch.randn(10, 2, 64).to(torch.bfloat16).cuda()
     km = torch.zeros(0, 2, 64, dtype=torch.bfloat16).cuda()
