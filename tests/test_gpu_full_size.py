@@ -17,7 +17,7 @@ from gpu_utils import csc_selection_one_head, dense_ref_one_head
 pytestmark = pytest.mark.gpu
 
 
-def _inputs(seqlens, H, D, chunk, seed):
+def _inputs(seqlens, H, D, chunk, seed, dtype=torch.bfloat16):
     g = torch.Generator(device="cuda").manual_seed(seed)
     T = sum(seqlens)
     q = torch.randn((T, H, D), generator=g, device="cuda")
@@ -30,8 +30,7 @@ def _inputs(seqlens, H, D, chunk, seed):
         k[pos:pos + L] += (0.5 * torch.randn((C, H, D), generator=g, device="cuda")).repeat_interleave(chunk, 0)[:L]
         pos += L
     cu = torch.tensor([0] + list(np.cumsum(seqlens)), dtype=torch.int32, device="cuda")
-    bf = torch.bfloat16
-    return q.to(bf), k.to(bf), v.to(bf), dout.to(bf), cu
+    return q.to(dtype), k.to(dtype), v.to(dtype), dout.to(dtype), cu
 
 
 def _check_csc(co, cn, ind, seqlens, H, chunk, topk):
@@ -127,7 +126,17 @@ def test_config3_fwd_bwd_32k(mods):
     q, k, v, dout, cu = _inputs(seqlens, H, D, chunk, 1003)
     co, cn, ind = api.flash_topk_varlen_func(q, k, cu, cu, 32768, 32768, topk, chunk, causal=True)
     _check_csc(co, cn, ind, seqlens, H, chunk, topk)
-    _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, [(0, 5)], grads=True, csc=(co, cn, ind))
+    _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, [(0, 5), (0, 17), (0, 31)], grads=True, csc=(co, cn, ind))
+
+
+def test_sweep_point_2x16k_fp16_fwd_bwd(mods):
+    # a point of the reference's own sweep (benchmarks/bench_flash_moba.py:66-78: batch 2, 16 heads of 128, fp16, chunk 128, top-k 8)
+    api, pool = mods
+    seqlens, H, D, chunk, topk = [16384, 16384], 16, 128, 128, 8
+    q, k, v, dout, cu = _inputs(seqlens, H, D, chunk, 1006, torch.float16)
+    co, cn, ind = api.flash_topk_varlen_func(q, k, cu, cu, 16384, 16384, topk, chunk, causal=True)
+    _check_csc(co, cn, ind, seqlens, H, chunk, topk)
+    _sampled_dense_check(api, pool, q, k, v, dout, cu, seqlens, chunk, topk, [(0, 3), (1, 12)], grads=True, csc=(co, cn, ind))
 
 
 def test_config4_headline_fwd_bwd_64k(mods):
@@ -209,6 +218,26 @@ def test_config5_long_context_262k(mods):
             assert bool(((out[r, h].float() - o_ref).abs() <= 2e-2 + 1e-2 * o_ref.abs()).all()), (r, h)
             assert bool(((qg.grad[r, h].float() - dq_ref).abs() <= 2e-2 + 1e-2 * dq_ref.abs()).all()), (r, h)
     assert checked >= 16
+    # dK and dV of three key chunks (first, middle, last) of two heads, in fp32 from the kernel's own lists and LSE:
+    #   P = exp(scale q k^T - lse), dV_j = sum_r P_rj dO_r, dS = P o (dO v^T - delta), dK_j = scale sum_r dS_rj q_r
+    lg = api.flash_moba_interface.decide_lg_block_m(topk, chunk, L, True)
+    _, lse, _ = api.flash_moba_attn_varlen_func(q, k, v, cu, cu, L, L, co, cn, ind, lg, chunk, causal=True, return_attn_probs=True)
+    for h in (3, 14):
+        for c in (0, 1023, 2047):
+            n, o0 = int(cn[0, h, c]), int(co[0, h, c])
+            assert n >= chunk
+            rows = ind[o0:o0 + n].long()
+            keys = torch.arange(c * chunk, (c + 1) * chunk, device=q.device)
+            qr, dor = q[rows, h].float(), dout[rows, h].float()
+            kc, vc = k[keys, h].float(), v[keys, h].float()
+            p_ = torch.exp(scale * (qr @ kc.T) - lse[h, rows][:, None])
+            p_ = torch.where(keys[None, :] <= rows[:, None], p_, torch.zeros_like(p_))
+            delta = (dor * out[rows, h].float()).sum(-1, keepdim=True)
+            ds = p_ * (dor @ vc.T - delta)
+            dv_ref, dk_ref = p_.T @ dor, scale * (ds.T @ qr)
+            for name, got, ref in (("dv", vg.grad[keys, h].float(), dv_ref), ("dk", kg.grad[keys, h].float(), dk_ref)):
+                nbad = int(((got - ref).abs() > 2e-2 + 1e-2 * ref.abs()).sum())
+                assert nbad == 0, (name, h, c, nbad, (got - ref).abs().max().item())
     # every probability row sums to one: sum_j dV_j = sum_r dO_r, per head and feature
     lhs, rhs = vg.grad.float().sum(0), dout.float().sum(0)
     assert bool(((lhs - rhs).abs() <= 2e-2 * rhs.abs().max()).all()), (lhs - rhs).abs().max().item()

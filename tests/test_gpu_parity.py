@@ -429,6 +429,25 @@ def test_attention_random_pattern(fm, sq, sk, d, mha, causal, dtype):
     _check_attention(fm, q, k, v, dout, cuq, cuk, co, cn, ind, 64, causal)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("d,mha,dtype", [(64, "mha", torch.bfloat16), (128, "gqa", torch.bfloat16), (128, "mqa", torch.float16), (80, "mha", torch.float16)])
+@pytest.mark.parametrize("sq,sk", [(1, 147), (113, 211), (108, 256), (1024, 1024), (1024, 1023), (2048, 2048), (4096, 4096)])
+def test_attention_random_pattern_remaining_reference_shapes(fm, sq, sk, d, mha, causal, dtype):
+    # the other shapes of tests/test_moba_attn.py:52-65; a batch whose longest query sequence has ONE row takes the
+    # "max_seqlen_q == 1 => not causal" rule of csrc/flash_moba/flash_moba_api.cpp:450 (the oracle applies it too)
+    big = max(sq, sk) >= 2048
+    H = 4 if big else 6
+    Hk = {"mha": H, "gqa": 2, "mqa": 1}[mha]
+    rng = np.random.RandomState(sq * 3 + sk)
+    nb = 2 if big else 3
+    lens_q = [max(1, sq - int(x)) for x in rng.randint(0, 20, nb)]
+    lens_k = [max(1, sk - int(x)) for x in rng.randint(0, 20, nb)]
+    q, k, v, dout, cuq, cuk = _attn_inputs(sq, lens_q, lens_k, H, Hk, d, dtype)
+    eff_causal = causal and max(lens_q) > 1
+    co, cn, ind = _random_csc(4, lens_q, lens_k, H, 64, 4, eff_causal)
+    _check_attention(fm, q, k, v, dout, cuq, cuk, co, cn, ind, 64, causal)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("mha", ["mha", "gqa"])
