@@ -351,7 +351,9 @@ class FlashMobaAttnVarlenFunc(torch.autograd.Function):
     Two trailing arguments beyond the reference's twenty, both optional: max_visits, the bound on a row's visits in
     forward key blocks when the caller knows it (a gated pattern: top-k * lg_block_n / key block), and the gating's
     selection bits.  Without a bound it is counted from the pattern once, here (eager mode; one device-to-host read)
-    or inside each op (while a graph is being traced, where a data-dependent integer cannot leave an op)."""
+    or inside each op (while a graph is being traced or captured, where a data-dependent integer cannot leave an op).
+    A caller's bound without selection bits is checked against the pattern in eager mode and raises if a row has more
+    visits; under tracing or capture it is taken as given."""
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
@@ -364,13 +366,25 @@ class FlashMobaAttnVarlenFunc(torch.autograd.Function):
         flash_moba_gpu._reject_unsupported(dropout_p, softcap, alibi_slopes, None, None, return_softmax and dropout_p > 0)
         head_size_og = q.size(2)
         q, k, v = _pad8(q, k, v)
+        can_read_back = not (torch.compiler.is_compiling() or (q.is_cuda and torch.cuda.is_current_stream_capturing()))
         if max_visits is None:
-            if torch.compiler.is_compiling() or lg_block_n <= 0 or lg_block_n % 64 != 0:
+            if not can_read_back or lg_block_n <= 0 or lg_block_n % 64 != 0:
                 max_visits = -1  # counted inside the ops (a malformed lg_block_n is reported there)
             else:
                 max_visits = flash_moba_gpu.count_max_visits(
                     q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k, k.shape[0], k.shape[1],
                     max_seqlen_q, max_seqlen_k, lg_block_n)
+        elif selection_bits is None and can_read_back and lg_block_n > 0 and lg_block_n % 64 == 0:
+            # A bound of the caller's own for a pattern of the caller's own (the gated path hands its selection bits
+            # along, and its bound, top-k, cannot be exceeded): visits beyond it would be dropped, so it is checked
+            # against the pattern here (one device-to-host read).  While a graph is traced or captured nothing can be
+            # read back: there the caller answers for the bound (the raw entry points report a violation through
+            # their visits_overflow word).
+            actual = flash_moba_gpu.count_max_visits(
+                q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k, k.shape[0], k.shape[1],
+                max_seqlen_q, max_seqlen_k, lg_block_n)
+            if actual > max_visits:
+                raise RuntimeError(f"max_visits = {max_visits}, but a row of the pattern has {actual} (row, key block) visits")
         out_padded, softmax_lse, S_dmask, rng_state = _wrapped_attn_varlen_forward_bounded(
             q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
             moba_col_offsets, moba_col_nnz, moba_row_indices, lg_block_m, lg_block_n,

@@ -100,7 +100,8 @@ int fmoba_fused_topk(const fmoba_fused_topk_args *a, void *stream);
  * that limit (the headline shape -- 65536 tokens, 16 heads, 224 chunks -- needs 30.3 MB and fits).
  * It calls no hipMalloc / hipFree.  All calls on one device share the array: calls that overlap on one
  * device (different streams or threads) race; calls in stream order are safe, every call clears what
- * it needs zeroed with a fill kernel of its own. */
+ * it needs zeroed with a fill kernel of its own.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress): make it outside any stream capture. */
 #define FMOBA_STATIC_SCRATCH_BYTES (32u << 20)
 int fmoba_fused_topk_static(const fmoba_fused_topk_args *a, void *stream);
 

@@ -519,6 +519,20 @@ def test_forward_both_forms(fm, form, sq, sk, d, Hk, chunk, topk, causal, dtype)
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
 
 
+def test_autograd_function_checks_a_callers_visit_bound(fm):
+    # FlashMobaAttnVarlenFunc takes an optional bound on a row's visits; one that is too small for the caller's own
+    # pattern would drop visits, so eager calls check it against the pattern
+    lens = [700, 300]
+    q, k, v, dout, cuq, cuk = _attn_inputs(2, lens, lens, 2, 2, 64, torch.bfloat16)
+    co, cn, ind = _random_csc(5, lens, lens, 2, 64, 4, True)
+    args = (q.cuda(), k.cuda(), v.cuda(), cuq.cuda(), cuk.cuda(), 700, 700, co.cuda(), cn.cuda(), ind.cuda(), 128, 64,
+            0.0, None, True, 0.0, None, False, False, False)
+    ref = fm.iface.FlashMobaAttnVarlenFunc.apply(*args)
+    assert torch.equal(fm.iface.FlashMobaAttnVarlenFunc.apply(*args, 4), ref)
+    with pytest.raises(RuntimeError, match="max_visits = 2, but a row of the pattern has 4"):
+        fm.iface.FlashMobaAttnVarlenFunc.apply(*args, 2)
+
+
 @pytest.mark.parametrize("lens,chunk,topk,Hk", [([640, 1, 0, 1300], 64, 6, 4), ([2100, 900], 128, 5, 2), ([300 * 64 + 17], 64, 33, 1)])
 def test_fused_path_hands_the_gating_selection_to_the_forward(fm, lens, chunk, topk, Hk):
     # flash_moba_varlen_func passes the gating's selection bits on; the attention entry point alone derives them from
