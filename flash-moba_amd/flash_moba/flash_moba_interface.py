@@ -366,15 +366,19 @@ class FlashMobaAttnVarlenFunc(torch.autograd.Function):
         flash_moba_gpu._reject_unsupported(dropout_p, softcap, alibi_slopes, None, None, return_softmax and dropout_p > 0)
         head_size_og = q.size(2)
         q, k, v = _pad8(q, k, v)
-        can_read_back = not (torch.compiler.is_compiling() or (q.is_cuda and torch.cuda.is_current_stream_capturing()))
+        def can_read_back():  # a device-to-host read is possible: not while tracing (fake tensors) or capturing a graph
+            if torch.compiler.is_compiling() or torch._subclasses.fake_tensor.is_fake(q) or not q.is_cuda:
+                return False
+            return not torch.cuda.is_current_stream_capturing()
+
         if max_visits is None:
-            if not can_read_back or lg_block_n <= 0 or lg_block_n % 64 != 0:
+            if lg_block_n <= 0 or lg_block_n % 64 != 0 or not can_read_back():
                 max_visits = -1  # counted inside the ops (a malformed lg_block_n is reported there)
             else:
                 max_visits = flash_moba_gpu.count_max_visits(
                     q, moba_col_offsets, moba_col_nnz, moba_row_indices, cu_seqlens_q, cu_seqlens_k, k.shape[0], k.shape[1],
                     max_seqlen_q, max_seqlen_k, lg_block_n)
-        elif selection_bits is None and can_read_back and lg_block_n > 0 and lg_block_n % 64 == 0:
+        elif selection_bits is None and lg_block_n > 0 and lg_block_n % 64 == 0 and can_read_back():
             # A bound of the caller's own for a pattern of the caller's own (the gated path hands its selection bits
             # along, and its bound, top-k, cannot be exceeded): visits beyond it would be dropped, so it is checked
             # against the pattern here (one device-to-host read).  While a graph is traced or captured nothing can be
