@@ -69,7 +69,42 @@ __global__ __launch_bounds__(256) void mean_pool_kernel(fmoba_mean_pool_args a) 
   }
 }
 
+// cu_km[b] = sum over b' < b of ceil(len_b' / chunk): one block, every thread a contiguous run of sequences.
+__global__ __launch_bounds__(256) void chunk_offsets_kernel(const int32_t *cu, int32_t *cu_km, int batch, int chunk) {
+  __shared__ int part[256];
+  const int tid = threadIdx.x;
+  const int per = (batch + 255) / 256;
+  const int lo = min(batch, tid * per), hi = min(batch, lo + per);
+  int s = 0;
+  for (int b = lo; b < hi; ++b) s += (cu[b + 1] - cu[b] + chunk - 1) / chunk;
+  part[tid] = s;
+  __syncthreads();
+  // inclusive scan over the 256 partial sums
+  for (int d = 1; d < 256; d <<= 1) {
+    const int v = tid >= d ? part[tid - d] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = part[tid] - s;
+  for (int b = lo; b < hi; ++b) {
+    cu_km[b] = run;
+    run += (cu[b + 1] - cu[b] + chunk - 1) / chunk;
+  }
+  if (tid == 255) cu_km[batch] = part[255];
+}
+
 }  // namespace fmoba
+
+extern "C" int fmoba_chunk_offsets(const int32_t *cu_seqlens, int32_t *cu_seqlens_km, int32_t batch, int32_t chunk, void *stream) {
+  using namespace fmoba;
+  FMOBA_REQUIRE(batch > 0, "chunk_offsets: batch size must be positive");
+  FMOBA_REQUIRE(chunk > 0, "chunk_offsets: chunk size must be positive");
+  FMOBA_REQUIRE(cu_seqlens && cu_seqlens_km, "chunk_offsets: null pointer");
+  hipLaunchKernelGGL(chunk_offsets_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, cu_seqlens, cu_seqlens_km, batch, chunk);
+  FMOBA_LAUNCH_CHECK("chunk_offsets");
+  return 0;
+}
 
 extern "C" int fmoba_mean_pool(const fmoba_mean_pool_args *a, void *stream) {
   using namespace fmoba;

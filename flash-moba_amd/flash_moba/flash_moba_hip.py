@@ -85,6 +85,7 @@ EXPORTS = {
     "fmoba_last_error": (ctypes.c_char_p, []),
     "fmoba_check_device": (c_i32, []),
     "fmoba_mean_pool": (c_i32, [ctypes.POINTER(MeanPoolArgs), c_vp]),
+    "fmoba_chunk_offsets": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_vp]),
     "fmoba_fused_topk_workspace_bytes": (c_sz, [c_i32, c_i32, c_i32, c_i32, c_i32, c_i32]),
     "fmoba_fused_topk": (c_i32, [ctypes.POINTER(FusedTopkArgs), c_vp]),
     "fmoba_fused_topk_static": (c_i32, [ctypes.POINTER(FusedTopkArgs), c_vp]),
@@ -180,6 +181,19 @@ def mean_pool(k: torch.Tensor, km: torch.Tensor, cu_seqlens_k: torch.Tensor, cu_
                          batch, int(max_chunks), k.shape[1], k.shape[2], int(chunk), _dt(k),
                          k.stride(0), k.stride(1), km.stride(0), km.stride(1))
         _check(load_library().fmoba_mean_pool(ctypes.byref(a), _stream()))
+
+
+def chunk_offsets(cu_seqlens: torch.Tensor, chunk: int) -> torch.Tensor:
+    """cu_seqlens of the pooled sequences: cumsum(ceil(len / chunk)) with a leading zero, int32, one launch
+    (the tensor expressions of flash_moba/triton_mean_pool.py:132-139)."""
+    batch = cu_seqlens.numel() - 1
+    _require(batch > 0, "batch size must be positive")
+    _check_cu("cu_seqlens", cu_seqlens, batch)
+    _require(chunk > 0, "chunk size must be positive")
+    with _device_guard(cu_seqlens):
+        out = torch.empty_like(cu_seqlens)
+        _check(load_library().fmoba_chunk_offsets(cu_seqlens.data_ptr(), out.data_ptr(), batch, int(chunk), _stream()))
+    return out
 
 
 # --------------------------------------------------------------------------------------

@@ -11,6 +11,8 @@ from flash_moba import flash_moba_hip as _hip
 
 def chunk_cu_seqlens(cu_seqlens: torch.Tensor, chunk: int) -> torch.Tensor:
     """cu_seqlens of the pooled sequences: cumsum(ceil(len / chunk)), int32, on the same device."""
+    if cu_seqlens.is_cuda and cu_seqlens.dtype == torch.int32 and cu_seqlens.is_contiguous() and cu_seqlens.numel() > 1 and chunk > 0:
+        return _hip.chunk_offsets(cu_seqlens, chunk)  # one launch instead of six
     lens = cu_seqlens[1:] - cu_seqlens[:-1]
     chunks = torch.div(lens + (chunk - 1), chunk, rounding_mode="floor")
     out = torch.zeros_like(cu_seqlens, dtype=torch.int32)

@@ -57,6 +57,10 @@ typedef struct {
   int64_t km_row_stride, km_head_stride;
 } fmoba_mean_pool_args;
 int fmoba_mean_pool(const fmoba_mean_pool_args *a, void *stream);
+/* cu_seqlens_km[b] = sum over b' < b of ceil((cu_seqlens[b'+1] - cu_seqlens[b']) / chunk), b = 0 .. batch: the offsets of
+ * the pooled sequences, in one launch.  Replaces the tensor expressions of flash_topk_mean_pool
+ * (flash_moba/triton_mean_pool.py:132-139: lengths, ceil-division, cumulative sum, padding with a leading zero). */
+int fmoba_chunk_offsets(const int32_t *cu_seqlens, int32_t *cu_seqlens_km, int32_t batch, int32_t chunk, void *stream);
 
 /* ------------------------------------------------------------------------------------
  * Fused top-k block gating + CSC build.

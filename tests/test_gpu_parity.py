@@ -71,6 +71,19 @@ def test_mean_pool_all_empty_and_strided(fm):
     assert torch.allclose(km.cpu().float(), ref.float(), atol=1e-2)
 
 
+@pytest.mark.parametrize("batch,chunk", [(1, 64), (3, 128), (8, 64), (255, 1), (256, 7), (257, 64), (1000, 33), (5000, 128)])
+def test_chunk_offsets_match_the_tensor_expression(fm, batch, chunk):
+    # flash_moba/triton_mean_pool.py:132-139: lengths, ceil-division, cumulative sum, a leading zero
+    rng = np.random.RandomState(batch * 131 + chunk)
+    lens = rng.randint(0, 700, batch)
+    lens[rng.randint(0, batch, max(1, batch // 7))] = 0
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    want = torch.zeros(batch + 1, dtype=torch.int32)
+    want[1:] = torch.cumsum(torch.div(cu[1:] - cu[:-1] + (chunk - 1), chunk, rounding_mode="floor"), 0)
+    got = fm.hip.chunk_offsets(cu.cuda(), chunk)
+    assert got.dtype == torch.int32 and torch.equal(got.cpu(), want)
+
+
 # ------------------------------------------------------------------------ gating + CSC
 def _gate_case(fm, seed, lens_q, lens_k, H, Hk, D, chunk, topk, causal, dtype=torch.bfloat16, integer=False):
     g = torch.Generator().manual_seed(seed)
