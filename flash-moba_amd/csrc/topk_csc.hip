@@ -756,18 +756,18 @@ template <typename T, int HD, int NT>
 __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(TopkParams p) {
   constexpr int CAP = 16, PL = 8;
   constexpr int KS = HD / 16;
-  constexpr int LD = HD + 16;
   constexpr int GC = NT * 32;             // chunks per group
   constexpr int VPR = HD / 8;             // 16-byte pieces of a row of chunk means
-  constexpr int NV = GC * VPR / 256;      // ... of a group's tile per thread
-  static_assert(GC * VPR % 256 == 0, "the tile is loaded in whole passes of the workgroup");
+  constexpr int RPI = 64 / VPR;           // tile rows one load instruction brings (64 lanes x 16 bytes)
+  constexpr int NV = GC / RPI / 4;        // load instructions per wave and tile
+  static_assert(NV >= 1 && NV * RPI * 4 == GC, "the four waves share a tile evenly");
+  constexpr int RB = HD * 2;              // bytes of a tile row: exactly HD elements, swizzled instead of padded
   constexpr int LS = CAP + 2;                 // slots of a row's list: 16 entries and the two lanes' next slots
   constexpr int EW = kGateRows * LS + 256;    // words of an entrant array: the lists, then a trash word per thread
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint16_t *sKm = reinterpret_cast<uint16_t *>(smem);
   uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [word columns of a pass][128], reuses the tile and the lists after the last group
-  float *sEv = reinterpret_cast<float *>(smem + (size_t)GC * LD * 2);  // [EW] scores of the entrants
-  constexpr size_t head = (size_t)GC * LD * 2 + (size_t)2 * EW * 4;
+  float *sEv = reinterpret_cast<float *>(smem + (size_t)GC * RB);  // [EW] scores of the entrants
+  constexpr size_t head = (size_t)GC * RB + (size_t)2 * EW * 4;
   int *sHist = reinterpret_cast<int *>(smem + head);                   // [32 chunks per word column of a pass]
 
   const fmoba_fused_topk_args &a = p.a;
@@ -815,15 +815,25 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
   const int kp = a.is_causal ? a.topk - 1 : a.topk;
 
   const uint16_t *kmp = reinterpret_cast<const uint16_t *>(a.km) + (int64_t)hk * a.km_head_stride;
-  Pack8 pre[NV];
-  auto fetch = [&](int g) {
+  // The chunk means of a group go from global memory straight into the LDS tile (global_load_lds: no registers hold
+  // them on the way), every wave a quarter of the rows, issued as soon as the scores of the group before have been
+  // formed and awaited at the top of the next group: the rest of a group's work runs under them.  Piece c of tile row
+  // r lies at piece c ^ tile_swz<HD>(r).  Rows past the last chunk that can be a candidate and features past head_dim
+  // are fetched from a row / piece that exists: such scores are masked, such features meet zeros of q.
+  const uint32_t ldsTile = (uint32_t)(uintptr_t)smem;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  auto tile_issue = [&](int g) {
     const int c0 = g * GC, gsc = min(GC, nsc - c0);
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-      const int x = tid + v * 256, c = x / VPR, e = (x - c * VPR) * 8;
-      pre[v] = (c < gsc && e < D) ? ld_global16(kmp + (int64_t)(km0 + c0 + c) * a.km_row_stride + e) : zero_pack8();
+      const int c = (wave_u * NV + v) * RPI + lane / VPR, pc = lane % VPR;
+      const int e = min((pc ^ tile_swz<HD>(c)) * 8, D - 8);
+      global_to_lds16(kmp + (int64_t)(km0 + c0 + min(c, gsc - 1)) * a.km_row_stride + e, ldsTile + (uint32_t)((wave_u * NV + v) * 1024));
     }
   };
+  // this lane's operand row of a 32-chunk tile: row lane % 32, pieces hh * KS ..
+  const uint32_t a_row = ldsTile + (uint32_t)((lane & 31) * RB);
+  const int a_swz = tile_swz<HD>(lane & 31);
   double win[PL];  // this lane's share of the row's winners, ascending (win[0] is the weakest the lane holds)
 #pragma unroll
   for (int j = 0; j < PL; ++j) win[j] = kSlotEmpty;
@@ -832,20 +842,14 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
   float *const my_trash = sEv + kGateRows * LS + tid;
   constexpr int kToIdx = EW;  // from a score of the entrant arrays to its chunk, in words
 
-  if (ngroups > 0) fetch(0);
+  if (ngroups > 0) tile_issue(0);
 #pragma nounroll
   for (int g = 0; g < ngroups; ++g) {
     const int c0 = g * GC;
     const int gsc = min(GC, nsc - c0);
     const int n_tiles = (gsc + 31) >> 5;
-    __syncthreads();  // the previous group's tile is no longer read
-#pragma unroll
-    for (int v = 0; v < NV; ++v) {
-      const int x = tid + v * 256, c = x / VPR, e = (x - c * VPR) * 8;
-      *reinterpret_cast<Pack8 *>(sKm + c * LD + e) = pre[v];
-    }
-    if (g + 1 < ngroups) fetch(g + 1);
-    __syncthreads();
+    wait_all_loads();
+    __syncthreads();  // this group's tile is in LDS
 
     // this group's scores; chunks that are no candidates of the row (its own chunk and later ones) count as -inf
     float sc[NT][16];
@@ -858,7 +862,7 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const Pack8 af = *reinterpret_cast<const Pack8 *>(sKm + (t * 32 + (lane & 31)) * LD + (hh * KS + ks) * 8);
+          const Pack8 af = lds_read16(a_row + (uint32_t)(t * 32 * RB) + (uint32_t)(((hh * KS + ks) ^ a_swz) * 16));
           acc = mfma32<T>(af, qf[ks], acc);
         }
         if (all_cand) {
@@ -873,6 +877,8 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
         for (int i = 0; i < 16; ++i) sc[t][i] = -INFINITY;
       }
     }
+    __syncthreads();  // everyone has read the tile: the next group's chunk means may land in it
+    if (g + 1 < ngroups) tile_issue(g + 1);
 
     // ---- later groups: streaming update ---------------------------------------------------------
     // A row that still has candidates in this group had at least GC of them in the first one, so it already holds
@@ -1400,7 +1406,7 @@ static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
 }
 template <int HD, int NT>
 static constexpr size_t gate_stream_smem() {
-  const size_t head = (size_t)NT * 32 * (HD + 16) * 2 + (size_t)2 * (kGateRows * 18 + 256) * 4;  // tile and lists; later the selection words of a pass
+  const size_t head = (size_t)NT * 32 * HD * 2 + (size_t)2 * (kGateRows * 18 + 256) * 4;  // tile and lists; later the selection words of a pass
   return head + head / (kGateRows * 4) * 32 * 4;
 }
 template <typename T, int HD, int NT>
