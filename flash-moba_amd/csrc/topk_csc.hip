@@ -62,10 +62,11 @@ __device__ __forceinline__ int count4_gt(int n, float x0, float x1, float x2, fl
 template <typename T, int HD, int NT>
 __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_kernel(TopkParams p) {
   constexpr int KS = HD / 16;
-  constexpr int LD = HD + 16;  // LDS row stride (elements)
+  constexpr int VPR = HD / 8;    // 16-byte pieces of a row of chunk means
+  constexpr int RPI = 64 / VPR;  // tile rows one load instruction brings (64 lanes x 16 bytes)
+  constexpr int RB = HD * 2;     // bytes of a tile row: exactly HD elements, swizzled instead of padded
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint16_t *sKm = reinterpret_cast<uint16_t *>(smem);
-  int *sHist = reinterpret_cast<int *>(smem + (size_t)NT * 32 * LD * 2);
+  int *sHist = reinterpret_cast<int *>(smem + (size_t)NT * 32 * RB);
 
   const fmoba_fused_topk_args &a = p.a;
   const int mb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -93,18 +94,22 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
   nsc = min(nsc, min(p.max_cols, NT * 32));  // never beyond the LDS tile, whatever max_seqlen_k the caller gave
   const int n_tiles = (nsc + 31) >> 5;
 
-  // stage the chunk means of this (sequence, kv head) in LDS, zero padded
-  {
+  // The chunk means of this (sequence, kv head) go from global memory straight into LDS (global_load_lds, all loads
+  // of a wave in flight at once): piece c of tile row r lies at piece c ^ tile_swz<HD>(r).  Rows past the last chunk
+  // that can be a candidate and features past head_dim are fetched from a row / piece that exists: such scores are
+  // masked below, such features meet zeros of q.
+  const uint32_t ldsTile = (uint32_t)(uintptr_t)smem;
+  if (nsc > 0) {
     const uint16_t *kmp = reinterpret_cast<const uint16_t *>(a.km) + (int64_t)hk * a.km_head_stride;
-    const int vecs = HD / 8;
-    for (int v = tid; v < n_tiles * 32 * vecs; v += 256) {
-      const int c = v / vecs, e = (v - c * vecs) * 8;
-      Pack8 x = zero_pack8();
-      if (c < nsc && e < D) x = ld_global16(kmp + (int64_t)(km0 + c) * a.km_row_stride + e);
-      *reinterpret_cast<Pack8 *>(sKm + c * LD + e) = x;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int ninstr = n_tiles * 32 / RPI;
+    for (int v = wave_u; v < ninstr; v += 4) {
+      const int c = v * RPI + lane / VPR, pc = lane % VPR;
+      const int e = min((pc ^ tile_swz<HD>(c)) * 8, D - 8);
+      global_to_lds16(kmp + (int64_t)(km0 + min(c, nsc - 1)) * a.km_row_stride + e, ldsTile + (uint32_t)v * 1024u);
     }
-    for (int v = tid; v < NT * 32; v += 256) sHist[v] = 0;
   }
+  for (int v = tid; v < NT * 32; v += 256) sHist[v] = 0;
 
   // this lane's query row and its operand slices (contraction index permuted so that each
   // half-wave reads one contiguous half of the row)
@@ -119,6 +124,7 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
       qf[ks] = (valid && e < D) ? ld_global16(qp + e) : zero_pack8();
     }
   }
+  wait_all_loads();
   __syncthreads();
 
   // scores: lane (query l%32) gets chunk t*32 + acc_row(i, hh) in register i of tile t;
@@ -140,7 +146,7 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
       for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const Pack8 af = *reinterpret_cast<const Pack8 *>(sKm + (t * 32 + (lane & 31)) * LD + (hh * KS + ks) * 8);
+        const Pack8 af = lds_read16(ldsTile + (uint32_t)((t * 32 + (lane & 31)) * RB) + (uint32_t)(((hh * KS + ks) ^ tile_swz<HD>(lane & 31)) * 16));
         acc = mfma32<T>(af, qf[ks], acc);
       }
 #pragma unroll
@@ -1369,7 +1375,7 @@ extern "C" size_t fmoba_fused_topk_workspace_bytes(int32_t batch, int32_t total_
 namespace fmoba {
 template <typename T, int HD, int NT>
 static int launch_gate(const TopkParams &p, dim3 grid, hipStream_t s) {
-  const size_t smem = (size_t)NT * 32 * (HD + 16) * 2 + (size_t)NT * 32 * 4;
+  const size_t smem = (size_t)NT * 32 * HD * 2 + (size_t)NT * 32 * 4;
   auto kern = topk_gate_kernel<T, HD, NT>;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("fused_topk: cannot reserve %zu bytes of LDS", smem);
