@@ -7,6 +7,10 @@
 // twice.  Longer segments ping-pong between the output and a caller-provided workspace.
 // Offsets are 64-bit throughout.
 //
+// Before the radix passes a segment tries the shortcut that row lists allow: keys that do not repeat and span less
+// than 32 (64 for the segments that go through HBM) times the buffer size are marked in a bitmap in LDS and enumerated
+// in order (bitmap_sort); a repeated key sends the segment to the radix passes.
+//
 // A counting pass is stable without any order between the waves: every wave owns a contiguous
 // block of the keys and a histogram of its own; after the scan, bin d of wave w starts where the
 // keys of smaller digits and the digit-d keys of waves before w end.  A wave then walks its block
@@ -91,9 +95,51 @@ __device__ __forceinline__ void radix_pass(Load load, Store store, int64_t n, in
   __syncthreads();
 }
 
-// range of the biased keys of the workgroup's segment -> number of byte passes (0: all keys equal)
+// Keys that do not repeat and whose range fits a bitmap in LDS need no radix pass: every key sets bit `key - mn`, the
+// set bits are counted per thread (a contiguous block of words each), scanned, and enumerated in order.  Returns false,
+// with nothing stored, when a key repeats (the caller then runs the radix passes).  `bits` holds nw words, red WAVES.
+template <int WAVES, typename Load, typename Store>
+__device__ __forceinline__ bool bitmap_sort(Load load, Store store, int64_t n, uint32_t mn, int nw, uint32_t *bits, uint32_t *red) {
+  constexpr int kThreads = WAVES * 64;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < nw; i += kThreads) bits[i] = 0u;
+  __syncthreads();
+  int dup = 0;
+  for (int64_t i = tid; i < n; i += kThreads) {
+    const uint32_t b = load(i) - mn;
+    const uint32_t m = 1u << (b & 31u);
+    dup |= (atomicOr(&bits[b >> 5], m) & m) != 0u;
+  }
+  if (__syncthreads_or(dup)) return false;
+  const int per = (nw + kThreads - 1) / kThreads;
+  const int w0 = min(nw, tid * per), w1 = min(nw, w0 + per);
+  int cnt = 0;
+  for (int w = w0; w < w1; ++w) cnt += __popc(bits[w]);
+  int incl = cnt;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int t = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += t;
+  }
+  if (lane == 63) red[wave] = (uint32_t)incl;
+  __syncthreads();
+  int pos = incl - cnt;
+  for (int w = 0; w < wave; ++w) pos += (int)red[w];
+  for (int w = w0; w < w1; ++w) {
+    uint32_t x = bits[w];
+    const uint32_t k0 = mn + 32u * (uint32_t)w;
+    while (x) {
+      store(pos++, k0 + (uint32_t)(__ffs((int)x) - 1));
+      x &= x - 1u;
+    }
+  }
+  __syncthreads();
+  return true;
+}
+
+// range of the biased keys of the workgroup's segment -> number of byte passes (0: all keys equal); mn, mx: the range
 template <int WAVES>
-__device__ __forceinline__ int radix_passes(uint32_t mn, uint32_t mx, uint32_t *red) {
+__device__ __forceinline__ int radix_passes(uint32_t &mn, uint32_t &mx, uint32_t *red) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) {
@@ -110,6 +156,7 @@ __device__ __forceinline__ int radix_passes(uint32_t mn, uint32_t mx, uint32_t *
     mn = min(mn, red[w]);
     mx = max(mx, red[WAVES + w]);
   }
+  __syncthreads();  // red is free again
   const uint32_t diff = mn ^ mx;
   return diff == 0u ? 0 : (32 - __clz(diff) + 7) / 8;
 }
@@ -168,6 +215,15 @@ __global__ __launch_bounds__(WAVES * 64) void varlen_sort_kernel(const int64_t *
           __syncthreads();
           continue;
         }
+        if ((uint64_t)(mx - mn) < (uint64_t)CAP * 32u) {  // the bitmap fits bufB
+          const uint32_t *c = bufA;
+          if (bitmap_sort<WAVES>([&](int64_t i) { return c[i]; }, [&](int pos, uint32_t k) { bufA[pos] = k; }, n, mn,
+                                 (int)((mx - mn) / 32u) + 1, bufB, red)) {
+            for (int i = tid; i < (int)n; i += kThreads) out0[i] = bufA[i] ^ 0x80000000u;
+            __syncthreads();
+            continue;
+          }
+        }
         uint32_t *cur = bufA, *oth = bufB;
         for (int pi = 0; pi < passes; ++pi) {
           const uint32_t *c = cur;
@@ -192,6 +248,11 @@ __global__ __launch_bounds__(WAVES * 64) void varlen_sort_kernel(const int64_t *
           for (int64_t i = tid; i < n; i += kThreads) out0[i] = in0[i];
           __syncthreads();
           continue;
+        }
+        if ((uint64_t)(mx - mn) < (uint64_t)CAP * 64u) {  // the bitmap fits the two buffers together
+          if (bitmap_sort<WAVES>([&](int64_t i) { return in0[i] ^ 0x80000000u; },
+                                 [&](int pos, uint32_t k) { out0[pos] = k ^ 0x80000000u; }, n, mn, (int)((mx - mn) / 32u) + 1, bufA, red))
+            continue;
         }
         uint32_t *t1 = reinterpret_cast<uint32_t *>(tmp + s);
         const uint32_t *cur = in0;

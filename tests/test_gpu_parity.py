@@ -347,6 +347,33 @@ def test_varlen_sort_size_classes(fm):
     assert torch.equal(out.cpu(), O.varlen_sort(starts, ends, src))
 
 
+def test_varlen_sort_keys_without_repeats_and_with_one(fm):
+    # segments of distinct keys in a narrow range take the bitmap shortcut of the kernel, one repeated key sends a
+    # segment back to the radix passes: every size class, lengths up to 300000 (through HBM), ranges on both sides of
+    # what the bitmaps hold (32 x 2048, 32 x 8192, 32 x 16384 and 64 x 16384 keys), keys of both signs
+    g = torch.Generator().manual_seed(77)
+    cases = [(1, 1, 0), (2, 2, -1), (63, 64, 5), (2048, 2048, -1000), (2048, 65536, 0), (2047, 65537, -7), (1500, 65535, 100),
+             (2049, 3000, 0), (8192, 262144, -3), (8000, 262145, 0), (8193, 10000, 2 ** 31 - 10001), (16384, 524288, -2 ** 31),
+             (16000, 524289, 0), (16385, 16385, -16000), (40000, 1048576, -500000), (40000, 1048577, 0), (300000, 300000, 0),
+             (300000, 600000, -300000), (5000, 14336, 0)]
+    chunks, starts, ends, pos = [], [], [], 2
+    for n, span, lo in cases:
+        for repeat in (False, True):
+            keys = torch.randperm(span, generator=g)[:n] + lo
+            if repeat and n > 1:
+                keys[int(torch.randint(0, n - 1, (1,), generator=g))] = keys[n - 1]
+            chunks.append((pos, keys))
+            starts.append(pos)
+            ends.append(pos + n)
+            pos += n + 3
+    src = torch.full((pos,), 12345, dtype=torch.int32)
+    for at, keys in chunks:
+        src[at:at + keys.numel()] = keys.to(torch.int32)
+    starts, ends = torch.tensor(starts, dtype=torch.int64), torch.tensor(ends, dtype=torch.int64)
+    out = fm.hip.varlen_sort(starts.cuda(), ends.cuda(), src.cuda())
+    assert torch.equal(out.cpu(), O.varlen_sort(starts, ends, src))
+
+
 def test_varlen_sort_restores_a_shuffled_csc(fm):
     # the op as the reference pipeline uses it: shuffle each column list, sort it back
     q, k, cuq, cuk = _gate_case(fm, 3, [700, 300], [700, 300], 4, 4, 64, 32, 6, True)
