@@ -284,9 +284,11 @@ def varlen_sort(cu_seq_starts: torch.Tensor, cu_seq_ends: torch.Tensor, src: tor
         dst = torch.empty_like(src)
         total = src.numel()
         if total:
-            ws = torch.empty_like(src)
-            _check(load_library().fmoba_varlen_sort(cu_seq_starts.data_ptr(), cu_seq_ends.data_ptr(), cu_seq_starts.numel(),
-                                                    src.data_ptr(), dst.data_ptr(), total, ws.data_ptr(), total * 4, _stream()))
+            lib = load_library()
+            ws_bytes = lib.fmoba_varlen_sort_workspace_bytes(total)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=src.device)
+            _check(lib.fmoba_varlen_sort(cu_seq_starts.data_ptr(), cu_seq_ends.data_ptr(), cu_seq_starts.numel(),
+                                         src.data_ptr(), dst.data_ptr(), total, ws.data_ptr(), ws_bytes, _stream()))
         return dst
 
 

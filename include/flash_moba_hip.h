@@ -113,7 +113,10 @@ int fmoba_fused_topk_static(const fmoba_fused_topk_args *a, void *stream);
  * Segmented ascending sort of signed int32 keys with 64-bit segment offsets.
  * Replaces varlen_sort (csrc/flash_topk/src/varlen_sort.cu:127-162, CUB
  * DeviceSegmentedSort).  dst[i] = 0 for positions outside every segment.  Segments must
- * not overlap.  `workspace` holds `total` int32 (used by segments too long for LDS).
+ * not overlap.  `workspace`: fmoba_varlen_sort_workspace_bytes(total) bytes -- `total` int32
+ * (marks of the segments, second buffer of segments too long for LDS) and 256 bytes of
+ * notes the launches leave each other.  A workspace of `total` int32 alone is accepted as
+ * well; the call then always clears dst first and every launch looks at every segment.
  * ---------------------------------------------------------------------------------- */
 size_t fmoba_varlen_sort_workspace_bytes(int64_t total);
 int fmoba_varlen_sort(const int64_t *seg_starts, const int64_t *seg_ends, int64_t num_segments,

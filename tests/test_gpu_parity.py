@@ -374,6 +374,30 @@ def test_varlen_sort_keys_without_repeats_and_with_one(fm):
     assert torch.equal(out.cpu(), O.varlen_sort(starts, ends, src))
 
 
+def test_varlen_sort_with_a_workspace_of_total_int32_only(fm):
+    # the C entry point also takes a workspace of exactly `total` int32 (then it always clears the whole output first);
+    # segments that tile the buffer and segments with gaps, ascending and not, both ways, into an output full of 77s
+    lib = fm.hip.load_library()
+    g = torch.Generator().manual_seed(9)
+    for gaps, reverse in ((False, False), (True, False), (True, True), (False, True)):
+        lens = torch.randint(0, 3000, (40,), generator=g)
+        ends = torch.cumsum(lens + (7 if gaps else 0), 0).to(torch.int64)
+        starts = ends - lens
+        total = int(ends[-1]) + (5 if gaps else 0)
+        if reverse:  # the segments need not come in ascending order
+            starts, ends = starts.flip(0).contiguous(), ends.flip(0).contiguous()
+        src = torch.randint(-10 ** 6, 10 ** 6, (total,), generator=g, dtype=torch.int64).to(torch.int32)
+        ref = O.varlen_sort(starts, ends, src)
+        sd, ed, xd = starts.cuda(), ends.cuda(), src.cuda()
+        for ws_bytes in (total * 4, lib.fmoba_varlen_sort_workspace_bytes(total)):
+            dst = torch.full((total,), 77, dtype=torch.int32, device="cuda")
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+            rc = lib.fmoba_varlen_sort(sd.data_ptr(), ed.data_ptr(), sd.numel(), xd.data_ptr(), dst.data_ptr(), total, ws.data_ptr(),
+                                       ws_bytes, torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, lib.fmoba_last_error()
+            assert torch.equal(dst.cpu(), ref)
+
+
 def test_varlen_sort_restores_a_shuffled_csc(fm):
     # the op as the reference pipeline uses it: shuffle each column list, sort it back
     q, k, cuq, cuk = _gate_case(fm, 3, [700, 300], [700, 300], 4, 4, 64, 32, 6, True)
