@@ -26,13 +26,17 @@ struct TopkParams {
 };
 
 // Rows per counting segment.  A wave of the fill kernel walks one segment of one 32-chunk word column, 64 rows at a
-// time, one after the other: segments of 2048 rows keep the counts small, but a short batch (one sequence of 8192
-// tokens: 128 waves) would leave most of the GPU idle for the 32 steps of a segment, so segments shrink (down to 256
-// rows, a multiple of the gate's 128-row blocks) until there are a few thousand waves.
+// time, one step after the other, and a step is a chain (load the words, 32 ballots, a store per chunk) that only
+// other waves can cover: segments of 2048 rows keep the counts small, but the fill wants many thousands of waves,
+// so segments shrink (down to 256 rows, a multiple of the gate's 128-row blocks) until there are 16384 of them.  The
+// headline batch (eight sequences, 65536 tokens) gets 512-row segments: fill 116 -> 63 us against 6272 waves of 2048
+// rows (256-row segments: 56 us, but twice the counts to clear, scan and keep); a single sequence of 8192 tokens
+// 86 -> 15 us against its 128 waves.  Beyond that the fill does not gain (262144 tokens: 131072 waves of 2048 rows
+// 1.55 ms, twice as many of 1024 rows 1.62 ms and the scan of the counts four times as long).
 static inline int csc_seg_rows(int64_t batch, int64_t heads, int64_t max_seqlen_q, int64_t W) {
   int seg_rows = kSegRows;
   const int64_t lq = max_seqlen_q > 0 ? max_seqlen_q : 1;
-  while (seg_rows > 256 && batch * heads * W * ((lq + seg_rows - 1) / seg_rows) < 2048) seg_rows >>= 1;
+  while (seg_rows > 256 && batch * heads * W * ((lq + seg_rows - 1) / seg_rows) < 16384) seg_rows >>= 1;
   return seg_rows;
 }
 

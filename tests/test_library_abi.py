@@ -39,9 +39,11 @@ def test_workspace_queries_are_pure_host_functions():
     lib = H.load_library()
     # selection bits: heads * ceil(maxC/32) * total_q words; counts: batch*heads*nseg*maxC words
     b = lib.fmoba_fused_topk_workspace_bytes(8, 65536, 16, 14336, 14336, 64)
-    assert b >= 16 * 7 * 65536 * 4 + 8 * 16 * 7 * 224 * 4
+    assert b >= 16 * 7 * 65536 * 4 + 8 * 16 * 28 * 224 * 4  # 512-row counting segments at this size
     assert lib.fmoba_fused_topk_workspace_bytes(0, 0, 0, 0, 0, 0) == 0
-    assert lib.fmoba_varlen_sort_workspace_bytes(1000) == 4000
+    # `total` int32, then 256 bytes of notes on a 256-byte boundary
+    assert lib.fmoba_varlen_sort_workspace_bytes(1000) == 4096 + 256
+    assert lib.fmoba_varlen_sort_workspace_bytes(0) == 0
     a = H.AttnBwdArgs()
     a.total_q, a.heads, a.head_dim, a.batch, a.total_k, a.lg_block_n, a.max_visits_per_row, a.num_row_indices = 1024, 4, 128, 1, 1024, 64, 8, 32768
     a.dq_mode = 2
