@@ -1233,7 +1233,10 @@ __global__ __launch_bounds__(256) void csc_scan_kernel(TopkParams p) {
 // grid (nseg * W, heads, batch), block 64: one wave walks the rows of one segment of one 32-chunk word column
 __global__ __launch_bounds__(64) void csc_fill_kernel(TopkParams p) {
   const fmoba_fused_topk_args &a = p.a;
-  const int seg = blockIdx.x / p.W, wc = blockIdx.x - seg * p.W;
+  // consecutive workgroups: consecutive segments of one word column, i.e. consecutive memory.  (With the word column
+  // as the fast index the waves that run at the same time read addresses a whole word column apart -- total_q words,
+  // a power of two more often than not -- and meet in the same memory channel.)
+  const int wc = blockIdx.x / p.nseg, seg = blockIdx.x - wc * p.nseg;
   const int h = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
   const int q0 = a.cu_seqlens_q[b];
   const int Lq = a.cu_seqlens_q[b + 1] - q0;
