@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   float *sLse = reinterpret_cast<float *>(smem + SM::oLse);
   float *sDelta = reinterpret_cast<float *>(smem + SM::oDelta);
 
-  const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + NKEY - 1) / NKEY);
+  const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + NKEY - 1) / NKEY, (int64_t)a.max_seqlen_q * HD * 4 >= kOnePairBytes);
   const int nb = item.idx, b = item.pair / a.heads, h = item.pair - b * a.heads;
   const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
   const int key0 = nb * NKEY;
@@ -480,7 +480,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         const Pack8 x = lds_read16(bx + SO + (uint32_t)(k * RPP * LDH * 2));
         const bool ok = (r2 >= 0) & (s2 < ws.cap);
         const int64_t pidx = ok ? ((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2 : trash;
-        if (kq * (NDH * 32) + col < D) *reinterpret_cast<Pack8 *>(ws.part + pidx * D + kq * (NDH * 32) + col) = x;
+        if (kq * (NDH * 32) + col < D) st_stream16(ws.part + pidx * D + kq * (NDH * 32) + col, x);
         if (kq == 0 && col == 0) ws.pid[pidx] = nb;
       }
       wave_lds_fence();
@@ -1045,11 +1045,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_combine_kernel(fmoba_attn_bwd
     for (; t + 4 <= n; t += 4) {  // independent loads, four in flight
       Pack8 x[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) x[u] = ld_global16(part + (int64_t)sOrd[t + u] * D + c8);
+      for (int u = 0; u < 4; ++u) x[u] = ld_stream16(part + (int64_t)sOrd[t + u] * D + c8);
 #pragma unroll
       for (int u = 0; u < 4; ++u) add(x[u]);
     }
-    for (; t < n; ++t) add(ld_global16(part + (int64_t)sOrd[t] * D + c8));
+    for (; t < n; ++t) add(ld_stream16(part + (int64_t)sOrd[t] * D + c8));
   }
   if (valid && mine) {
     Pack8 o;

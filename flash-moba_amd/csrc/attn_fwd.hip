@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
   int *sRow = reinterpret_cast<int *>(smem + SM::oRow);
   int *sSlot = reinterpret_cast<int *>(smem + SM::oSlot);
 
-  const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + KB - 1) / KB);
+  const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + KB - 1) / KB, (int64_t)a.max_seqlen_q * HD * 4 >= kOnePairBytes);
   const int nb = item.idx, b = item.pair / a.heads, h = item.pair - b * a.heads;
   const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
   const int key0 = nb * KB;
@@ -365,7 +365,7 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
       for (int k = 0; k < 8; ++k) x[k] = lds_read16(bx + (uint32_t)(4 * k * LDO * 2));
 #pragma unroll
       for (int k = 0; k < 8; ++k)
-        if (p2[k] >= 0) *reinterpret_cast<Pack8 *>(ws.part + ((uint64_t)(uint32_t)p2[k] * (uint32_t)D + (uint32_t)((lane & 15) * 8))) = x[k];
+        if (p2[k] >= 0) st_stream16(ws.part + ((uint64_t)(uint32_t)p2[k] * (uint32_t)D + (uint32_t)((lane & 15) * 8)), x[k]);
     }
     wave_lds_fence();
   };
@@ -468,13 +468,13 @@ __global__ __launch_bounds__(256) void attn_fwd_combine_kernel(fmoba_attn_fwd_ar
         float w[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          x[u] = ld_global16(part + (int64_t)sOrd[base + t + u] * D + c8);
+          x[u] = ld_stream16(part + (int64_t)sOrd[base + t + u] * D + c8);
           w[u] = sWgt[sg][t + u];
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) add(x[u], w[u]);
       }
-      for (; t < cntb; ++t) add(ld_global16(part + (int64_t)sOrd[base + t] * D + c8), sWgt[sg][t]);
+      for (; t < cntb; ++t) add(ld_stream16(part + (int64_t)sOrd[base + t] * D + c8), sWgt[sg][t]);
     }
   }
   if (!valid) return;

@@ -409,13 +409,19 @@ __device__ __forceinline__ void static_for(F &&f) {
 // Workgroup i runs on XCD i % 8.  With a multiple of 8 pairs, pair p gets XCD p % 8 for all its
 // items, so what the items of a pair share (its K / V, or the Q / dO rows that its key blocks
 // gather again and again) stays in one L2; otherwise the items of a pair are simply consecutive.
+// one_pair_at_a_time asks for the consecutive order in any case: when the rows a pair's items gather
+// are far more than the L2s hold (kOnePairBytes and up), eight pairs at once also overflow the
+// 256 MB memory-side cache, and the whole chip on one pair keeps that pair's rows in it
+// (262144 tokens: dK/dV 20.9 -> 20.1 ms, forward columns 10.8 -> 10.3; at 32768 tokens, where
+// an L2 still holds a good part of a pair, the same order costs 13 %).
 // ------------------------------------------------------------------------------------
+constexpr long long kOnePairBytes = 64ll << 20;
 struct PairItem {
   int pair, idx;
 };
-__device__ __forceinline__ PairItem xcd_pair_item(int id, int npairs, int nper) {
+__device__ __forceinline__ PairItem xcd_pair_item(int id, int npairs, int nper, bool one_pair_at_a_time = false) {
   PairItem w;
-  if (npairs % 8 == 0) {
+  if (npairs % 8 == 0 && !one_pair_at_a_time) {
     const int s = id >> 3;
     const int pl = s / nper;
     w.pair = pl * 8 + (id & 7);
@@ -428,6 +434,28 @@ __device__ __forceinline__ PairItem xcd_pair_item(int id, int npairs, int nper) 
 }
 
 __device__ __forceinline__ Pack8 ld_global16(const void *p) { return *reinterpret_cast<const Pack8 *>(p); }
+// Partial results (one per visit of a row, written by the column passes and added up by the combine kernels) go
+// through the caches once in each direction: non-temporal stores and loads keep them from pushing the rows that
+// the column passes gather again and again out of the caches (262144 tokens: dK/dV 20.0 -> 18.4 ms, forward
+// columns 10.1 -> 9.6; 32768 tokens: step 9.95 -> 9.55 ms).  The dS tiles of the dS form were tried the same
+// way: no difference on the headline batch (3.35-3.41 against 3.37-3.40 ms).
+// 16 bytes that are read once: a non-temporal load
+__device__ __forceinline__ Pack8 ld_stream16(const void *p) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const u32x4 x = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+  Pack8 r;
+  r.w[0] = x[0];
+  r.w[1] = x[1];
+  r.w[2] = x[2];
+  r.w[3] = x[3];
+  return r;
+}
+// 16 bytes that are written once and read once by a later kernel: a non-temporal store
+__device__ __forceinline__ void st_stream16(void *p, const Pack8 &v) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 x = {v.w[0], v.w[1], v.w[2], v.w[3]};
+  __builtin_nontemporal_store(x, reinterpret_cast<u32x4 *>(p));
+}
 __device__ __forceinline__ Pack8 zero_pack8() {
   Pack8 r;
   r.w[0] = r.w[1] = r.w[2] = r.w[3] = 0u;
