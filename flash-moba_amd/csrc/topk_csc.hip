@@ -752,16 +752,41 @@ __device__ __forceinline__ uint32_t mad24_u32(int a, int b, uint32_t c) {
   return (uint32_t)(a * b) + c;
 #endif
 }
-// n + (x >= y): the compare and an add with carry (left alone, the compiler materialises the flag as 0 / 1 first)
-__device__ __forceinline__ int count_if_ge(int n, float x, float y) {
+// n + (x >= y) in two halves: four compares into four scalar register pairs first, then an add with carry per flag
+// where the count is needed (a vector instruction that reads a scalar register written by the one before it has to
+// wait two slots: with the compares of four scores ahead of their adds nothing waits; left alone, the compiler
+// materialises every flag as 0 / 1 first).  Volatile, so that the compares stay ahead of the adds.
+struct Flags4 {
+  unsigned long long m[4];
+};
+__device__ __forceinline__ Flags4 flags4_ge(float x0, float x1, float x2, float x3, float y) {
+  Flags4 f;
 #if defined(__HIP_DEVICE_COMPILE__)
-  asm("v_cmp_ge_f32 vcc, %1, %2\n\ts_nop 1\n\tv_addc_co_u32 %0, vcc, 0, %0, vcc" : "+v"(n) : "v"(x), "v"(y) : "vcc");
+  asm volatile("v_cmp_ge_f32_e64 %0, %4, %8\n\t"
+               "v_cmp_ge_f32_e64 %1, %5, %8\n\t"
+               "v_cmp_ge_f32_e64 %2, %6, %8\n\t"
+               "v_cmp_ge_f32_e64 %3, %7, %8"
+               : "=&s"(f.m[0]), "=&s"(f.m[1]), "=&s"(f.m[2]), "=&s"(f.m[3])
+               : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "v"(y));
+#else
+  f.m[0] = x0 >= y;
+  f.m[1] = x1 >= y;
+  f.m[2] = x2 >= y;
+  f.m[3] = x3 >= y;
+#endif
+  return f;
+}
+__device__ __forceinline__ int count_flag(int n, unsigned long long flag) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("v_addc_co_u32_e64 %0, vcc, 0, %0, %1" : "+v"(n) : "s"(flag) : "vcc");
   return n;
 #else
-  return n + (x >= y ? 1 : 0);
+  return n + (int)(flag & 1);
 #endif
 }
 
+constexpr int kStreamListMargin = 64;  // words on either side of a wave's lists
+constexpr int kStreamListWords = 4 * (32 * 18 + 2 * kStreamListMargin) + 256;
 template <typename T, int HD, int NT>
 __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(TopkParams p) {
   constexpr int CAP = 16, PL = 8;
@@ -773,7 +798,11 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
   static_assert(NV >= 1 && NV * RPI * 4 == GC, "the four waves share a tile evenly");
   constexpr int RB = HD * 2;              // bytes of a tile row: exactly HD elements, swizzled instead of padded
   constexpr int LS = CAP + 2;                 // slots of a row's list: 16 entries and the two lanes' next slots
-  constexpr int EW = kGateRows * LS + 256;    // words of an entrant array: the lists, then a trash word per thread
+  // words of an entrant array: per wave the lists of its 32 rows between two margins, then a trash word per thread.
+  // A lane with more entrants than its row's list holds writes on into the lists of the wave's other rows and, from
+  // the first and the last row, into a margin (at most 63 - 17 slots beyond the list): such a wave takes the bisection
+  // and rebuilds its lists, and no other wave's list is touched, so the slot needs no clamp.
+  constexpr int EW = kStreamListWords;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint32_t *sSel = reinterpret_cast<uint32_t *>(smem);  // [word columns of a pass][128], reuses the tile and the lists after the last group
   float *sEv = reinterpret_cast<float *>(smem + (size_t)GC * RB);  // [EW] scores of the entrants
@@ -848,8 +877,8 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
 #pragma unroll
   for (int j = 0; j < PL; ++j) win[j] = kSlotEmpty;
   int m_prev = 0;    // winners the row holds
-  float *const my_list_v = sEv + rs * LS;
-  float *const my_trash = sEv + kGateRows * LS + tid;
+  float *const my_list_v = sEv + wave * (32 * LS + 2 * kStreamListMargin) + kStreamListMargin + (lane & 31) * LS;
+  float *const my_trash = sEv + 4 * (32 * LS + 2 * kStreamListMargin) + tid;
   constexpr int kToIdx = EW;  // from a score of the entrant arrays to its chunk, in words
 
   if (ngroups > 0) tile_issue(0);
@@ -910,12 +939,16 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
       for (int t = 0; t < NT; ++t)
         if (t < n_tiles) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            // (before position LS - 1 the lane cannot have that many entrants)
-            const uint32_t d = mad24_u32(t * 16 + i < LS - 1 ? cnt : min(cnt, LS - 1), slot_step, slot0);
-            lds_write_vec<float>(d, sc[t][i]);
-            lds_write_vec<int>(d + (uint32_t)kToIdx * 4u, cbase + t * 32 + 8 * (i >> 2) + (i & 3));
-            cnt = count_if_ge(cnt, sc[t][i], pmin);
+          for (int i4 = 0; i4 < 4; ++i4) {
+            const Flags4 ge = flags4_ge(sc[t][4 * i4], sc[t][4 * i4 + 1], sc[t][4 * i4 + 2], sc[t][4 * i4 + 3], pmin);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int i = 4 * i4 + j;
+              const uint32_t d = mad24_u32(cnt, slot_step, slot0);
+              lds_write_vec<float>(d, sc[t][i]);
+              lds_write_vec<int>(d + (uint32_t)kToIdx * 4u, cbase + t * 32 + 8 * (i >> 2) + (i & 3));
+              cnt = count_flag(cnt, ge.m[j]);
+            }
           }
         }
       const int cnt_o = shfl_xor32_i(cnt);
@@ -1419,7 +1452,7 @@ static int launch_gate_big(const TopkParams &p, dim3 grid, hipStream_t s) {
 }
 template <int HD, int NT>
 static constexpr size_t gate_stream_smem() {
-  const size_t head = (size_t)NT * 32 * HD * 2 + (size_t)2 * (kGateRows * 18 + 256) * 4;  // tile and lists; later the selection words of a pass
+  const size_t head = (size_t)NT * 32 * HD * 2 + (size_t)2 * kStreamListWords * 4;  // tile and lists; later the selection words of a pass
   return head + head / (kGateRows * 4) * 32 * 4;
 }
 template <typename T, int HD, int NT>
