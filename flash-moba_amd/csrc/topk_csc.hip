@@ -786,7 +786,8 @@ __device__ __forceinline__ int count_flag(int n, unsigned long long flag) {
 }
 
 constexpr int kStreamListMargin = 64;  // words on either side of a wave's lists
-constexpr int kStreamListWords = 4 * (32 * 18 + 2 * kStreamListMargin) + 256;
+constexpr int kStreamListStride = 19;  // words from one row's list (18 slots) to the next
+constexpr int kStreamListWords = 4 * (32 * kStreamListStride + 2 * kStreamListMargin) + 256;
 template <typename T, int HD, int NT>
 __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(TopkParams p) {
   constexpr int CAP = 16, PL = 8;
@@ -877,8 +878,10 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
 #pragma unroll
   for (int j = 0; j < PL; ++j) win[j] = kSlotEmpty;
   int m_prev = 0;    // winners the row holds
-  float *const my_list_v = sEv + wave * (32 * LS + 2 * kStreamListMargin) + kStreamListMargin + (lane & 31) * LS;
-  float *const my_trash = sEv + 4 * (32 * LS + 2 * kStreamListMargin) + tid;
+  // (lists kStreamListStride = 19 words apart: with 18, an even number, rows l and l + 16 share a bank and every
+  // store of the 32 lanes of a half wave takes two turns)
+  float *const my_list_v = sEv + wave * (32 * kStreamListStride + 2 * kStreamListMargin) + kStreamListMargin + (lane & 31) * kStreamListStride;
+  float *const my_trash = sEv + 4 * (32 * kStreamListStride + 2 * kStreamListMargin) + tid;
   constexpr int kToIdx = EW;  // from a score of the entrant arrays to its chunk, in words
 
   if (ngroups > 0) tile_issue(0);
