@@ -374,6 +374,35 @@ def test_varlen_sort_keys_without_repeats_and_with_one(fm):
     assert torch.equal(out.cpu(), O.varlen_sort(starts, ends, src))
 
 
+def test_varlen_sort_tiny_segments_at_every_alignment(fm):
+    # lengths 0 .. 13 starting at every offset modulo four (the bitmap launch reads whole 16-byte vectors between up to
+    # three keys before and after them), distinct keys and keys with a repeat, one call
+    g = torch.Generator().manual_seed(13)
+    starts, ends, pieces, pos = [], [], [], 0
+    for n in range(14):
+        for shift in range(4):
+            for repeat in (False, True):
+                while pos % 4 != shift:
+                    pos += 1
+                keys = torch.randperm(40, generator=g)[:n] - 20
+                if repeat and n > 1:
+                    keys[0] = keys[n - 1]
+                starts.append(pos)
+                ends.append(pos + n)
+                pieces.append((pos, keys))
+                pos += n
+    src = torch.full((pos + 2,), -99, dtype=torch.int32)
+    for at, keys in pieces:
+        src[at:at + keys.numel()] = keys.to(torch.int32)
+    starts, ends = torch.tensor(starts, dtype=torch.int64), torch.tensor(ends, dtype=torch.int64)
+    out = fm.hip.varlen_sort(starts.cuda(), ends.cuda(), src.cuda())
+    assert torch.equal(out.cpu(), O.varlen_sort(starts, ends, src))
+    # the same keys behind an odd offset of the buffers themselves (a view that starts one int32 into an allocation)
+    src1 = torch.cat([torch.zeros(1, dtype=torch.int32), src]).cuda()[1:]
+    out1 = fm.hip.varlen_sort(starts.cuda(), ends.cuda(), src1)
+    assert torch.equal(out1.cpu(), out.cpu())
+
+
 def test_varlen_sort_with_a_workspace_of_total_int32_only(fm):
     # the C entry point also takes a workspace of exactly `total` int32 (then it always clears the whole output first);
     # segments that tile the buffer and segments with gaps, ascending and not, both ways, into an output full of 77s
