@@ -1266,6 +1266,32 @@ __global__ __launch_bounds__(256) void csc_scan_kernel(TopkParams p) {
   for (int64_t i = start + tid; i < end; i += 256) a.flat_indices[i] = 0;
 }
 
+// x with the value of lane `lane` (the same in every lane) replaced by v (the same in every lane)
+template <int LANE>
+__device__ __forceinline__ uint32_t write_lane(uint32_t x, uint32_t v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm("v_writelane_b32 %0, %1, %2" : "+v"(x) : "s"(v), "n"(LANE));
+#else
+  (void)v;
+#endif
+  return x;
+}
+// base[byte_offset] = value in the lanes of `lanes`, all others do nothing (base: the same in every lane)
+__device__ __forceinline__ void store_i32_in_lanes(int32_t *base, uint32_t byte_offset, int value, unsigned long long lanes) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  unsigned long long saved;
+  asm volatile("s_mov_b64 %0, exec\n\t"
+               "s_mov_b64 exec, %1\n\t"
+               "global_store_dword %2, %3, %4\n\t"
+               "s_mov_b64 exec, %0"
+               : "=&s"(saved)
+               : "s"(lanes), "v"(byte_offset), "v"(value), "s"(base)
+               : "memory");
+#else
+  (void)base, (void)byte_offset, (void)value, (void)lanes;
+#endif
+}
+
 // grid (nseg * W, heads, batch), block 64: one wave walks the rows of one segment of one 32-chunk word column
 __global__ __launch_bounds__(64) void csc_fill_kernel(TopkParams p) {
   const fmoba_fused_topk_args &a = p.a;
@@ -1280,30 +1306,36 @@ __global__ __launch_bounds__(64) void csc_fill_kernel(TopkParams p) {
   if (r0 >= Lq) return;
   const int r1 = min(Lq, r0 + p.seg_rows);
   const int64_t bh = (int64_t)b * a.heads + h;
-  int64_t pos = 0;
+  // Where the next rows of chunk wc * 32 + j go: lane j keeps the position relative to the start of the word column's
+  // first list (the 32 lists follow each other, far less than 2^30 entries), the start itself is a scalar.  A step
+  // costs vector instructions and nothing else (the vector pipes are busy 85 % of the kernel's time), so a chunk that
+  // some row of the step selects takes five: the lane's rank among the rows (mbcnt), the slot, the store in the lanes
+  // of the ballot (the ballot itself is the exec mask), and the new position written back into lane j.
+  const int64_t first = a.col_offsets[bh * p.max_cols + wc * 32];
+  int32_t *const lists = a.flat_indices + first;
+  uint32_t rel = 0u;
   {
     const int c = wc * 32 + lane;
     if (lane < 32 && c < p.max_cols)
-      pos = a.col_offsets[bh * p.max_cols + c] + p.segcnt[(bh * p.nseg + seg) * p.max_cols + c];
+      rel = (uint32_t)(a.col_offsets[bh * p.max_cols + c] - first) + (uint32_t)p.segcnt[(bh * p.nseg + seg) * p.max_cols + c];
   }
   const uint32_t *words = p.sel + ((int64_t)h * p.W + wc) * a.total_q + q0;
-  const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   for (int rb = r0; rb < r1; rb += 64) {
     const int r = rb + lane;
     const uint32_t w = (r < r1) ? words[r] : 0u;
-    if (!__any(w != 0u)) continue;
-#pragma unroll
-    for (int j = 0; j < 32; ++j) {
-      const bool bit = (w >> j) & 1u;
-      const unsigned long long m = __ballot(bit);
-      if (m) {
-        const uint32_t lo = __builtin_amdgcn_readlane((uint32_t)pos, j);
-        const uint32_t hi = __builtin_amdgcn_readlane((uint32_t)((uint64_t)pos >> 32), j);
-        const int64_t bj = (int64_t)(((uint64_t)hi << 32) | lo);
-        if (bit) a.flat_indices[bj + __popcll(m & lt)] = r;
-        if (lane == j) pos += __popcll(m);
+    // the chunks that some row of the step selects (a scalar, so that the others cost no vector instruction)
+    const uint32_t present = __builtin_amdgcn_readfirstlane(__ockl_wfred_or_u32(w));
+    if (present == 0u) continue;
+    static_for<32>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      if (present & (1u << j)) {
+        const unsigned long long m = __ballot((w & (1u << j)) != 0u);
+        const uint32_t at = __builtin_amdgcn_readlane(rel, j);
+        const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        store_i32_in_lanes(lists, (at + rank) << 2, r, m);
+        rel = write_lane<j>(rel, at + (uint32_t)__popcll(m));
       }
-    }
+    });
   }
 }
 
@@ -1531,6 +1563,9 @@ static int fused_topk_run(const fmoba_fused_topk_args *a, void *workspace, size_
   }
   const bool big = max_cols > 256;  // more chunks than the register-resident gate holds: grouped gate
   FMOBA_REQUIRE(max_cols <= kMaxChunksPerSequence, "fused_topk: %d key chunks per sequence; at most %d are supported", max_cols, kMaxChunksPerSequence);
+  // (the fill keeps list positions as 32-bit byte offsets from the first of the 32 lists of a word column)
+  FMOBA_REQUIRE(a->max_seqlen_q < (1 << 24), "fused_topk: max_seqlen_q = %d; sequences of up to %d query rows are supported", a->max_seqlen_q,
+                (1 << 24) - 1);
   FMOBA_REQUIRE(a->q && a->km, "fused_topk: null q/km pointer");
   FMOBA_REQUIRE(a->q_row_stride % 8 == 0 && a->q_head_stride % 8 == 0 && a->km_row_stride % 8 == 0 && a->km_head_stride % 8 == 0,
                 "fused_topk: strides must be multiples of 8 elements");
