@@ -63,6 +63,67 @@ __device__ __forceinline__ int count4_gt(int n, float x0, float x1, float x2, fl
 #endif
 }
 
+// n + (x >= y) in two halves: four compares into four scalar register pairs first, then an add with carry per flag
+// where the count is needed (a vector instruction that reads a scalar register written by the one before it has to
+// wait two slots: with the compares of four scores ahead of their adds nothing waits; left alone, the compiler
+// materialises every flag as 0 / 1 first).  Volatile, so that the compares stay ahead of the adds.
+struct Flags4 {
+  unsigned long long m[4];
+};
+__device__ __forceinline__ Flags4 flags4_ge(float x0, float x1, float x2, float x3, float y) {
+  Flags4 f;
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("v_cmp_ge_f32_e64 %0, %4, %8\n\t"
+               "v_cmp_ge_f32_e64 %1, %5, %8\n\t"
+               "v_cmp_ge_f32_e64 %2, %6, %8\n\t"
+               "v_cmp_ge_f32_e64 %3, %7, %8"
+               : "=&s"(f.m[0]), "=&s"(f.m[1]), "=&s"(f.m[2]), "=&s"(f.m[3])
+               : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "v"(y));
+#else
+  f.m[0] = x0 >= y;
+  f.m[1] = x1 >= y;
+  f.m[2] = x2 >= y;
+  f.m[3] = x3 >= y;
+#endif
+  return f;
+}
+__device__ __forceinline__ int count_flag(int n, unsigned long long flag) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("v_addc_co_u32_e64 %0, vcc, 0, %0, %1" : "+v"(n) : "s"(flag) : "vcc");
+  return n;
+#else
+  return n + (int)(flag & 1);
+#endif
+}
+
+// the same with x > y
+__device__ __forceinline__ Flags4 flags4_gt(float x0, float x1, float x2, float x3, float y) {
+  Flags4 f;
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("v_cmp_gt_f32_e64 %0, %4, %8\n\t"
+               "v_cmp_gt_f32_e64 %1, %5, %8\n\t"
+               "v_cmp_gt_f32_e64 %2, %6, %8\n\t"
+               "v_cmp_gt_f32_e64 %3, %7, %8"
+               : "=&s"(f.m[0]), "=&s"(f.m[1]), "=&s"(f.m[2]), "=&s"(f.m[3])
+               : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "v"(y));
+#else
+  f.m[0] = x0 > y;
+  f.m[1] = x1 > y;
+  f.m[2] = x2 > y;
+  f.m[3] = x3 > y;
+#endif
+  return f;
+}
+// (w << 1) | flag of the lane: one add with carry
+__device__ __forceinline__ uint32_t shift_in_flag(uint32_t w, unsigned long long flag) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("v_addc_co_u32_e64 %0, vcc, %0, %0, %1" : "+v"(w) : "s"(flag) : "vcc");
+  return w;
+#else
+  return (w << 1) | (uint32_t)(flag & 1);
+#endif
+}
+
 template <typename T, int HD, int NT>
 __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_kernel(TopkParams p) {
   constexpr int KS = HD / 16;
@@ -184,6 +245,7 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
   float tau_eq = INFINITY;  // no tie group by default
   int n_eq = 0;
   uint32_t iota = 0u;
+  bool any_tie = false;     // some row of the wave has a tie across its cut
   {
     uint32_t lo_k = float_order_key(vmin) - 1u;  // count(x > lo) = nc > K'
     uint32_t hi_k = float_order_key(vmax);       // count(x > hi) = 0  < K'
@@ -229,7 +291,8 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
     }
     // a tie group keeps its n_eq highest chunk indices
     const bool tie = n_eq > 0;
-    if (__any(tie)) {
+    any_tie = __any(tie);
+    if (any_tie) {
       int ceq = 0;
 #pragma unroll
       for (int t = 0; t < NT; ++t)
@@ -272,12 +335,26 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
     if (t < p.W) {
       uint32_t w = 0u;
       if (t < n_tiles && kp > 0) {
+        if (!any_tie) {
+          // no row of the wave has a tie across its cut: a score is selected iff it lies above tau.  The flags of the
+          // lane's 16 scores are shifted in one by one (w + w + flag: one add with carry each), highest first, and the
+          // four nibbles then move to the places of the lane's chunks (4 hh + 8 g .. + 3).
+          uint32_t bits = 0u;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
-          const float x = sc[t][i];
-          const bool s = (x > tau) | ((x == tau_eq) & (c >= iota));
-          w |= s ? (1u << ((8 * (i >> 2) + (i & 3)) + 4 * hh)) : 0u;
+          for (int i4 = 3; i4 >= 0; --i4) {
+            const Flags4 f = flags4_gt(sc[t][4 * i4 + 3], sc[t][4 * i4 + 2], sc[t][4 * i4 + 1], sc[t][4 * i4], tau);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bits = shift_in_flag(bits, f.m[j]);
+          }
+          w = ((bits & 0xfu) | ((bits & 0xf0u) << 4) | ((bits & 0xf00u) << 8) | ((bits & 0xf000u) << 12)) << (4 * hh);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
+            const float x = sc[t][i];
+            const bool s = (x > tau) | ((x == tau_eq) & (c >= iota));
+            w |= s ? (1u << ((8 * (i >> 2) + (i & 3)) + 4 * hh)) : 0u;
+          }
         }
       }
       {
@@ -752,39 +829,6 @@ __device__ __forceinline__ uint32_t mad24_u32(int a, int b, uint32_t c) {
   return (uint32_t)(a * b) + c;
 #endif
 }
-// n + (x >= y) in two halves: four compares into four scalar register pairs first, then an add with carry per flag
-// where the count is needed (a vector instruction that reads a scalar register written by the one before it has to
-// wait two slots: with the compares of four scores ahead of their adds nothing waits; left alone, the compiler
-// materialises every flag as 0 / 1 first).  Volatile, so that the compares stay ahead of the adds.
-struct Flags4 {
-  unsigned long long m[4];
-};
-__device__ __forceinline__ Flags4 flags4_ge(float x0, float x1, float x2, float x3, float y) {
-  Flags4 f;
-#if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("v_cmp_ge_f32_e64 %0, %4, %8\n\t"
-               "v_cmp_ge_f32_e64 %1, %5, %8\n\t"
-               "v_cmp_ge_f32_e64 %2, %6, %8\n\t"
-               "v_cmp_ge_f32_e64 %3, %7, %8"
-               : "=&s"(f.m[0]), "=&s"(f.m[1]), "=&s"(f.m[2]), "=&s"(f.m[3])
-               : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "v"(y));
-#else
-  f.m[0] = x0 >= y;
-  f.m[1] = x1 >= y;
-  f.m[2] = x2 >= y;
-  f.m[3] = x3 >= y;
-#endif
-  return f;
-}
-__device__ __forceinline__ int count_flag(int n, unsigned long long flag) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("v_addc_co_u32_e64 %0, vcc, 0, %0, %1" : "+v"(n) : "s"(flag) : "vcc");
-  return n;
-#else
-  return n + (int)(flag & 1);
-#endif
-}
-
 constexpr int kStreamListMargin = 64;  // words on either side of a wave's lists
 constexpr int kStreamListStride = 19;  // words from one row's list (18 slots) to the next
 constexpr int kStreamListWords = 4 * (32 * kStreamListStride + 2 * kStreamListMargin) + 256;
