@@ -696,6 +696,18 @@ __device__ __forceinline__ DqItem dq_decode_item(int id, int npairs, int nsb_max
   return w;
 }
 
+// a * b of two values below 2^24, b the same in every lane: one full-rate instruction (a 32-bit multiply takes four
+// times as long)
+__device__ __forceinline__ uint32_t mul24_u32(uint32_t a, uint32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  uint32_t d;
+  asm("v_mul_u32_u24 %0, %1, %2" : "=v"(d) : "v"(a), "s"(b));
+  return d;
+#else
+  return a * b;
+#endif
+}
+
 template <int N>
 __device__ __forceinline__ void wait_loads_but() {  // until at most N of the wave's vector memory loads are outstanding
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -795,7 +807,8 @@ __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq
       const int code = sStep[st];
       const int cl = code >> 8, kb = code & 255;
       const int64_t pos0 = sOff[cl];
-      sInfo[st] = make_int4((cb + cl) * Bn + kb * 64, sCnt[cl], (int)(uint32_t)(pos0 & 0xffffffffll), (int)(pos0 >> 32));
+      // (y: rows of the run, at most 512, and above them the 64-key block's number inside its column)
+      sInfo[st] = make_int4((cb + cl) * Bn + kb * 64, sCnt[cl] | (kb << 16), (int)(uint32_t)(pos0 & 0xffffffffll), (int)(pos0 >> 32));
     }
     __syncthreads();  // (also: everyone has read the scratch arrays before the first tile loads overwrite them)
     return nsteps;
@@ -838,14 +851,14 @@ __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq
     if (nsteps == 0) continue;
     auto row_id = [&](int step) {  // row of list position tid of the step (clamped)
       const int4 info = sInfo[min(step, nsteps - 1)];
-      const int n = __builtin_amdgcn_readfirstlane(info.y);
+      const int n = __builtin_amdgcn_readfirstlane(info.y) & 0xffff;
       const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
       return a.row_indices[pos0 + min(tid & (ROWS - 1), n - 1)];
     };
     auto put_pos = [&](int step, int rr) {  // thread t tells row rr, the t-th of the step's run, where it is
       if (step < nsteps && tid < ROWS) {
         const int4 info = sInfo[step];
-        const int key0 = info.x, n = info.y;
+        const int key0 = info.x, n = info.y & 0xffff;
         const int first_rel = causal ? key0 - off - m0 : -0x40000000;  // rows before it see no key of the block
         const int rel = rr - m0;
         if ((tid < n) & ((uint32_t)rel < (uint32_t)rows_sb) & (rel >= first_rel)) sPos[(step % NS) * ROWS + rel] = ((tag_base + step + 1) << 10) | tid;
@@ -876,15 +889,21 @@ __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq
       int v[RT];
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) v[rt] = sPos[(sc_ % NS) * ROWS + myrow[rt]];
-      const int key0 = __builtin_amdgcn_readfirstlane(info.x);
-      const int n = __builtin_amdgcn_readfirstlane(info.y);
+      const int ny = __builtin_amdgcn_readfirstlane(info.y);
+      const int n = ny & 0xffff, kb = ny >> 16;
       const int64_t pos0 = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane(info.z) | ((int64_t)__builtin_amdgcn_readfirstlane(info.w) << 32);
-      const int koff = key0 - (key0 / Bn) * Bn;
+      // ds_piece_offset(pos0 + j, 8 kb + hh + 2 s4, Bn / 8) in two parts: what the step's run has in common (the tile of
+      // its first position and the block's first piece: scalar arithmetic, 64 bits) and the lane's own part (at most
+      // 17 tiles further on: 32 bits, no wide multiply among the vector instructions)
+      const uint32_t kgs = (uint32_t)Bn >> 3, r0s = (uint32_t)pos0 & 31u;
+      const uint16_t *base = ds_ws + (((pos0 >> 5) * (int64_t)kgs + 8 * kb) << 8);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         const bool pres = (step < nsteps) & ((v[rt] >> 10) == tag_base + sc_ + 1);
-        const uint32_t j = pres ? (uint32_t)(v[rt] & 1023) : (uint32_t)(myrow[rt] * n) / (uint32_t)ROWS;
-        const uint16_t *rp = ds_ws + ds_piece_offset(pos0 + j, (koff >> 3) + hh, Bn >> 3);
+        const uint32_t j = pres ? (uint32_t)(v[rt] & 1023) : mul24_u32((uint32_t)myrow[rt], (uint32_t)n) / (uint32_t)ROWS;
+        const uint32_t t = r0s + j;
+        const uint32_t lane_bytes = ((mul24_u32(t >> 5, kgs) + (uint32_t)hh) << 9) + ((t & 31u) << 4);
+        const uint16_t *rp = reinterpret_cast<const uint16_t *>(reinterpret_cast<const uint8_t *>(base) + lane_bytes);
 #pragma unroll
         for (int s4 = 0; s4 < 4; ++s4) df[R][rt][s4] = ld_global16(rp + 512 * s4);
         dfp[R][rt] = pres;
