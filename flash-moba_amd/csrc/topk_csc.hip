@@ -618,10 +618,11 @@ __global__ __launch_bounds__(256, CAP < kBigCap ? 2 : 1) void topk_gate_big_kern
       for (int t = 0; t < NT; ++t)
         if (t < n_tiles) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) cnt += (sc[t][i] > probe) ? 1 : 0;
+          for (int i = 0; i < 16; i += 4) cnt = count4_gt(cnt, sc[t][i], sc[t][i + 1], sc[t][i + 2], sc[t][i + 3], probe);
         }
+      static_assert(PL % 4 == 0, "the winners are counted four at a time");
 #pragma unroll
-      for (int j = 0; j < PL; ++j) cnt += (pv[j] > probe) ? 1 : 0;
+      for (int j = 0; j < PL; j += 4) cnt = count4_gt(cnt, pv[j], pv[j + 1], pv[j + 2], pv[j + 3], probe);
       return sum_xor32_i(cnt);
     };
     float tau = -INFINITY, tau_eq = INFINITY;
@@ -813,6 +814,55 @@ __device__ __forceinline__ double winner_word(float score, int chunk) {
 __device__ __forceinline__ bool winner_real(double w) { return w >= 0.0 && w < (double)INFINITY; }
 __device__ __forceinline__ uint32_t winner_key(double w) { return (uint32_t)(w * (1.0 / kChunkSpan)); }  // (truncates)
 __device__ __forceinline__ int winner_chunk(double w) { return (int)fma(-(double)winner_key(w), kChunkSpan, w); }
+// minimum and maximum of two winners as one instruction each (fmin / fmax first bring every operand that comes round a
+// loop into canonical form, one more instruction per operand and turn; winners are never NaN)
+__device__ __forceinline__ double min_winner(double a, double b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  double d;
+  asm("v_min_f64 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+#else
+  return a < b ? a : b;
+#endif
+}
+__device__ __forceinline__ double max_winner(double a, double b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  double d;
+  asm("v_max_f64 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+#else
+  return a > b ? a : b;
+#endif
+}
+// score and chunk of a list entry (the chunk lies TO_CHUNK bytes after the score), requested here and awaited there: the
+// compiler waits for an LDS read of its own where it issues it when the address comes round a loop.  Nothing else of
+// the wave may be on its way from LDS between the two calls, and the values may only be used after the second.
+template <int TO_CHUNK>
+__device__ __forceinline__ void entrant_request(uint32_t lds_addr, float &score, int &chunk) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("ds_read_b32 %0, %2\n\tds_read_b32 %1, %2 offset:%3" : "=&v"(score), "=&v"(chunk) : "v"(lds_addr), "n"(TO_CHUNK));
+#else
+  score = 0.f;
+  chunk = (int)lds_addr;
+#endif
+}
+__device__ __forceinline__ void entrant_await(float &score, int &chunk) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(score), "+v"(chunk));
+#endif
+}
+// 16 bytes of LDS as ONE read (as a struct of four words the read of the stream gate's operands came out as two
+// 8-byte reads of 4-byte alignment, which meet in half of the banks)
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ Pack8 lds_read16_whole(uint32_t byte_addr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const u32x4_t v = *(__attribute__((address_space(3))) const u32x4_t *)byte_addr;
+  return Pack8{{v[0], v[1], v[2], v[3]}};
+#else
+  (void)byte_addr;
+  return Pack8{{0, 0, 0, 0}};
+#endif
+}
 __device__ __forceinline__ double shfl_xor32_d(double v) {
   const uint64_t u = (uint64_t)__double_as_longlong(v);
   const uint64_t o = ((uint64_t)(uint32_t)shfl_xor32_i((int)(u >> 32)) << 32) | (uint32_t)shfl_xor32_i((int)(uint32_t)u);
@@ -940,27 +990,43 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
     // this group's scores; chunks that are no candidates of the row (its own chunk and later ones) count as -inf
     float sc[NT][16];
     const bool all_cand = __all(nc >= c0 + GC);
+    {
+      // The tiles of the group side by side, and the operands of contraction step ks + 1 on their way from LDS while
+      // the products of step ks run: one tile after the other, every read awaited by its product, a wave spent a
+      // group's worth of LDS latencies in a single chain.  (A tile past the group's last chunk holds copies of
+      // chunks that exist, see tile_issue; its scores are masked like those of every chunk that is no candidate.)
+      f32x16 acc[NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      if (t < n_tiles) {
-        f32x16 acc;
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+        for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+      auto operand = [&](int t, int ks) { return lds_read16_whole(a_row + (uint32_t)(t * 32 * RB) + (uint32_t)(((hh * KS + ks) ^ a_swz) * 16)); };
+      Pack8 af[NT];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const Pack8 af = lds_read16(a_row + (uint32_t)(t * 32 * RB) + (uint32_t)(((hh * KS + ks) ^ a_swz) * 16));
-          acc = mfma32<T>(af, qf[ks], acc);
+      for (int t = 0; t < NT; ++t) af[t] = operand(t, 0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        Pack8 nx[NT];
+        if (ks + 1 < KS) {
+#pragma unroll
+          for (int t = 0; t < NT; ++t) nx[t] = operand(t, ks + 1);
         }
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = mfma32<T>(af[t], qf[ks], acc[t]);
+        if (ks + 1 < KS) {
+#pragma unroll
+          for (int t = 0; t < NT; ++t) af[t] = nx[t];
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
         if (all_cand) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) sc[t][i] = acc[i];
+          for (int i = 0; i < 16; ++i) sc[t][i] = acc[t][i];
         } else {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) sc[t][i] = (c0 + t * 32 + acc_row(i, hh) < nc) ? acc[i] : -INFINITY;
+          for (int i = 0; i < 16; ++i) sc[t][i] = (c0 + t * 32 + acc_row(i, hh) < nc) ? acc[t][i] : -INFINITY;
         }
-      } else {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sc[t][i] = -INFINITY;
       }
     }
     __syncthreads();  // everyone has read the tile: the next group's chunk means may land in it
@@ -970,58 +1036,88 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
     // A row that still has candidates in this group had at least GC of them in the first one, so it already holds
     // kp winners.  Only the new scores that reach its weakest winner can enter (a new chunk has a higher index than
     // every earlier one, so an equal score wins the tie).
+    // In the groups right after the first a row expects about kp ln((g + 1) / g) entrants (every position of a random
+    // stream enters with probability kp / position), which for the second group of a row with sixteen winners is more
+    // than a list takes for some row of nearly every wave: such groups are streamed tile by tile.
     bool streamed = false;
     if (g > 0 && __all(m_prev == kp || nc <= c0)) {
-      const double weakest = fmin(win[0], shfl_xor32_d(win[0]));
-      // (a row without winners, or one whose list is not full because it has no candidates left, admits nothing)
-      const float pmin = winner_real(weakest) ? order_key_float(winner_key(weakest)) : INFINITY;
-      // slot c of the lane with chunks 0..3 is entry c, of its partner entry LS - 1 - c; beyond the list both stay
-      // on the row's last slot
-      const uint32_t slot0 = (uint32_t)(uintptr_t)(my_list_v + (hh ? LS - 1 : 0));
-      const int slot_step = hh ? -4 : 4;  // bytes
-      int cbase = c0 + 4 * hh;
-      asm volatile("" : "+v"(cbase));  // (one register: the compiler would add its scalar and vector parts per position)
-      int cnt = 0;
+      const int part_tiles = (kp > 10 * g) ? 1 : NT;
+      streamed = true;
+#pragma nounroll
+      for (int t0 = 0; t0 < n_tiles; t0 += part_tiles) {
+        const int t1 = t0 + part_tiles;
+        const double weakest = fmin(win[0], shfl_xor32_d(win[0]));
+        // (a row without winners, or one whose list is not full because it has no candidates left, admits nothing)
+        const float pmin = winner_real(weakest) ? order_key_float(winner_key(weakest)) : INFINITY;
+        // slot c of the lane with chunks 0..3 is entry c, of its partner entry LS - 1 - c; beyond the list both stay
+        // on the row's last slot
+        const uint32_t slot0 = (uint32_t)(uintptr_t)(my_list_v + (hh ? LS - 1 : 0));
+        const int slot_step = hh ? -4 : 4;  // bytes
+        int cbase = c0 + 4 * hh;
+        asm volatile("" : "+v"(cbase));  // (one register: the compiler would add its scalar and vector parts per position)
+        int cnt = 0;
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
-        if (t < n_tiles) {
+        for (int t = 0; t < NT; ++t)
+          if (t >= t0 && t < t1 && t < n_tiles) {
 #pragma unroll
-          for (int i4 = 0; i4 < 4; ++i4) {
-            const Flags4 ge = flags4_ge(sc[t][4 * i4], sc[t][4 * i4 + 1], sc[t][4 * i4 + 2], sc[t][4 * i4 + 3], pmin);
+            for (int i4 = 0; i4 < 4; ++i4) {
+              const Flags4 ge = flags4_ge(sc[t][4 * i4], sc[t][4 * i4 + 1], sc[t][4 * i4 + 2], sc[t][4 * i4 + 3], pmin);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const int i = 4 * i4 + j;
-              const uint32_t d = mad24_u32(cnt, slot_step, slot0);
-              lds_write_vec<float>(d, sc[t][i]);
-              lds_write_vec<int>(d + (uint32_t)kToIdx * 4u, cbase + t * 32 + 8 * (i >> 2) + (i & 3));
-              cnt = count_flag(cnt, ge.m[j]);
+              for (int j = 0; j < 4; ++j) {
+                const int i = 4 * i4 + j;
+                const uint32_t d = mad24_u32(cnt, slot_step, slot0);
+                lds_write_vec<float>(d, sc[t][i]);
+                lds_write_vec<int>(d + (uint32_t)kToIdx * 4u, cbase + t * 32 + 8 * (i >> 2) + (i & 3));
+                cnt = count_flag(cnt, ge.m[j]);
+              }
             }
           }
+        const int cnt_o = shfl_xor32_i(cnt);
+        const int ne_row = cnt + cnt_o;
+        if (!__all(ne_row <= CAP)) {
+          // the search below takes over; tiles whose entrants have gone into the winners leave the competition
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            if (t < t0) {
+#pragma unroll
+              for (int i = 0; i < 16; ++i) sc[t][i] = -INFINITY;
+            }
+          streamed = false;
+          break;
         }
-      const int cnt_o = shfl_xor32_i(cnt);
-      const int ne_row = cnt + cnt_o;
-      if (__all(ne_row <= CAP)) {
         wave_lds_fence();
         const int ne_lo = hh ? cnt_o : cnt;  // entrants that came from the bottom of the list
         auto stream = [&](auto plc) {
           constexpr int PLX = decltype(plc)::value;
+          // (entrant e + 1 is on its way from the list while entrant e goes up the entries)
+          auto slot_of = [&](int e) { return e < ne_row ? (e < ne_lo ? e : LS - 1 - (e - ne_lo)) : 0; };
+          const uint32_t list_b = (uint32_t)(uintptr_t)my_list_v;
+          float xv;
+          int xc;
+          entrant_request<kToIdx * 4>(list_b + 4u * (uint32_t)slot_of(0), xv, xc);
+          entrant_await(xv, xc);
 #pragma nounroll
           for (int e = 0; __any(e < ne_row); ++e) {
             const bool has = e < ne_row;
-            const int at = has ? (e < ne_lo ? e : LS - 1 - (e - ne_lo)) : 0;
-            const double x = winner_word(my_list_v[at], reinterpret_cast<const int *>(my_list_v)[kToIdx + at]);
+            const double x = winner_word(xv, xc);
+            float xv_next;
+            int xc_next;
+            entrant_request<kToIdx * 4>(list_b + 4u * (uint32_t)slot_of(e + 1), xv_next, xc_next);
             // the row's weakest winner is the lower of the two lanes' first entries; the lane that holds it drops it
             // and passes the entrant up its sorted entries (a lane that keeps its entries passes its own first entry)
             const double vo = shfl_xor32_d(win[0]);
             const bool rep = has & (win[0] <= vo) & (x > win[0]);
             const double xs = rep ? x : win[0];
             double nw[PLX];
-            nw[0] = fmin(xs, win[1]);
+            nw[0] = min_winner(xs, win[1]);
 #pragma unroll
-            for (int j = 1; j + 1 < PLX; ++j) nw[j] = fmin(fmax(win[j], xs), win[j + 1]);
-            nw[PLX - 1] = fmax(win[PLX - 1], xs);
+            for (int j = 1; j + 1 < PLX; ++j) nw[j] = min_winner(max_winner(win[j], xs), win[j + 1]);
+            nw[PLX - 1] = max_winner(win[PLX - 1], xs);
 #pragma unroll
             for (int j = 0; j < PLX; ++j) win[j] = nw[j];
+            entrant_await(xv_next, xc_next);
+            xv = xv_next;
+            xc = xc_next;
           }
         };
         // (a lane holds at most (kp + 1) / 2 winners; the fillers above them never move)
@@ -1030,7 +1126,6 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
         else
           stream(std::integral_constant<int, PL>{});
         wave_lds_fence();  // (the list takes the next entrants)
-        streamed = true;
       }
     }
     if (streamed) continue;
@@ -1071,10 +1166,11 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
       for (int t = 0; t < NT; ++t)
         if (t < n_tiles) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) cnt += (sc[t][i] > probe) ? 1 : 0;
+          for (int i = 0; i < 16; i += 4) cnt = count4_gt(cnt, sc[t][i], sc[t][i + 1], sc[t][i + 2], sc[t][i + 3], probe);
         }
+      static_assert(PL % 4 == 0, "the winners are counted four at a time");
 #pragma unroll
-      for (int j = 0; j < PL; ++j) cnt += (pv[j] > probe) ? 1 : 0;
+      for (int j = 0; j < PL; j += 4) cnt = count4_gt(cnt, pv[j], pv[j + 1], pv[j + 2], pv[j + 3], probe);
       return sum_xor32_i(cnt);
     };
     float tau = -INFINITY, tau_eq = INFINITY;
@@ -1349,6 +1445,14 @@ __global__ __launch_bounds__(64) void csc_fill_kernel(TopkParams p) {
   const int r0 = seg * p.seg_rows;
   if (r0 >= Lq) return;
   const int r1 = min(Lq, r0 + p.seg_rows);
+  // with the causal rule a row selects no chunk beyond its own: the rows before the word column's first chunk hold zeros
+  int rb0 = r0;
+  if (a.is_causal) {
+    const int64_t off = (int64_t)(a.cu_seqlens_k[b + 1] - a.cu_seqlens_k[b]) - Lq;
+    const int64_t first_row = (int64_t)wc * 32 * a.chunk - off;
+    if (first_row >= r1) return;
+    if (first_row > r0) rb0 = r0 + (int)((first_row - r0) / 64 * 64);
+  }
   const int64_t bh = (int64_t)b * a.heads + h;
   // Where the next rows of chunk wc * 32 + j go: lane j keeps the position relative to the start of the word column's
   // first list (the 32 lists follow each other, far less than 2^30 entries), the start itself is a scalar.  A step
@@ -1364,7 +1468,7 @@ __global__ __launch_bounds__(64) void csc_fill_kernel(TopkParams p) {
       rel = (uint32_t)(a.col_offsets[bh * p.max_cols + c] - first) + (uint32_t)p.segcnt[(bh * p.nseg + seg) * p.max_cols + c];
   }
   const uint32_t *words = p.sel + ((int64_t)h * p.W + wc) * a.total_q + q0;
-  for (int rb = r0; rb < r1; rb += 64) {
+  for (int rb = rb0; rb < r1; rb += 64) {
     const int r = rb + lane;
     const uint32_t w = (r < r1) ? words[r] : 0u;
     // the chunks that some row of the step selects (a scalar, so that the others cost no vector instruction)
