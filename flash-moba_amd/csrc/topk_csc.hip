@@ -245,12 +245,17 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
   float tau_eq = INFINITY;  // no tie group by default
   int n_eq = 0;
   uint32_t iota = 0u;
-  bool any_tie = false;     // some row of the wave has a tie across its cut
-  {
-    uint32_t lo_k = float_order_key(vmin) - 1u;  // count(x > lo) = nc > K'
-    uint32_t hi_k = float_order_key(vmax);       // count(x > hi) = 0  < K'
-    int c_hi = 0;
-    bool open = need;
+  uint32_t lo_k = float_order_key(vmin) - 1u;  // count(x > lo) = nc > K'
+  uint32_t hi_k = float_order_key(vmax);       // count(x > hi) = 0  < K'
+  int c_lo = nc, c_hi = 0;
+  bool open = need;
+  // A row whose bracket holds exactly one score too many, or one too few, needs no more probes: the cut lies right
+  // below the largest score of the bracket, or right at its smallest.  When every open row of the wave is in that state
+  // (about eight probes in, where the search of the slowest row takes twelve or thirteen), one pass over the scores
+  // finds that score for all of them, the largest of -x for the rows that want the smallest.  The cut it gives is
+  // exact unless the score occurs twice; such rows are found by their count below and searched to the end.
+  bool guessed = false;
+  auto bisect = [&](bool may_finish) {
     for (int iter = 0;; ++iter) {
       if (open && hi_k - lo_k <= 1u) {
         // nothing representable strictly inside: every score in (lo, hi] equals hi
@@ -262,6 +267,36 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
         open = false;
       }
       if (!__any(open)) break;
+      if (may_finish) {
+        const bool up = kp - c_hi == 1, dn = c_lo - kp == 1;
+        if (__all(!open || up || dn)) {
+          const bool want_min = open && !up;
+          const uint32_t flip = want_min ? 0x80000000u : 0u;
+          // (x > lo for a score x is x >= the next float above lo, which after -0 is the smallest positive number)
+          const uint32_t above_lo = lo_k + (lo_k == 0x7fffffffu ? 2u : 1u);
+          const float bound = want_min ? -order_key_float(above_lo) : order_key_float(hi_k);
+          float best = -INFINITY;
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            if (t < n_tiles) {
+#pragma unroll
+              for (int i = 0; i < 16; ++i) {
+                const float y = __uint_as_float(__float_as_uint(sc[t][i]) ^ flip);
+                best = fmaxf(best, y <= bound ? y : -INFINITY);
+              }
+            }
+          best = max_xor32_f(best);
+          if (open) {
+            const float v = __uint_as_float(__float_as_uint(best) ^ flip);
+            uint32_t below = float_order_key(v) - 1u;  // (the float below +0 that compares below it is not -0)
+            if (below == 0x7fffffffu) below -= 1u;
+            tau = up ? order_key_float(below) : v;
+            guessed = true;
+            open = false;
+          }
+          break;
+        }
+      }
       uint32_t pk = lo_k + ((hi_k - lo_k) >> 1);
       if (iter < 12) {
         const float mf = 0.5f * order_key_float(lo_k + 1u) + 0.5f * order_key_float(hi_k);
@@ -283,45 +318,95 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
           open = false;
         } else if (cnt > kp) {
           lo_k = pk;
+          c_lo = cnt;
         } else {
           hi_k = pk;
           c_hi = cnt;
         }
       }
     }
-    // a tie group keeps its n_eq highest chunk indices
-    const bool tie = n_eq > 0;
-    any_tie = __any(tie);
-    if (any_tie) {
-      int ceq = 0;
+  };
+  // K' = number of scored chunks to keep (the own chunk takes one slot in causal mode).
+  // A row keeps every candidate x with x > tau, plus, among the candidates equal to tau_eq,
+  // those with chunk index >= iota.  tau is found by bisection between the row's smallest
+  // and largest score and the search stops as soon as exactly K' scores lie above the probe.
+  // The bracket is kept as order-preserving integer keys (lo_k, hi_k]; the first probes
+  // bisect the VALUE range (few steps for ordinary score distributions), later ones the key
+  // range (at most 32 more steps whatever the values).  If the bracket closes first, the
+  // scores inside it are all equal and tie across the cut: the highest chunk indices win.
+  bisect(true);
+  bool any_tie = __any(n_eq > 0);  // some row of the wave has a tie across its cut
+  // Without a tie in the wave a score is selected iff it lies above tau: the flags of the lane's 16 scores of a tile,
+  // shifted in one by one (w + w + flag: one add with carry each), highest first.
+  uint32_t bits[NT];
+  auto flags_above_tau = [&]() {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      bits[t] = 0u;
+      if (t < n_tiles) {
+#pragma unroll
+        for (int i4 = 3; i4 >= 0; --i4) {
+          const Flags4 f = flags4_gt(sc[t][4 * i4 + 3], sc[t][4 * i4 + 2], sc[t][4 * i4 + 1], sc[t][4 * i4], tau);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) bits[t] = shift_in_flag(bits[t], f.m[j]);
+        }
+      }
+    }
+  };
+  if (!any_tie) flags_above_tau();
+  if (__any(guessed)) {
+    int above = 0;
+    if (!any_tie) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) above += __popc(bits[t]);
+    } else {
 #pragma unroll
       for (int t = 0; t < NT; ++t)
         if (t < n_tiles) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) ceq += (sc[t][i] == tau_eq) ? 1 : 0;
+          for (int i = 0; i < 16; i += 4) above = count4_gt(above, sc[t][i], sc[t][i + 1], sc[t][i + 2], sc[t][i + 3], tau);
         }
-      ceq = sum_xor32_i(ceq);
-      const bool split = tie && ceq > n_eq;
-      if (__any(split)) {
-        uint32_t i_acc = 0u;
-        constexpr int IB = (NT * 32 <= 64) ? 6 : (NT * 32 <= 128 ? 7 : 8);
-        for (int bit = IB - 1; bit >= 0; --bit) {
-          const uint32_t trial = i_acc | (1u << bit);
-          int cnt = 0;
+    }
+    above = sum_xor32_i(above);
+    const bool again = guessed && above != kp;
+    if (__any(again)) {
+      open = again;
+      bisect(false);
+      any_tie = __any(n_eq > 0);
+      if (!any_tie) flags_above_tau();
+    }
+  }
+  // a tie group keeps its n_eq highest chunk indices
+  if (any_tie) {
+    const bool tie = n_eq > 0;
+    int ceq = 0;
 #pragma unroll
-          for (int t = 0; t < NT; ++t)
-            if (t < n_tiles) {
+    for (int t = 0; t < NT; ++t)
+      if (t < n_tiles) {
 #pragma unroll
-              for (int i = 0; i < 16; ++i) {
-                const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
-                cnt += ((sc[t][i] == tau_eq) & (c >= trial)) ? 1 : 0;
-              }
-            }
-          cnt = sum_xor32_i(cnt);
-          if (cnt >= n_eq) i_acc = trial;
-        }
-        if (split) iota = i_acc;
+        for (int i = 0; i < 16; ++i) ceq += (sc[t][i] == tau_eq) ? 1 : 0;
       }
+    ceq = sum_xor32_i(ceq);
+    const bool split = tie && ceq > n_eq;
+    if (__any(split)) {
+      uint32_t i_acc = 0u;
+      constexpr int IB = (NT * 32 <= 64) ? 6 : (NT * 32 <= 128 ? 7 : 8);
+      for (int bit = IB - 1; bit >= 0; --bit) {
+        const uint32_t trial = i_acc | (1u << bit);
+        int cnt = 0;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          if (t < n_tiles) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const uint32_t c = (uint32_t)(t * 32 + acc_row(i, hh));
+              cnt += ((sc[t][i] == tau_eq) & (c >= trial)) ? 1 : 0;
+            }
+          }
+        cnt = sum_xor32_i(cnt);
+        if (cnt >= n_eq) i_acc = trial;
+      }
+      if (split) iota = i_acc;
     }
   }
 
@@ -336,17 +421,9 @@ __global__ __launch_bounds__(256, (NT == 8 || HD > 128) ? 2 : 4) void topk_gate_
       uint32_t w = 0u;
       if (t < n_tiles && kp > 0) {
         if (!any_tie) {
-          // no row of the wave has a tie across its cut: a score is selected iff it lies above tau.  The flags of the
-          // lane's 16 scores are shifted in one by one (w + w + flag: one add with carry each), highest first, and the
-          // four nibbles then move to the places of the lane's chunks (4 hh + 8 g .. + 3).
-          uint32_t bits = 0u;
-#pragma unroll
-          for (int i4 = 3; i4 >= 0; --i4) {
-            const Flags4 f = flags4_gt(sc[t][4 * i4 + 3], sc[t][4 * i4 + 2], sc[t][4 * i4 + 1], sc[t][4 * i4], tau);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) bits = shift_in_flag(bits, f.m[j]);
-          }
-          w = ((bits & 0xfu) | ((bits & 0xf0u) << 4) | ((bits & 0xf00u) << 8) | ((bits & 0xf000u) << 12)) << (4 * hh);
+          // the four nibbles of the flags move to the places of the lane's chunks (4 hh + 8 g .. + 3)
+          const uint32_t b = bits[t];
+          w = ((b & 0xfu) | ((b & 0xf0u) << 4) | ((b & 0xf00u) << 8) | ((b & 0xf000u) << 12)) << (4 * hh);
         } else {
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
