@@ -63,6 +63,79 @@ struct BwdWs {
   uint16_t *ds;    // dS tiles (row-stationary dQ form): [row list position / 32][key of the column / 8][position % 32][8 keys]
 };
 
+// MFMAs of the dK/dV pass with the register file of every operand named.  The wave owns all 512 registers of its
+// SIMD lane, 256 ordinary ones and 256 accumulation registers, which only MFMAs and copies can address.  What fits
+// without a copy: dK^T and dV^T (128) and the resident K and V operands (64) in accumulation registers, S and dP and
+// every operand that vector instructions produce or consume in ordinary ones.  Left to itself the compiler puts every
+// MFMA result into accumulation registers, keeps the resident operands there as spills and copies them (and whole
+// accumulator tiles) to and fro around the products: 550 copies per 160 MFMAs of the loop.
+// An MFMA in assembly hides from the compiler that its result arrives late: mfma_results_ready() follows the last
+// product of a chain whose result vector instructions read.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4_t pack8_vec(const Pack8 &p) {
+  u32x4_t v;
+  __builtin_memcpy(&v, &p, 16);
+  return v;
+}
+// c = a b (FIRST) or c += a b: c and a in ordinary registers, b in accumulation registers
+template <typename T, bool FIRST>
+__device__ __forceinline__ void mfma32_b_acc(f32x16 &c, const Pack8 &a, const u32x4_t &b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const u32x4_t av = pack8_vec(a);
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(av), "a"(b));
+    else
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "a"(b));
+  } else {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(av), "a"(b));
+    else
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "a"(b));
+  }
+#else
+  (void)c, (void)a, (void)b;
+#endif
+}
+// c += a b: c in the accumulation registers a[16 SLOT .. 16 SLOT + 15], named so that the sum of a whole walk stays where
+// it is (as a value with a free choice of registers it is copied to ordinary registers and back once per turn of the
+// loop); a and b in ordinary registers
+#define FMOBA_MFMA_SLOT(N, REGS)                                                                                   \
+  if constexpr (SLOT == N) {                                                                                       \
+    if constexpr (std::is_same<T, bf16_t>::value)                                                                  \
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+{" REGS "}"(c) : "v"(av), "v"(bv));              \
+    else                                                                                                           \
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+{" REGS "}"(c) : "v"(av), "v"(bv));               \
+  }
+template <typename T, int SLOT>
+__device__ __forceinline__ void mfma32_c_acc(f32x16 &c, const Pack8 &a, const Pack8 &b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const u32x4_t av = pack8_vec(a), bv = pack8_vec(b);
+  static_assert(SLOT >= 0 && SLOT < 8, "eight accumulator tiles");
+  FMOBA_MFMA_SLOT(0, "a[0:15]")
+  FMOBA_MFMA_SLOT(1, "a[16:31]")
+  FMOBA_MFMA_SLOT(2, "a[32:47]")
+  FMOBA_MFMA_SLOT(3, "a[48:63]")
+  FMOBA_MFMA_SLOT(4, "a[64:79]")
+  FMOBA_MFMA_SLOT(5, "a[80:95]")
+  FMOBA_MFMA_SLOT(6, "a[96:111]")
+  FMOBA_MFMA_SLOT(7, "a[112:127]")
+#else
+  (void)c, (void)a, (void)b;
+#endif
+}
+#undef FMOBA_MFMA_SLOT
+// A 32x32x16 product writes its result eight passes of four clocks after it starts; a vector instruction that reads
+// the result has to start at least eleven instruction slots after the product, which the compiler counts for its own
+// MFMAs and cannot for these.
+__device__ __forceinline__ void mfma_results_ready(f32x16 &x, f32x16 &y) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_nop 7\n\ts_nop 4" : "+v"(x), "+v"(y));
+#else
+  (void)x, (void)y;
+#endif
+}
+
 // DQP = true: dQ partials per visit (for the combine kernel); false: dS^T tiles to ws.ds (for the row-stationary dQ kernel).
 // KB = 1: the workgroup owns 64 keys, wave pair px takes tiles 2 px, 2 px + 1 of a round and wave kq of the pair the
 // key half kq.  KB = 2 (columns of a multiple of 128 keys, whose two 64-key blocks share one row list): it owns 128
@@ -163,14 +236,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   __syncthreads();
   // B operands of S and dP: this lane's key, its half of the head dim; K^T of this wave's half of the features for
   // the dQ products.  They never change, so they stay in registers.
-  Pack8 kb[KS], vb[KS];
+  u32x4_t kb[KS], vb[KS];  // (in accumulation registers)
   Pack8 kt[NDH][4 * KB];
   {
     const uint16_t *sK = reinterpret_cast<const uint16_t *>(smem), *sV = sK + NKEY * LDQ;
 #pragma unroll
     for (int t = 0; t < KS; ++t) {
-      kb[t] = *reinterpret_cast<const Pack8 *>(sK + (kq * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
-      vb[t] = *reinterpret_cast<const Pack8 *>(sV + (kq * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8);
+      kb[t] = pack8_vec(*reinterpret_cast<const Pack8 *>(sK + (kq * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8));
+      vb[t] = pack8_vec(*reinterpret_cast<const Pack8 *>(sV + (kq * 32 + (lane & 31)) * LDQ + (hh * KS + t) * 8));
+#if defined(__HIP_DEVICE_COMPILE__)
+      asm volatile("" : "+a"(kb[t]), "+a"(vb[t]));
+#endif
     }
     if constexpr (DQP) {
       lds_cu16 *trK = tr_lane_base(sK, LDQ, lane) + 8 * hh * LDQ;
@@ -337,18 +413,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     };
     auto mm_a = [&](auto tsc, auto gc) {
       constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
-      if constexpr (G == 0) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          s[TS][i] = 0.f;
-          dp[TS][i] = 0.f;
-        }
-      }
 #pragma unroll
       for (int t = 0; t < KC; ++t) {
-        s[TS] = mfma32<T>(qa[G & 1][t], kb[G * KC + t], s[TS]);
-        dp[TS] = mfma32<T>(doa[G & 1][t], vb[G * KC + t], dp[TS]);
+        if (G == 0 && t == 0) {
+          mfma32_b_acc<T, true>(s[TS], qa[G & 1][t], kb[G * KC + t]);
+          mfma32_b_acc<T, true>(dp[TS], doa[G & 1][t], vb[G * KC + t]);
+        } else {
+          mfma32_b_acc<T, false>(s[TS], qa[G & 1][t], kb[G * KC + t]);
+          mfma32_b_acc<T, false>(dp[TS], doa[G & 1][t], vb[G * KC + t]);
+        }
       }
+      if constexpr (G == 3) mfma_results_ready(s[TS], dp[TS]);
     };
     auto ld_b = [&](auto pc, auto pp, auto tsc, auto gc) {
       constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value) * TB;
@@ -370,8 +445,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 #pragma unroll
       for (int t = 0; t < BC; ++t) {
         const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
-        dv[dt] = mfma32<T>(dot[G & 1][t], pf[TS][s2], dv[dt]);
-        dk[dt] = mfma32<T>(qt[G & 1][t], dsf[TS][s2], dk[dt]);
+        static_for<NDT>([&](auto dc) {
+          constexpr int DT = decltype(dc)::value;
+          if (DT == dt) {
+            mfma32_c_acc<T, 2 * DT>(dv[DT], dot[G & 1][t], pf[TS][s2]);
+            mfma32_c_acc<T, 2 * DT + 1>(dk[DT], qt[G & 1][t], dsf[TS][s2]);
+          }
+        });
       }
     };
     // this lane's key; key j is visible to row r iff r >= row_thr (rows that do not exist are stored as -1)
