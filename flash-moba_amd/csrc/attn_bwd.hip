@@ -97,6 +97,26 @@ __device__ __forceinline__ void mfma32_b_acc(f32x16 &c, const Pack8 &a, const u3
   (void)c, (void)a, (void)b;
 #endif
 }
+// the same with a in accumulation registers and b in ordinary ones
+template <typename T, bool FIRST>
+__device__ __forceinline__ void mfma32_a_acc(f32x16 &c, const u32x4_t &a, const Pack8 &b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const u32x4_t bv = pack8_vec(b);
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "a"(a), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "v"(bv));
+  } else {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "a"(a), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "v"(bv));
+  }
+#else
+  (void)c, (void)a, (void)b;
+#endif
+}
 // c += a b: c in the accumulation registers a[16 SLOT .. 16 SLOT + 15], named so that the sum of a whole walk stays where
 // it is (as a value with a free choice of registers it is copied to ordinary registers and back once per turn of the
 // loop); a and b in ordinary registers
@@ -128,11 +148,18 @@ __device__ __forceinline__ void mfma32_c_acc(f32x16 &c, const Pack8 &a, const Pa
 // A 32x32x16 product writes its result eight passes of four clocks after it starts; a vector instruction that reads
 // the result has to start at least eleven instruction slots after the product, which the compiler counts for its own
 // MFMAs and cannot for these.
-__device__ __forceinline__ void mfma_results_ready(f32x16 &x, f32x16 &y) {
+__device__ __forceinline__ void mfma_results_ready(f32x16 &x, f32x16 &y) {  // (two different results)
 #if defined(__HIP_DEVICE_COMPILE__)
   asm volatile("s_nop 7\n\ts_nop 4" : "+v"(x), "+v"(y));
 #else
   (void)x, (void)y;
+#endif
+}
+__device__ __forceinline__ void mfma_results_ready(f32x16 &x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_nop 7\n\ts_nop 4" : "+v"(x));
+#else
+  (void)x;
 #endif
 }
 
@@ -237,7 +264,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   // B operands of S and dP: this lane's key, its half of the head dim; K^T of this wave's half of the features for
   // the dQ products.  They never change, so they stay in registers.
   u32x4_t kb[KS], vb[KS];  // (in accumulation registers)
-  Pack8 kt[NDH][4 * KB];
+  u32x4_t kt[NDH][4 * KB];  // (in accumulation registers)
   {
     const uint16_t *sK = reinterpret_cast<const uint16_t *>(smem), *sV = sK + NKEY * LDQ;
 #pragma unroll
@@ -255,7 +282,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 #pragma unroll
         for (int d2 = 0; d2 < NDH; ++d2) {
           const int lo = 16 * s4 * LDQ + (kq * NDH + d2) * 32;
-          kt[d2][s4] = tr_frag8_at(trK, lo, lo + 4 * LDQ);
+          kt[d2][s4] = pack8_vec(tr_frag8_at(trK, lo, lo + 4 * LDQ));
+#if defined(__HIP_DEVICE_COMPILE__)
+          asm volatile("" : "+a"(kt[d2][s4]));
+#endif
         }
     }
   }
@@ -525,12 +555,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       constexpr int G = decltype(gc)::value;
 #pragma unroll
       for (int d2 = 0; d2 < NDH; ++d2) {
-        if constexpr (G == 0) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) dqa[d2][i] = 0.f;
+        for (int t = 0; t < KB; ++t) {
+          if (G == 0 && t == 0)
+            mfma32_a_acc<T, true>(dqa[d2], kt[d2][G * KB + t], dsx[G * KB + t]);
+          else
+            mfma32_a_acc<T, false>(dqa[d2], kt[d2][G * KB + t], dsx[G * KB + t]);
         }
-#pragma unroll
-        for (int t = 0; t < KB; ++t) dqa[d2] = mfma32<T>(kt[d2][G * KB + t], dsx[G * KB + t], dqa[d2]);
+      }
+      if constexpr (G == 3) {
+        static_assert(NDH <= 2, "one or two feature tiles of dQ per wave");
+        if constexpr (NDH == 1)
+          mfma_results_ready(dqa[0]);
+        else
+          mfma_results_ready(dqa[0], dqa[1]);
       }
     };
     const int64_t trash = (int64_t)a.total_q * a.heads * ws.cap;  // spare row: takes the writes of absent rows, no branch
