@@ -145,14 +145,20 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
   }
   __syncthreads();
   // K of this block as the A operand of S^T = K Q^T: lane -> key (lane % 32) of each 32-key tile
-  Pack8 kfr[KT][KS];
+  // (kept in accumulation registers, where the MFMAs read them; S^T and O^T tiles are produced in ordinary registers,
+  // where the softmax and the packing read them: no copy between the two register files in the loop)
+  u32x4_t kfr[KT][KS];
   {
     const uint16_t *sK = reinterpret_cast<const uint16_t *>(smem + SM::oQ);
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        kfr[kt][ks] = *reinterpret_cast<const Pack8 *>(sK + (kt * 32 + (lane & 31)) * LDQ + (hh * KS + ks) * 8);
+      for (int ks = 0; ks < KS; ++ks) {
+        kfr[kt][ks] = pack8_vec(*reinterpret_cast<const Pack8 *>(sK + (kt * 32 + (lane & 31)) * LDQ + (hh * KS + ks) * 8));
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("" : "+a"(kfr[kt][ks]));
+#endif
+      }
   }
   if (tid < kFwdRoundRows) {
     sRid[tid] = rid01[0];
@@ -253,11 +259,20 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
     __builtin_amdgcn_sched_barrier(0);
     f32x16 st[KT];  // S^T: register i of tile kt <-> key kt*32 + acc_row(i, hh), this lane's row
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
+    for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) st[kt][i] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) st[kt] = mfma32<T>(kfr[kt][ks], qb[ks], st[kt]);
+      for (int kt = 0; kt < KT; ++kt) {
+        if (ks == 0)
+          mfma32_a_acc<T, true>(st[kt], kfr[kt][ks], qb[ks]);
+        else
+          mfma32_a_acc<T, false>(st[kt], kfr[kt][ks], qb[ks]);
+      }
+    static_assert(KT == 2 || KT == 4, "key blocks of 64 or 128 keys");
+    if constexpr (KT == 2) {
+      mfma_results_ready(st[0], st[1]);
+    } else {
+      mfma_results_ready(st[0], st[1]);
+      mfma_results_ready(st[2], st[3]);
     }
     __builtin_amdgcn_sched_barrier(0);
     // V^T operands of the first half of the feature tiles: their LDS latency runs under the softmax arithmetic
@@ -325,11 +340,15 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
       }
       f32x16 o;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[i] = 0.f;
-#pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) o = mfma32<T>(vt[dt][kt][s2], pf[kt][s2], o);
+        for (int s2 = 0; s2 < 2; ++s2) {
+          if (kt == 0 && s2 == 0)
+            mfma32_vv<T, true>(o, vt[dt][kt][s2], pf[kt][s2]);
+          else
+            mfma32_vv<T, false>(o, vt[dt][kt][s2], pf[kt][s2]);
+        }
+      mfma_results_ready(o);
       // to the wave's row-major output tile, four features (8 bytes) at a time
       uint32_t bo = ldsOut + (uint32_t)(((lane & 31) * LDO + 4 * hh) * 2);
       opaque(bo);

@@ -124,6 +124,126 @@ __device__ __forceinline__ f32x16 mfma32<f16_t>(const Pack8 &a, const Pack8 &b, 
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c, 0, 0, 0);
 }
 
+// MFMAs with the register file of every operand named, for kernels whose waves own all 512 registers of their SIMD
+// lane: 256 ordinary ones and 256 accumulation registers, which only MFMAs and copies can address.  What fits without
+// a copy in the dK/dV pass: dK^T and dV^T (128) and the resident K and V operands (64) in accumulation registers, S
+// and dP and every operand that vector instructions produce or consume in ordinary ones.  Left to itself the compiler
+// puts every MFMA result of such a kernel into accumulation registers, keeps the resident operands there as spills and
+// copies them (and whole accumulator tiles) to and fro around the products: 550 copies per 160 MFMAs of that loop.
+// An MFMA in assembly hides from the compiler that its result arrives late: mfma_results_ready() follows the last
+// product of a chain whose result vector instructions read.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4_t pack8_vec(const Pack8 &p) {
+  u32x4_t v;
+  __builtin_memcpy(&v, &p, 16);
+  return v;
+}
+// c = a b (FIRST) or c += a b: c and a in ordinary registers, b in accumulation registers
+template <typename T, bool FIRST>
+__device__ __forceinline__ void mfma32_b_acc(f32x16 &c, const Pack8 &a, const u32x4_t &b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const u32x4_t av = pack8_vec(a);
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(av), "a"(b));
+    else
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "a"(b));
+  } else {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(av), "a"(b));
+    else
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "a"(b));
+  }
+#else
+  (void)c, (void)a, (void)b;
+#endif
+}
+// c = a b (FIRST) or c += a b, everything in ordinary registers
+template <typename T, bool FIRST>
+__device__ __forceinline__ void mfma32_vv(f32x16 &c, const Pack8 &a, const Pack8 &b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const u32x4_t av = pack8_vec(a), bv = pack8_vec(b);
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(av), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
+  } else {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(av), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
+  }
+#else
+  (void)c, (void)a, (void)b;
+#endif
+}
+// the same with a in accumulation registers and b in ordinary ones
+template <typename T, bool FIRST>
+__device__ __forceinline__ void mfma32_a_acc(f32x16 &c, const u32x4_t &a, const Pack8 &b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const u32x4_t bv = pack8_vec(b);
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "a"(a), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "v"(bv));
+  } else {
+    if constexpr (FIRST)
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "a"(a), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "v"(bv));
+  }
+#else
+  (void)c, (void)a, (void)b;
+#endif
+}
+// c += a b: c in the accumulation registers a[16 SLOT .. 16 SLOT + 15], named so that the sum of a whole walk stays where
+// it is (as a value with a free choice of registers it is copied to ordinary registers and back once per turn of the
+// loop); a and b in ordinary registers
+#define FMOBA_MFMA_SLOT(N, REGS)                                                                                   \
+  if constexpr (SLOT == N) {                                                                                       \
+    if constexpr (std::is_same<T, bf16_t>::value)                                                                  \
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+{" REGS "}"(c) : "v"(av), "v"(bv));              \
+    else                                                                                                           \
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+{" REGS "}"(c) : "v"(av), "v"(bv));               \
+  }
+template <typename T, int SLOT>
+__device__ __forceinline__ void mfma32_c_acc(f32x16 &c, const Pack8 &a, const Pack8 &b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const u32x4_t av = pack8_vec(a), bv = pack8_vec(b);
+  static_assert(SLOT >= 0 && SLOT < 8, "eight accumulator tiles");
+  FMOBA_MFMA_SLOT(0, "a[0:15]")
+  FMOBA_MFMA_SLOT(1, "a[16:31]")
+  FMOBA_MFMA_SLOT(2, "a[32:47]")
+  FMOBA_MFMA_SLOT(3, "a[48:63]")
+  FMOBA_MFMA_SLOT(4, "a[64:79]")
+  FMOBA_MFMA_SLOT(5, "a[80:95]")
+  FMOBA_MFMA_SLOT(6, "a[96:111]")
+  FMOBA_MFMA_SLOT(7, "a[112:127]")
+#else
+  (void)c, (void)a, (void)b;
+#endif
+}
+#undef FMOBA_MFMA_SLOT
+// A 32x32x16 product writes its result eight passes of four clocks after it starts; a vector instruction that reads
+// the result has to start at least eleven instruction slots after the product, which the compiler counts for its own
+// MFMAs and cannot for these.
+__device__ __forceinline__ void mfma_results_ready(f32x16 &x, f32x16 &y) {  // (two different results)
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_nop 7\n\ts_nop 4" : "+v"(x), "+v"(y));
+#else
+  (void)x, (void)y;
+#endif
+}
+__device__ __forceinline__ void mfma_results_ready(f32x16 &x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_nop 7\n\ts_nop 4" : "+v"(x));
+#else
+  (void)x;
+#endif
+}
+
 // MFMA 16x16x32 (gfx950).  Operand layout, lane l, g = l / 16:
 //   A (16 x 32): lane holds A[l % 16][g*8 .. g*8+7]
 //   B (32 x 16): lane holds B[g*8 .. g*8+7][l % 16]

@@ -930,7 +930,6 @@ __device__ __forceinline__ void entrant_await(float &score, int &chunk) {
 }
 // 16 bytes of LDS as ONE read (as a struct of four words the read of the stream gate's operands came out as two
 // 8-byte reads of 4-byte alignment, which meet in half of the banks)
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ Pack8 lds_read16_whole(uint32_t byte_addr) {
 #if defined(__HIP_DEVICE_COMPILE__)
   const u32x4_t v = *(__attribute__((address_space(3))) const u32x4_t *)byte_addr;
