@@ -297,9 +297,34 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     const uint32_t rowoff = (uint32_t)((lane & 31) * RB + (((hh * KS) ^ tile_swz<HD>(lane & 31)) * 16));
     const int li = lane & 15, r0t = (li >> 2) + 4 * hh;
     const uint32_t troff = (uint32_t)(r0t * RB + ((((((lane >> 4) & 1) * 2 + ((li & 3) >> 1))) ^ tile_swz<HD>(r0t)) * 16) + (li & 1) * 8);
-    // (re-made opaque wherever they are used: the operand addresses derived from them must not be kept in
-    // registers from one use to the next, there are none to spare)
-    uint32_t aQ = pairQ + rowoff, adO = pairdO + rowoff, tQ = pairQ + troff, tdO = pairdO + troff;  // (never change; not const so that they can be made opaque in place)
+    // The operand addresses derived from them (an exclusive-or per piece) are formed once and stay in registers: the
+    // products leave room for them since their sums live in the accumulation registers.  (Made opaque, or the
+    // compiler forms them again at every read.)
+    // (The form with dQ partials has no registers to spare: there the bases are re-made opaque wherever they are used,
+    // so that nothing derived from them is kept from one use to the next.)
+    constexpr bool kKeepAddresses = !DQP;
+    uint32_t aQ = pairQ + rowoff, adO = pairdO + rowoff, tQ = pairQ + troff, tdO = pairdO + troff;
+    uint32_t aQk[KS], adOk[KS];                              // row reads: piece hh * KS + k of this lane's row
+    uint32_t tQlo[NDT], tQhi[NDT], tdOlo[NDT], tdOhi[NDT];  // transposing reads: feature tile dt, rows (0..3) + 4 hh and the same + 8
+#pragma unroll
+    for (int k = 0; k < (kKeepAddresses ? KS : 0); ++k) {
+      aQk[k] = aQ ^ (uint32_t)(k * 16);
+      adOk[k] = adO ^ (uint32_t)(k * 16);
+#if defined(__HIP_DEVICE_COMPILE__)
+      asm volatile("" : "+v"(aQk[k]), "+v"(adOk[k]));
+#endif
+    }
+#pragma unroll
+    for (int dt = 0; dt < (kKeepAddresses ? NDT : 0); ++dt) {
+      const uint32_t xlo = (uint32_t)(dt * 4 * 16), xhi = (uint32_t)(((dt * 4) ^ TileSwz<HD>::kRow8) * 16);
+      tQlo[dt] = tQ ^ xlo;
+      tQhi[dt] = tQ ^ xhi;
+      tdOlo[dt] = tdO ^ xlo;
+      tdOhi[dt] = tdO ^ xhi;
+#if defined(__HIP_DEVICE_COMPILE__)
+      asm volatile("" : "+v"(tQlo[dt]), "+v"(tQhi[dt]), "+v"(tdOlo[dt]), "+v"(tdOhi[dt]));
+#endif
+    }
     auto opaque = [](uint32_t &x, uint32_t &y) {
 #if defined(__HIP_DEVICE_COMPILE__)
       asm volatile("" : "+v"(x), "+v"(y));
@@ -334,11 +359,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     auto ld_a = [&](auto pc, auto pp, auto tsc, auto gc) {
       constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value) * TB;
       constexpr int G = decltype(gc)::value;
-      opaque(aQ, adO);
+      if constexpr (!kKeepAddresses) opaque(aQ, adO);
 #pragma unroll
       for (int t = 0; t < KC; ++t) {
-        qa[G & 1][t] = lds_read16((aQ ^ (uint32_t)((G * KC + t) * 16)) + TO);
-        doa[G & 1][t] = lds_read16((adO ^ (uint32_t)((G * KC + t) * 16)) + TO);
+        if constexpr (kKeepAddresses) {
+          qa[G & 1][t] = lds_read16(aQk[G * KC + t] + TO);
+          doa[G & 1][t] = lds_read16(adOk[G * KC + t] + TO);
+        } else {
+          qa[G & 1][t] = lds_read16((aQ ^ (uint32_t)((G * KC + t) * 16)) + TO);
+          doa[G & 1][t] = lds_read16((adO ^ (uint32_t)((G * KC + t) * 16)) + TO);
+        }
       }
     };
     auto mm_a = [&](auto tsc, auto gc) {
@@ -358,15 +388,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     auto ld_b = [&](auto pc, auto pp, auto tsc, auto gc) {
       constexpr uint32_t TO = (uint32_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value) * TB;
       constexpr int G = decltype(gc)::value;
-      opaque(tQ, tdO);
+      if constexpr (!kKeepAddresses) opaque(tQ, tdO);
 #pragma unroll
       for (int t = 0; t < BC; ++t) {
         const int pi = G * BC + t, dt = pi >> 1, s2 = pi & 1;
         // rows 16 s2 + (0..3) + 4 hh and the same + 8, features dt * 32 ..
-        const uint32_t xlo = (uint32_t)(dt * 4 * 16), xhi = (uint32_t)(((dt * 4) ^ TileSwz<HD>::kRow8) * 16);
         const uint32_t olo = TO + (uint32_t)(16 * s2 * RB), ohi = olo + (uint32_t)(8 * RB);
-        dot[G & 1][t] = lds_tr8((tdO ^ xlo) + olo, (tdO ^ xhi) + ohi);
-        qt[G & 1][t] = lds_tr8((tQ ^ xlo) + olo, (tQ ^ xhi) + ohi);
+        if constexpr (kKeepAddresses) {
+          dot[G & 1][t] = lds_tr8(tdOlo[dt] + olo, tdOhi[dt] + ohi);
+          qt[G & 1][t] = lds_tr8(tQlo[dt] + olo, tQhi[dt] + ohi);
+        } else {
+          const uint32_t xlo = (uint32_t)(dt * 4 * 16), xhi = (uint32_t)(((dt * 4) ^ TileSwz<HD>::kRow8) * 16);
+          dot[G & 1][t] = lds_tr8((tdO ^ xlo) + olo, (tdO ^ xhi) + ohi);
+          qt[G & 1][t] = lds_tr8((tQ ^ xlo) + olo, (tQ ^ xhi) + ohi);
+        }
       }
     };
     auto mm_b = [&](auto tsc, auto gc) {

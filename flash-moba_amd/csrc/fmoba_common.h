@@ -49,6 +49,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 template <typename T> struct ElemTraits;
 template <> struct ElemTraits<f16_t> {
@@ -132,7 +133,6 @@ __device__ __forceinline__ f32x16 mfma32<f16_t>(const Pack8 &a, const Pack8 &b, 
 // copies them (and whole accumulator tiles) to and fro around the products: 550 copies per 160 MFMAs of that loop.
 // An MFMA in assembly hides from the compiler that its result arrives late: mfma_results_ready() follows the last
 // product of a chain whose result vector instructions read.
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ u32x4_t pack8_vec(const Pack8 &p) {
   u32x4_t v;
   __builtin_memcpy(&v, &p, 16);
@@ -599,10 +599,13 @@ struct TileSwz {
   static constexpr int kRow8 = HD > 64 ? 2 : 0;  // tile_swz(r + 8) ^ tile_swz(r)
 };
 
-typedef __attribute__((address_space(3))) const Pack8 lds_cpack8;
+// (read as ONE vector: as a struct of four words the read is split and put together again by what the compiler knows
+// of the address bits, and where it knows nothing -- an address that comes out of an assembly statement, or round a
+// loop -- it comes out as two 8-byte reads of 4-byte alignment, which meet in half of the banks)
 __device__ __forceinline__ Pack8 lds_read16(uint32_t byte_addr) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  return *(lds_cpack8 *)byte_addr;
+  const u32x4_t v = *(__attribute__((address_space(3))) const u32x4_t *)byte_addr;
+  return Pack8{{v[0], v[1], v[2], v[3]}};
 #else
   (void)byte_addr;
   return Pack8{{0, 0, 0, 0}};

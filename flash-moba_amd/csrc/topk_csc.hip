@@ -928,17 +928,6 @@ __device__ __forceinline__ void entrant_await(float &score, int &chunk) {
   asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(score), "+v"(chunk));
 #endif
 }
-// 16 bytes of LDS as ONE read (as a struct of four words the read of the stream gate's operands came out as two
-// 8-byte reads of 4-byte alignment, which meet in half of the banks)
-__device__ __forceinline__ Pack8 lds_read16_whole(uint32_t byte_addr) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  const u32x4_t v = *(__attribute__((address_space(3))) const u32x4_t *)byte_addr;
-  return Pack8{{v[0], v[1], v[2], v[3]}};
-#else
-  (void)byte_addr;
-  return Pack8{{0, 0, 0, 0}};
-#endif
-}
 __device__ __forceinline__ double shfl_xor32_d(double v) {
   const uint64_t u = (uint64_t)__double_as_longlong(v);
   const uint64_t o = ((uint64_t)(uint32_t)shfl_xor32_i((int)(u >> 32)) << 32) | (uint32_t)shfl_xor32_i((int)(uint32_t)u);
@@ -1076,7 +1065,7 @@ __global__ __launch_bounds__(256, NT <= 2 ? 3 : 2) void topk_gate_stream_kernel(
       for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
-      auto operand = [&](int t, int ks) { return lds_read16_whole(a_row + (uint32_t)(t * 32 * RB) + (uint32_t)(((hh * KS + ks) ^ a_swz) * 16)); };
+      auto operand = [&](int t, int ks) { return lds_read16(a_row + (uint32_t)(t * 32 * RB) + (uint32_t)(((hh * KS + ks) ^ a_swz) * 16)); };
       Pack8 af[NT];
 #pragma unroll
       for (int t = 0; t < NT; ++t) af[t] = operand(t, 0);
