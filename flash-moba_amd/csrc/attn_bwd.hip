@@ -1133,27 +1133,40 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_combine_kernel(fmoba_attn_bwd
 
 // grid (ceil(max_seqlen_q / rows_per_block), heads, batch), block 256.
 // LPR lanes cooperate on one row (LPR = power of two >= head_dim / 8).
+constexpr int kPrepRows = 4;  // rows per thread: eight 16-byte loads in flight (with one row a thread had two, 4.7 TB/s)
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_prep_kernel(fmoba_attn_bwd_args a, int LPR) {
-  const int rows_per_block = 256 / LPR;
+  const int rows_per_pass = 256 / LPR;
   const int h = blockIdx.y, b = blockIdx.z;
   const int q0 = a.cu_seqlens_q[b], Lq = a.cu_seqlens_q[b + 1] - q0;
-  const int r = blockIdx.x * rows_per_block + threadIdx.x / LPR;
+  const int r0 = blockIdx.x * rows_per_pass * kPrepRows + threadIdx.x / LPR;
+  if (blockIdx.x * rows_per_pass * kPrepRows >= Lq) return;
   const int sub = threadIdx.x % LPR;
   const int e = sub * 8;
   const int D = a.head_dim;
-  float acc = 0.f;
-  if (r < Lq && e < D) {
-    const Pack8 o = ld_global16(reinterpret_cast<const uint16_t *>(a.out) + (int64_t)(q0 + r) * a.o_row_stride + (int64_t)h * a.o_head_stride + e);
-    const Pack8 g = ld_global16(reinterpret_cast<const uint16_t *>(a.dout) + (int64_t)(q0 + r) * a.do_row_stride + (int64_t)h * a.do_head_stride + e);
+  Pack8 o[kPrepRows], g[kPrepRows];
+#pragma unroll
+  for (int k = 0; k < kPrepRows; ++k) {
+    const int r = r0 + k * rows_per_pass;
+    o[k] = zero_pack8();
+    g[k] = zero_pack8();
+    if (r < Lq && e < D) {
+      o[k] = ld_global16(reinterpret_cast<const uint16_t *>(a.out) + (int64_t)(q0 + r) * a.o_row_stride + (int64_t)h * a.o_head_stride + e);
+      g[k] = ld_global16(reinterpret_cast<const uint16_t *>(a.dout) + (int64_t)(q0 + r) * a.do_row_stride + (int64_t)h * a.do_head_stride + e);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kPrepRows; ++k) {
+    const int r = r0 + k * rows_per_pass;
     float fo[8], fg[8];
-    unpack8<T>(o, fo);
-    unpack8<T>(g, fg);
+    unpack8<T>(o[k], fo);
+    unpack8<T>(g[k], fg);
+    float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc = fmaf(fo[i], fg[i], acc);
+    for (int w = LPR >> 1; w >= 1; w >>= 1) acc += __shfl_xor(acc, w, 64);
+    if (r < Lq && sub == 0) a.softmax_d[(int64_t)h * ((int64_t)a.total_q + 128 * (int64_t)a.batch) + q0 + 128 * b + r] = acc;
   }
-  for (int o = LPR >> 1; o >= 1; o >>= 1) acc += __shfl_xor(acc, o, 64);
-  if (r < Lq && sub == 0) a.softmax_d[(int64_t)h * ((int64_t)a.total_q + 128 * (int64_t)a.batch) + q0 + 128 * b + r] = acc;
 }
 
 __global__ void zero_rows_kernel(void *p, int64_t rows, int64_t row_stride, int heads, int64_t head_stride, int D) {
@@ -1246,7 +1259,7 @@ static int run_bwd(const fmoba_attn_bwd_args &a, const BwdWs &ws, int phases, hi
     int lpr = 1;
     while (lpr * 8 < a.head_dim) lpr <<= 1;
     const int rows_per_block = 256 / lpr;
-    hipLaunchKernelGGL(bwd_prep_kernel<T>, dim3(ceil_div(a.max_seqlen_q, rows_per_block), a.heads, a.batch), dim3(256), 0, s, a, lpr);
+    hipLaunchKernelGGL(bwd_prep_kernel<T>, dim3(ceil_div(a.max_seqlen_q, rows_per_block * kPrepRows), a.heads, a.batch), dim3(256), 0, s, a, lpr);
   }
   if (a.head_dim > 128) {
     // the plain feature-split dK/dV kernel (attn_bwd_wide.hip), then the row-block dQ pass over its dS tiles
