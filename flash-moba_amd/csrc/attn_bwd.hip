@@ -63,6 +63,18 @@ struct BwdWs {
   uint16_t *ds;    // dS tiles (row-stationary dQ form): [row list position / 32][key of the column / 8][position % 32][8 keys]
 };
 
+// a * b of two values below 2^24, b the same in every lane: one full-rate instruction (a 32-bit multiply takes four
+// times as long)
+__device__ __forceinline__ uint32_t mul24_u32(uint32_t a, uint32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  uint32_t d;
+  asm("v_mul_u32_u24 %0, %1, %2" : "=v"(d) : "v"(a), "s"(b));
+  return d;
+#else
+  return a * b;
+#endif
+}
+
 // DQP = true: dQ partials per visit (for the combine kernel); false: dS^T tiles to ws.ds (for the row-stationary dQ kernel).
 // KB = 1: the workgroup owns 64 keys, wave pair px takes tiles 2 px, 2 px + 1 of a round and wave kq of the pair the
 // key half kq.  KB = 2 (columns of a multiple of 128 keys, whose two 64-key blocks share one row list): it owns 128
@@ -250,6 +262,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         sDelta[i] = ok ? m_del : 0.f;
       }
     };
+    const bool near_rows = Lq < (1 << 24) && a.q_row_stride < (1 << 22) && a.do_row_stride < (1 << 22) &&
+                           (int64_t)Lq * a.q_row_stride < (int64_t)0x7fff0000 && (int64_t)Lq * a.do_row_stride < (int64_t)0x7fff0000;
     auto tile_issue = [&](int sr) {  // tile `wave` of round sr
       constexpr int RPI = 64 / VPR, NI = 32 / RPI;  // tile rows per instruction, instructions per tile
       const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
@@ -261,11 +275,22 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       int src[NI];
 #pragma unroll
       for (int i = 0; i < NI; ++i) src[i] = sRid[(sr & 1) * kBwdRoundRows + wave * 32 + i * RPI + rl] & 0x7fffffff;
+      if (near_rows) {
+        // the sequence's rows lie within 4 GB of its first one: a 32-bit byte offset per lane from a wave-uniform base,
+        // one full-rate multiply (the 64-bit products take four times as long, and an address takes two more additions)
 #pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const uint32_t e = (uint32_t)min((p ^ tile_swz<HD>(i * RPI + rl)) * 8, D - 8);
-        global_to_lds16(qg + ((uint64_t)(uint32_t)src[i] * qs + e), ldsQ + dst + (uint32_t)(i * RPI * RB));
-        global_to_lds16(dog + ((uint64_t)(uint32_t)src[i] * dos + e), ldsdO + dst + (uint32_t)(i * RPI * RB));
+        for (int i = 0; i < NI; ++i) {
+          const uint32_t e2 = (uint32_t)min((p ^ tile_swz<HD>(i * RPI + rl)) * 8, D - 8) * 2u;
+          global_to_lds16_sbase(mul24_u32((uint32_t)src[i], qs * 2u) + e2, qg, ldsQ + dst + (uint32_t)(i * RPI * RB));
+          global_to_lds16_sbase(mul24_u32((uint32_t)src[i], dos * 2u) + e2, dog, ldsdO + dst + (uint32_t)(i * RPI * RB));
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          const uint32_t e = (uint32_t)min((p ^ tile_swz<HD>(i * RPI + rl)) * 8, D - 8);
+          global_to_lds16(qg + ((uint64_t)(uint32_t)src[i] * qs + e), ldsQ + dst + (uint32_t)(i * RPI * RB));
+          global_to_lds16(dog + ((uint64_t)(uint32_t)src[i] * dos + e), ldsdO + dst + (uint32_t)(i * RPI * RB));
+        }
       }
     };
 
@@ -747,18 +772,6 @@ __device__ __forceinline__ DqItem dq_decode_item(int id, int npairs, int nsb_max
   w.pair = item.pair < npairs ? item.pair : -1;
   w.sb = nsb_max - 1 - item.idx;
   return w;
-}
-
-// a * b of two values below 2^24, b the same in every lane: one full-rate instruction (a 32-bit multiply takes four
-// times as long)
-__device__ __forceinline__ uint32_t mul24_u32(uint32_t a, uint32_t b) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  uint32_t d;
-  asm("v_mul_u32_u24 %0, %1, %2" : "=v"(d) : "v"(a), "s"(b));
-  return d;
-#else
-  return a * b;
-#endif
 }
 
 template <int N>
