@@ -374,7 +374,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     Pack8 qa[2][KC], doa[2][KC];     // A operands of S and dP (this lane's row, its half of the head dim), double-buffered by chunk
     Pack8 dot[2][BC], qt[2][BC];     // dO^T / Q^T operands of the dV / dK products, double-buffered by chunk
     f32x4 lse4[2], del4[2];          // softmax inputs of a chunk's four rows
-    int4 row4[2];
     Pack8 pf[2][2], dsf[2][2];       // P and dS of both tiles of the round as MFMA operands
     Pack8 dsx[4 * KB];               // dS^T of all keys of the block as the B operand of the dQ products
     f32x16 dqa[NDH];
@@ -396,12 +395,35 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         }
       }
     };
-    auto mm_a = [&](auto tsc, auto gc) {
+    // this lane's key; key j is visible to row r iff r >= row_thr (rows that do not exist are stored as -1)
+    const int j = key0 + kq * 32 + (lane & 31);
+    const int row_thr = j >= Lk ? 0x7fffffff : (causal ? max(0, j - off) : 0);
+    // rows from this one on see every key of the block (no row does if the block reaches past the sequence)
+    const int all_visible_from = key0 + NKEY > Lk ? 0x7fffffff : (causal ? max(0, key0 + NKEY - 1 - off) : 0);
+    // The causal rule and the end of the sequence enter S as its starting value: 0 where row and key see each other,
+    // -inf elsewhere (the products then leave -inf there and the exponential gives 0), and only in rounds that have
+    // such pairs at all (`masked`, the same for the whole wave): the rows of a list come in ascending order, so
+    // from the first row that sees every key of the block on, S starts from nothing and no comparison is made.
+    auto mm_a = [&](auto pc, auto pp, auto tsc, auto gc, bool masked) {
       constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
 #pragma unroll
       for (int t = 0; t < KC; ++t) {
         if (G == 0 && t == 0) {
-          mfma32_b_acc<T, true>(s[TS], qa[G & 1][t], kb[G * KC + t]);
+          if (masked) {
+            constexpr int TSG = decltype(pc)::value * 4 + decltype(pp)::value * 2 + TS;
+            opaque1(smx0);
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+              const int4 r4 = lds_read_vec<int4>(smx0 + (uint32_t)(TSG * 32 + 8 * g4) * 4);
+              s[TS][4 * g4] = r4.x >= row_thr ? 0.f : -INFINITY;
+              s[TS][4 * g4 + 1] = r4.y >= row_thr ? 0.f : -INFINITY;
+              s[TS][4 * g4 + 2] = r4.z >= row_thr ? 0.f : -INFINITY;
+              s[TS][4 * g4 + 3] = r4.w >= row_thr ? 0.f : -INFINITY;
+            }
+            mfma32_b_acc<T, false>(s[TS], qa[G & 1][t], kb[G * KC + t]);
+          } else {
+            mfma32_b_acc<T, true>(s[TS], qa[G & 1][t], kb[G * KC + t]);
+          }
           mfma32_b_acc<T, true>(dp[TS], doa[G & 1][t], vb[G * KC + t]);
         } else {
           mfma32_b_acc<T, false>(s[TS], qa[G & 1][t], kb[G * KC + t]);
@@ -444,27 +466,22 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         });
       }
     };
-    // this lane's key; key j is visible to row r iff r >= row_thr (rows that do not exist are stored as -1)
-    const int j = key0 + kq * 32 + (lane & 31);
-    const int row_thr = j >= Lk ? 0x7fffffff : (causal ? max(0, j - off) : 0);
     auto ld_s = [&](auto pc, auto pp, auto tsc, auto gc) {
       constexpr int TS = decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value, G = decltype(gc)::value;
       // accumulator registers 4G..4G+3 hold rows TS * 32 + 8 G + 4 hh + (0..3); one address register, the rest
       // are offsets in the instructions
       constexpr uint32_t O = (uint32_t)(TS * 32 + 8 * G) * 4;
       opaque1(smx0);
-      row4[G & 1] = lds_read_vec<int4>(smx0 + O);
       lse4[G & 1] = lds_read_vec<f32x4>(smx0 + O + (uint32_t)(SM::oLse - SM::oRow));
       del4[G & 1] = lds_read_vec<f32x4>(smx0 + O + (uint32_t)(SM::oDelta - SM::oRow));
     };
     auto smx = [&](auto tsc, auto gc) {
       constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
-      const int rr[4] = {row4[G & 1].x, row4[G & 1].y, row4[G & 1].z, row4[G & 1].w};
       float pr[4], ds[4];
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
         const int i = 4 * G + jj;
-        const float x = rr[jj] >= row_thr ? fmaf(s[TS][i], scale_log2, -lse4[G & 1][jj]) : -INFINITY;
+        const float x = fmaf(s[TS][i], scale_log2, -lse4[G & 1][jj]);  // (-inf for a masked pair, see mm_a)
         pr[jj] = __builtin_amdgcn_exp2f(x);
         ds[jj] = pr[jj] * (dp[TS][i] - del4[G & 1][jj]);
       }
@@ -567,13 +584,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     // absent rows (row id -1, zero data): they run through the same code and add nothing.
     auto process_round = [&](auto pc, auto pp, int r) {  // pc: parity of r = the LDS buffer that holds the round
       const int tile0 = 4 * r + 2 * (KB == 1 ? px : decltype(pp)::value);  // position of the pair's first tile in the list
+      // (the first row of the pair's first tile is its earliest; -1 if the pair has no row)
+      const bool masked = __builtin_amdgcn_readfirstlane(pRow[(decltype(pc)::value * 4 + decltype(pp)::value * 2) * 32]) < all_visible_from;
       // S, dP of the first tile
       ld_a(pc, pp, C0{}, C0{});
       fence();
       static_for<4>([&](auto gc) {
         constexpr int G = decltype(gc)::value;
         if constexpr (G < 3) ld_a(pc, pp, C0{}, std::integral_constant<int, G + 1>{});
-        mm_a(C0{}, gc);
+        mm_a(pc, pp, C0{}, gc, masked);
         fence();
       });
       // S, dP of the second tile between the softmax rows of the first
@@ -586,7 +605,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           ld_a(pc, pp, C1{}, std::integral_constant<int, G + 1>{});
           ld_s(pc, pp, C0{}, std::integral_constant<int, G + 1>{});
         }
-        mm_a(C1{}, gc);
+        mm_a(pc, pp, C1{}, gc, masked);
         smx(C0{}, gc);
         fence();
       });
