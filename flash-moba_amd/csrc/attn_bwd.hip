@@ -591,19 +591,24 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       fence();
       static_for<4>([&](auto gc) {
         constexpr int G = decltype(gc)::value;
-        if constexpr (G < 3) ld_a(pc, pp, C0{}, std::integral_constant<int, G + 1>{});
+        if constexpr (G < 3) {
+          ld_a(pc, pp, C0{}, std::integral_constant<int, G + 1>{});
+        } else {  // the first operands of the next stage: a stage that began with its own reads began with their latency
+          ld_a(pc, pp, C1{}, C0{});
+          ld_s(pc, pp, C0{}, C0{});
+        }
         mm_a(pc, pp, C0{}, gc, masked);
         fence();
       });
       // S, dP of the second tile between the softmax rows of the first
-      ld_a(pc, pp, C1{}, C0{});
-      ld_s(pc, pp, C0{}, C0{});
-      fence();
       static_for<4>([&](auto gc) {
         constexpr int G = decltype(gc)::value;
         if constexpr (G < 3) {
           ld_a(pc, pp, C1{}, std::integral_constant<int, G + 1>{});
           ld_s(pc, pp, C0{}, std::integral_constant<int, G + 1>{});
+        } else {
+          ld_b(pc, pp, C0{}, C0{});
+          ld_s(pc, pp, C1{}, C0{});
         }
         mm_a(pc, pp, C1{}, gc, masked);
         smx(C0{}, gc);
@@ -613,8 +618,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       // (a second pair of the same waves reuses the dS^T tiles of the first: its readers have to be done)
       if constexpr (DQP && decltype(pp)::value == 1) __syncthreads();
       ds_write(C0{});
-      ld_b(pc, pp, C0{}, C0{});
-      ld_s(pc, pp, C1{}, C0{});
       if constexpr (!DQP) ds_read(pc, pp, C0{});
       fence();
       static_for<4>([&](auto gc) {
@@ -622,6 +625,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         if constexpr (G < 3) {
           ld_b(pc, pp, C0{}, std::integral_constant<int, G + 1>{});
           ld_s(pc, pp, C1{}, std::integral_constant<int, G + 1>{});
+        } else {
+          ld_b(pc, pp, C1{}, C0{});
         }
         mm_b(C0{}, gc);
         smx(C1{}, gc);
@@ -632,7 +637,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       // groups have put dS^T of both tiles into LDS, so the one barrier the exchange needs hardly ever waits
       ds_write(C1{});
       if constexpr (DQP) __syncthreads();
-      ld_b(pc, pp, C1{}, C0{});
       if constexpr (DQP)
         dq_load(C0{});
       else
