@@ -104,18 +104,18 @@ def time_events(fn, iters, warmup=1):
 # same counter reads for a plain 1 GiB copy (the summaries of those runs are kept under profiles/, one per workload).
 # Counter runs cannot be made from inside this script, so the figures are the committed measurement.
 MEASURED_TRAFFIC_BYTES = {
-    ("headline", "attn_fwd_rows_kernel"): 1.297e9,
-    ("headline", "attn_bwd_dkdv_kernel"): 6.686e9,
-    ("headline", "attn_bwd_dq_kernel"): 5.132e9,
-    ("c2", "attn_fwd_col_kernel"): 4.420e8,
-    ("c3", "attn_fwd_col_kernel"): 8.219e9,
-    ("c3", "attn_bwd_dkdv_kernel"): 1.302e10,
+    ("headline", "attn_fwd_rows_kernel"): 1.296e9,
+    ("headline", "attn_bwd_dkdv_kernel"): 6.689e9,
+    ("headline", "attn_bwd_dq_kernel"): 5.114e9,
+    ("c2", "attn_fwd_col_kernel"): 4.422e8,
+    ("c3", "attn_fwd_col_kernel"): 8.220e9,
+    ("c3", "attn_bwd_dkdv_kernel"): 1.279e10,
     ("c5", "attn_fwd_col_kernel"): 3.995e10,
-    ("c5", "attn_bwd_dkdv_kernel"): 6.651e10,
-    ("sweep16k", "attn_fwd_col_kernel"): 1.942e9,
-    ("sweep16k", "attn_bwd_dkdv_kernel"): 2.971e9,
-    ("sweep64k", "attn_fwd_col_kernel"): 9.668e9,
-    ("sweep64k", "attn_bwd_dkdv_kernel"): 1.558e10,
+    ("c5", "attn_bwd_dkdv_kernel"): 6.636e10,
+    ("sweep16k", "attn_fwd_col_kernel"): 1.941e9,
+    ("sweep16k", "attn_bwd_dkdv_kernel"): 2.946e9,
+    ("sweep64k", "attn_fwd_col_kernel"): 9.670e9,
+    ("sweep64k", "attn_bwd_dkdv_kernel"): 1.551e10,
 }
 
 
