@@ -697,6 +697,37 @@ def test_backward_both_dq_forms(fm, dq_mode, d, chunk):
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
 
 
+@pytest.mark.parametrize("dq_mode", [1, 2])
+def test_backward_with_rows_far_apart(fm, dq_mode):
+    # The dK/dV pass fetches the rows of a list with a 32-bit byte offset per lane where a sequence's rows lie within
+    # 4 GB of its first one, and with 64-bit addresses otherwise: q and dout as views with a row stride of 2^22
+    # elements (8 MB) take the second way and must give the bits of the packed tensors.
+    lens = [200, 90]
+    d, chunk, heads = 128, 64, 2
+    q, k, v, cu, dout = O.make_inputs(lens, heads, d, chunk, 35, torch.bfloat16, with_dout=True)
+    Q, K, V, CU, DO = q.cuda(), k.cuda(), v.cuda(), cu.cuda(), dout.cuda()
+    co, cn, ind = fm.api.flash_topk_varlen_func(Q, K, CU, CU, max(lens), max(lens), 2, chunk, causal=True)
+    scale = d ** -0.5
+    out, lse, _, _ = fm.hip.moba_varlen_fwd(Q, K, V, None, co, cn, ind, CU, CU, None, None, None, max(lens), max(lens), 0.0, scale,
+                                            False, True, 0.0, False, 128, chunk, None)
+    ref = fm.hip.moba_varlen_bwd(DO, Q, K, V, out, lse, None, None, None, co, cn, ind, CU, CU, None, max(lens), max(lens),
+                                 0.0, scale, False, True, 0.0, False, 128, chunk, None, None, _dq_mode=dq_mode)[:3]
+    total = sum(lens)
+    wide = 1 << 22
+
+    def far_apart(t):
+        big = torch.zeros((total, wide), dtype=t.dtype, device=t.device)
+        view = big[:, :heads * d].view(total, heads, d)
+        view.copy_(t)
+        assert view.stride(0) == wide and view.stride(1) == d
+        return view
+
+    got = fm.hip.moba_varlen_bwd(far_apart(DO), far_apart(Q), K, V, out, lse, None, None, None, co, cn, ind, CU, CU, None,
+                                 max(lens), max(lens), 0.0, scale, False, True, 0.0, False, 128, chunk, None, None, _dq_mode=dq_mode)[:3]
+    for name, x, y in zip(("dq", "dk", "dv"), ref, got):
+        assert torch.equal(x, y), name
+
+
 @pytest.mark.parametrize("chunk,topk,visits", [(64, 40, 40), (128, 24, 24), (256, 10, 20)])
 def test_partial_forms_are_bitwise_repeatable_beyond_16_visits_per_row(fm, chunk, topk, visits):
     # Column forward and partial-sum dQ hand out a row's partial slots from a counter, in whatever order the
