@@ -252,12 +252,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         }
       }
     };
+    const int64_t trash = (int64_t)a.total_q * a.heads * ws.cap;  // spare row: takes the writes of absent rows, no branch
     auto meta_store = [&](int sr) {
       if (tid < kBwdRoundRows) {
         const int i = (sr & 1) * kBwdRoundRows + ft;
         const bool ok = m_rid >= 0;
         sRow[i] = m_rid;
-        sSlot[i] = m_slot;
+        // where the visit's dQ partial goes, as an index of partial rows (2^31 of them would be half a terabyte): the
+        // row's slot, or the spare row for an absent row and for a visit beyond the caller's bound
+        if constexpr (DQP) sSlot[i] = (ok && m_slot < ws.cap) ? (int)((((int64_t)(q0 + m_rid)) * a.heads + h) * ws.cap + m_slot) : (int)trash;
         sLse[i] = ok ? m_lse * kLog2e : INFINITY;  // absent rows: exp2(x - inf) = 0
         sDelta[i] = ok ? m_del : 0.f;
       }
@@ -548,7 +551,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           mfma_results_ready(dqa[0], dqa[1]);
       }
     };
-    const int64_t trash = (int64_t)a.total_q * a.heads * ws.cap;  // spare row: takes the writes of absent rows, no branch
     auto dq_store = [&](auto pc, auto pp, auto tsc) {
       constexpr int TS = decltype(pc)::value * 4 + decltype(pp)::value * 2 + decltype(tsc)::value;
       constexpr uint32_t SO = (uint32_t)(decltype(pc)::value * 4 + decltype(pp)::value * 2) * TB;  // the tile that serves as staging
@@ -570,12 +572,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       opaque(bs, bx);
 #pragma unroll
       for (int k = 0; k < 32 / RPP; ++k) {
-        const int r2 = lds_read_vec<int>(bs + (uint32_t)(TS * 32 + k * RPP) * 4);
-        const int s2 = lds_read_vec<int>(bs + (uint32_t)(TS * 32 + k * RPP) * 4 + (uint32_t)(SM::oSlot - SM::oRow));
+        const uint32_t pidx = (uint32_t)lds_read_vec<int>(bs + (uint32_t)(TS * 32 + k * RPP) * 4 + (uint32_t)(SM::oSlot - SM::oRow));
         const Pack8 x = lds_read16(bx + SO + (uint32_t)(k * RPP * LDH * 2));
-        const bool ok = (r2 >= 0) & (s2 < ws.cap);
-        const int64_t pidx = ok ? ((int64_t)(q0 + r2) * a.heads + h) * ws.cap + s2 : trash;
-        if (kq * (NDH * 32) + col < D) st_stream16(ws.part + pidx * D + kq * (NDH * 32) + col, x);
+        if (kq * (NDH * 32) + col < D) st_stream16(ws.part + ((uint64_t)pidx * (uint32_t)D + (uint32_t)(kq * (NDH * 32) + col)), x);
         if (kq == 0 && col == 0) ws.pid[pidx] = nb;
       }
       wave_lds_fence();
@@ -1413,6 +1412,9 @@ extern "C" int fmoba_attn_bwd_phases(const fmoba_attn_bwd_args *a, int32_t phase
   uintptr_t wp = ((uintptr_t)a->workspace + 255) & ~(uintptr_t)255;
   BwdWs ws;
   ws.cap = bwd_partial_cap(*a);
+  // (the dK/dV pass keeps the place of a visit's dQ partial as a 32-bit index of partial rows)
+  FMOBA_REQUIRE(!fmoba::bwd_dq_partials(*a) || rows * (size_t)ws.cap + 1 < ((size_t)1 << 31),
+                "attn_bwd: %zu rows x heads with up to %d dQ partials each are more partial rows than the partials form addresses", rows, ws.cap);
   ws.ds = reinterpret_cast<uint16_t *>(wp);
   ws.cnt = reinterpret_cast<int32_t *>(wp);
   wp += bwd_align256(rows * 4);
