@@ -570,12 +570,21 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       uint32_t bs = (uint32_t)(uintptr_t)(smem + SM::oRow) + (uint32_t)((px * 64 + lane / LPR) * 4);
       uint32_t bx = (uint32_t)(uintptr_t)sdQ0 + (uint32_t)(((lane / LPR) * LDH + col) * 2);
       opaque(bs, bx);
+      // (one test around all rows of the tile rather than one per store: a lane either has features of the head
+      // dimension in its piece or it has not)
+      uint32_t pidx[32 / RPP];
 #pragma unroll
-      for (int k = 0; k < 32 / RPP; ++k) {
-        const uint32_t pidx = (uint32_t)lds_read_vec<int>(bs + (uint32_t)(TS * 32 + k * RPP) * 4 + (uint32_t)(SM::oSlot - SM::oRow));
-        const Pack8 x = lds_read16(bx + SO + (uint32_t)(k * RPP * LDH * 2));
-        if (kq * (NDH * 32) + col < D) st_stream16(ws.part + ((uint64_t)pidx * (uint32_t)D + (uint32_t)(kq * (NDH * 32) + col)), x);
-        if (kq == 0 && col == 0) ws.pid[pidx] = nb;
+      for (int k = 0; k < 32 / RPP; ++k) pidx[k] = (uint32_t)lds_read_vec<int>(bs + (uint32_t)(TS * 32 + k * RPP) * 4 + (uint32_t)(SM::oSlot - SM::oRow));
+      if (kq * (NDH * 32) + col < D) {
+#pragma unroll
+        for (int k = 0; k < 32 / RPP; ++k) {
+          const Pack8 x = lds_read16(bx + SO + (uint32_t)(k * RPP * LDH * 2));
+          st_stream16(ws.part + ((uint64_t)pidx[k] * (uint32_t)D + (uint32_t)(kq * (NDH * 32) + col)), x);
+        }
+      }
+      if (kq == 0 && col == 0) {
+#pragma unroll
+        for (int k = 0; k < 32 / RPP; ++k) ws.pid[pidx[k]] = nb;
       }
       wave_lds_fence();
     };
