@@ -257,16 +257,30 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qb[ks] = lds_read16((bq ^ (uint32_t)(ks * 16)) + (uint32_t)(PB * 4) * TB);
     __builtin_amdgcn_sched_barrier(0);
+    // block-local softmax of the row, log2 domain; keys beyond lim are masked: in a tile that has such pairs S^T starts
+    // from 0 / -inf per pair and the products add to that (the exponential of -inf is 0), in the others it starts from
+    // nothing, and the softmax has no comparison in either
+    const int lim = rid < 0 ? -1 : min(causal ? rid + off : 0x7fffffff, Lk - 1) - key0;  // last visible key, relative
     f32x16 st[KT];  // S^T: register i of tile kt <-> key kt*32 + acc_row(i, hh), this lane's row
+    const bool masked = !__all(lim >= KB - 1);
+    if (masked) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
+      for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt) {
-        if (ks == 0)
-          mfma32_a_acc<T, true>(st[kt], kfr[kt][ks], qb[ks]);
-        else
-          mfma32_a_acc<T, false>(st[kt], kfr[kt][ks], qb[ks]);
-      }
+        for (int i = 0; i < 16; ++i) {
+          const int jrel = kt * 32 + 8 * (i >> 2) + (i & 3) + 4 * hh;
+          st[kt][i] = jrel <= lim ? 0.f : -INFINITY;
+        }
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) mfma32_a_acc<T, false>(st[kt], kfr[kt][0], qb[0]);
+    } else {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) mfma32_a_acc<T, true>(st[kt], kfr[kt][0], qb[0]);
+    }
+#pragma unroll
+    for (int ks = 1; ks < KS; ++ks)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) mfma32_a_acc<T, false>(st[kt], kfr[kt][ks], qb[ks]);
     static_assert(KT == 2 || KT == 4, "key blocks of 64 or 128 keys");
     if constexpr (KT == 2) {
       mfma_results_ready(st[0], st[1]);
@@ -287,25 +301,12 @@ __global__ __launch_bounds__(256) void attn_fwd_col_kernel(fmoba_attn_fwd_args a
           vt[dt][kt][s2] = tr_frag8_at(trV, lo, lo + 8 * LDQ);
         }
     __builtin_amdgcn_sched_barrier(0);
-    // block-local softmax of the row, log2 domain; keys beyond lim are masked
-    const int lim = rid < 0 ? -1 : min(causal ? rid + off : 0x7fffffff, Lk - 1) - key0;  // last visible key, relative
     // (the scores stay raw: the scale, positive, goes into the exponent's multiply-add)
     float m = -INFINITY;
-    if (__all(lim >= KB - 1)) {
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt)
+    for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) m = fmaxf(m, st[kt][i]);
-    } else {
-#pragma unroll
-      for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int jrel = kt * 32 + 8 * (i >> 2) + (i & 3) + 4 * hh;
-          st[kt][i] = jrel <= lim ? st[kt][i] : -INFINITY;
-          m = fmaxf(m, st[kt][i]);
-        }
-    }
+      for (int i = 0; i < 16; ++i) m = fmaxf(m, st[kt][i]);
     m = max_xor32_f(m) * scale_log2;
     const float m_use = m == -INFINITY ? 0.f : m;
     float l = 0.f;
