@@ -105,17 +105,17 @@ def time_events(fn, iters, warmup=1):
 # Counter runs cannot be made from inside this script, so the figures are the committed measurement.
 MEASURED_TRAFFIC_BYTES = {
     ("headline", "attn_fwd_rows_kernel"): 1.296e9,
-    ("headline", "attn_bwd_dkdv_kernel"): 6.689e9,
-    ("headline", "attn_bwd_dq_kernel"): 5.114e9,
-    ("c2", "attn_fwd_col_kernel"): 4.422e8,
-    ("c3", "attn_fwd_col_kernel"): 8.220e9,
-    ("c3", "attn_bwd_dkdv_kernel"): 1.279e10,
-    ("c5", "attn_fwd_col_kernel"): 3.995e10,
-    ("c5", "attn_bwd_dkdv_kernel"): 6.636e10,
-    ("sweep16k", "attn_fwd_col_kernel"): 1.941e9,
-    ("sweep16k", "attn_bwd_dkdv_kernel"): 2.946e9,
-    ("sweep64k", "attn_fwd_col_kernel"): 9.670e9,
-    ("sweep64k", "attn_bwd_dkdv_kernel"): 1.551e10,
+    ("headline", "attn_bwd_dkdv_kernel"): 6.680e9,
+    ("headline", "attn_bwd_dq_kernel"): 5.128e9,
+    ("c2", "attn_fwd_col_kernel"): 4.421e8,
+    ("c3", "attn_fwd_col_kernel"): 8.212e9,
+    ("c3", "attn_bwd_dkdv_kernel"): 1.273e10,
+    ("c5", "attn_fwd_col_kernel"): 3.996e10,
+    ("c5", "attn_bwd_dkdv_kernel"): 6.673e10,
+    ("sweep16k", "attn_fwd_col_kernel"): 1.943e9,
+    ("sweep16k", "attn_bwd_dkdv_kernel"): 2.924e9,
+    ("sweep64k", "attn_fwd_col_kernel"): 9.663e9,
+    ("sweep64k", "attn_bwd_dkdv_kernel"): 1.546e10,
 }
 
 
