@@ -80,7 +80,9 @@ __device__ __forceinline__ uint32_t mul24_u32(uint32_t a, uint32_t b) {
 // key half kq.  KB = 2 (columns of a multiple of 128 keys, whose two 64-key blocks share one row list): it owns 128
 // keys, every wave takes all four tiles for its key quarter kq, so a gathered row serves twice the keys and a visit
 // leaves one dQ partial instead of two.
-template <typename T, int HD, bool DQP, int KB>
+// NEAR: the host has checked that a gathered row's place in q and dout is a 32-bit byte offset from the sequence's first
+// row that one 24-bit multiply makes (launch_dkdv); otherwise the loads take 64-bit addresses per lane.
+template <typename T, int HD, bool DQP, int KB, bool NEAR>
 __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args a, BwdWs ws) {
   typedef BwdSmem<HD> SM;
   constexpr int KS = HD / 16, LDQ = SM::LDQ, LDS_ = SM::LDS_, NDT = HD / 32, VPR = HD / 8, LDR = SM::LDR;
@@ -100,8 +102,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 
   const PairItem item = xcd_pair_item(blockIdx.x, a.batch * a.heads, (a.max_seqlen_k + NKEY - 1) / NKEY, (int64_t)a.max_seqlen_q * HD * 4 >= kOnePairBytes);
   const int nb = item.idx, b = item.pair / a.heads, h = item.pair - b * a.heads;
-  const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
   const int key0 = nb * NKEY;
+  // One workgroup per compute unit: nothing covers the dependent loads before the first round, so their chain is kept
+  // short.  Where the block's column list lies depends on nothing that is loaded: asked for together with the
+  // sequence bounds.
+  const int Bn = a.lg_block_n;
+  const int c = key0 / Bn;
+  const int64_t bh = (int64_t)b * a.heads + h;
+  int nnz = 0;
+  int64_t lbase = 0;
+  if (c < a.max_cols) {
+    nnz = a.col_nnz[bh * a.max_cols + c];
+    lbase = a.col_offsets[bh * a.max_cols + c];
+  }
+  const int k0 = a.cu_seqlens_k[b], Lk = a.cu_seqlens_k[b + 1] - k0;
   if (key0 >= Lk) return;
   const int q0 = a.cu_seqlens_q[b], Lq = a.cu_seqlens_q[b + 1] - q0;
   const int off = Lk - Lq;
@@ -136,18 +150,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   }
 
   // ---- this block's column list --------------------------------------------------------------
-  const int Bn = a.lg_block_n;
-  const int c = key0 / Bn;
-  const int64_t bh = (int64_t)b * a.heads + h;
-  int nnz = 0;
-  int64_t lbase = 0;
-  int start = 0;
-  if (c < a.max_cols) {
-    nnz = a.col_nnz[bh * a.max_cols + c];
-    lbase = a.col_offsets[bh * a.max_cols + c];
-    // rows r with r + off < key0 see no key of this block
-    if (causal && nnz > 0) start = lower_bound_wave_i32(a.row_indices + lbase, nnz, key0 - off);
+  // The rows of the first two rounds are asked for together with the probes of the search below, as if the walk
+  // began at the head of the list (it does unless rows of the list lie before the block); otherwise they are
+  // fetched again.
+  int spec01[2] = {0, 0};
+  if (tid < kBwdRoundRows && nnz > 0) {
+#pragma unroll
+    for (int sr = 0; sr < 2; ++sr) spec01[sr] = a.row_indices[lbase + min(sr * kBwdRoundRows + tid, nnz - 1)];
   }
+  int start = 0;
+  // rows r with r + off < key0 see no key of this block
+  if (causal && nnz > 0) start = lower_bound_wave_i32(a.row_indices + lbase, nnz, key0 - off);
   const int32_t *list = a.row_indices + lbase + start;
   const int n = nnz - start;               // rows of the list that the block walks
   const int nround = (n + kBwdRoundRows - 1) / kBwdRoundRows;
@@ -157,7 +170,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 #pragma unroll
     for (int sr = 0; sr < 2; ++sr) {
       const int j = sr * kBwdRoundRows + tid;
-      const int r = list[min(j, n - 1)];
+      const int r = start == 0 ? spec01[sr] : list[min(j, n - 1)];
       rid01[sr] = tile_row_code(r, j < n, Lq);
     }
   }
@@ -265,8 +278,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
         sDelta[i] = ok ? m_del : 0.f;
       }
     };
-    const bool near_rows = Lq < (1 << 24) && a.q_row_stride < (1 << 22) && a.do_row_stride < (1 << 22) &&
-                           (int64_t)Lq * a.q_row_stride < (int64_t)0x7fff0000 && (int64_t)Lq * a.do_row_stride < (int64_t)0x7fff0000;
     auto tile_issue = [&](int sr) {  // tile `wave` of round sr
       constexpr int RPI = 64 / VPR, NI = 32 / RPI;  // tile rows per instruction, instructions per tile
       const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
@@ -278,7 +289,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
       int src[NI];
 #pragma unroll
       for (int i = 0; i < NI; ++i) src[i] = sRid[(sr & 1) * kBwdRoundRows + wave * 32 + i * RPI + rl] & 0x7fffffff;
-      if (near_rows) {
+      if constexpr (NEAR) {
         // the sequence's rows lie within 4 GB of its first one: a 32-bit byte offset per lane from a wave-uniform base,
         // one full-rate multiply (the 64-bit products take four times as long, and an address takes two more additions)
 #pragma unroll
@@ -295,6 +306,38 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           global_to_lds16(dog + ((uint64_t)(uint32_t)src[i] * dos + e), ldsdO + dst + (uint32_t)(i * RPI * RB));
         }
       }
+    };
+
+    // The same loads one at a time, for rows near the base.  A load instruction of a kilobyte holds the wave for about
+    // 70 clocks while the unit's four waves issue theirs together (the unit's vector memory path takes 64 bytes per
+    // clock: a round's 64 KB are a thousand clocks of it), and a wave that waits there issues no products either.  So
+    // the Q loads go between the products of the round's first stage, one per two products, and the dO loads between
+    // those of the second, instead of all at the start of the round; the offsets stay in registers until then.  (With
+    // a test per load of whether the rows are near, that gain was lost: hence the NEAR instantiations.)
+    constexpr bool kSpreadLoads = NEAR;
+    constexpr int NTI = 32 / (64 / VPR);  // load instructions per tile and operand
+    static_assert(NTI == KS, "one pair of tile loads per k-step of the first stage");
+    uint32_t t_q[kSpreadLoads ? NTI : 1], t_do[kSpreadLoads ? NTI : 1], t_dst = 0;  // byte offsets of this lane's pieces
+    auto tile_rows = [&](int sr) {
+      constexpr int RPI = 64 / VPR;
+      const int fl = ft & 63, rl = fl / VPR, p = fl - rl * VPR;
+      t_dst = (uint32_t)__builtin_amdgcn_readfirstlane(((sr & 1) * 4 + wave) * (int)TB);
+      const uint32_t qs = (uint32_t)a.q_row_stride, dos = (uint32_t)a.do_row_stride;
+#pragma unroll
+      for (int i = 0; i < (kSpreadLoads ? NTI : 0); ++i) {
+        const uint32_t src = (uint32_t)(sRid[(sr & 1) * kBwdRoundRows + wave * 32 + i * RPI + rl] & 0x7fffffff);
+        const uint32_t e2 = (uint32_t)min((p ^ tile_swz<HD>(i * RPI + rl)) * 8, D - 8) * 2u;
+        t_q[i] = mul24_u32(src, qs * 2u) + e2;
+        t_do[i] = mul24_u32(src, dos * 2u) + e2;
+      }
+    };
+    auto tile_issue_q = [&](auto ic) {
+      constexpr int I = decltype(ic)::value, RPI = 64 / VPR;
+      if constexpr (kSpreadLoads) global_to_lds16_sbase(t_q[I], qg, ldsQ + t_dst + (uint32_t)(I * RPI * RB));
+    };
+    auto tile_issue_do = [&](auto ic) {
+      constexpr int I = decltype(ic)::value, RPI = 64 / VPR;
+      if constexpr (kSpreadLoads) global_to_lds16_sbase(t_do[I], dog, ldsdO + t_dst + (uint32_t)(I * RPI * RB));
     };
 
     if (tid < kBwdRoundRows) {
@@ -407,10 +450,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
     // -inf elsewhere (the products then leave -inf there and the exponential gives 0), and only in rounds that have
     // such pairs at all (`masked`, the same for the whole wave): the rows of a list come in ascending order, so
     // from the first row that sees every key of the block on, S starts from nothing and no comparison is made.
-    auto mm_a = [&](auto pc, auto pp, auto tsc, auto gc, bool masked) {
+    auto mm_a = [&](auto pc, auto pp, auto tsc, auto gc, bool masked, auto &&after_step) {
       constexpr int TS = decltype(tsc)::value, G = decltype(gc)::value;
-#pragma unroll
-      for (int t = 0; t < KC; ++t) {
+      static_for<KC>([&](auto tc) {
+        constexpr int t = decltype(tc)::value;
         if (G == 0 && t == 0) {
           if (masked) {
             constexpr int TSG = decltype(pc)::value * 4 + decltype(pp)::value * 2 + TS;
@@ -432,7 +475,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           mfma32_b_acc<T, false>(s[TS], qa[G & 1][t], kb[G * KC + t]);
           mfma32_b_acc<T, false>(dp[TS], doa[G & 1][t], vb[G * KC + t]);
         }
-      }
+        after_step(std::integral_constant<int, G * KC + t>{});
+      });
       if constexpr (G == 3) mfma_results_ready(s[TS], dp[TS]);
     };
     auto ld_b = [&](auto pc, auto pp, auto tsc, auto gc) {
@@ -605,7 +649,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           ld_a(pc, pp, C1{}, C0{});
           ld_s(pc, pp, C0{}, C0{});
         }
-        mm_a(pc, pp, C0{}, gc, masked);
+        mm_a(pc, pp, C0{}, gc, masked, [&](auto ic) {
+          if constexpr (kSpreadLoads && decltype(pp)::value == 0) tile_issue_q(ic);
+        });
         fence();
       });
       // S, dP of the second tile between the softmax rows of the first
@@ -618,7 +664,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
           ld_b(pc, pp, C0{}, C0{});
           ld_s(pc, pp, C1{}, C0{});
         }
-        mm_a(pc, pp, C1{}, gc, masked);
+        mm_a(pc, pp, C1{}, gc, masked, [&](auto ic) {
+          if constexpr (kSpreadLoads && decltype(pp)::value == 0) tile_issue_do(ic);
+        });
         smx(C0{}, gc);
         fence();
       });
@@ -684,7 +732,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
 #endif
       rid_issue(r + 2);
       meta_issue(v_rid);
-      tile_issue(r + 1);
+      if constexpr (kSpreadLoads)
+        tile_rows(r + 1);
+      else
+        tile_issue(r + 1);
       process_round(pc, C0{}, r);
       if constexpr (KB == 2) process_round(pc, C1{}, r);
       if constexpr (!DQP) {
@@ -1234,9 +1285,9 @@ __global__ void zero_f32_kernel(float *p, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.f;
 }
 
-template <typename T, int HD, bool DQP, int KB>
-static int launch_dkdv(const fmoba_attn_bwd_args &a, const BwdWs &ws, hipStream_t s) {
-  auto kern = attn_bwd_dkdv_kernel<T, HD, DQP, KB>;
+template <typename T, int HD, bool DQP, int KB, bool NEAR>
+static int launch_dkdv_form(const fmoba_attn_bwd_args &a, const BwdWs &ws, hipStream_t s) {
+  auto kern = attn_bwd_dkdv_kernel<T, HD, DQP, KB, NEAR>;
   const size_t smem = BwdSmem<HD>::bytes;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     set_error("attn_bwd: cannot reserve %zu bytes of LDS", smem);
@@ -1249,6 +1300,14 @@ static int launch_dkdv(const fmoba_attn_bwd_args &a, const BwdWs &ws, hipStream_
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)items), dim3(256), smem, s, a, ws);
   return 0;
+}
+// NEAR: every row of a sequence's q and dout lies within 2 GB of the sequence's first row and is less than 2^24 rows
+// and 2^22 elements per row away, so a gathered row's place is a 32-bit offset made by one 24-bit multiply.
+template <typename T, int HD, bool DQP, int KB>
+static int launch_dkdv(const fmoba_attn_bwd_args &a, const BwdWs &ws, hipStream_t s) {
+  const bool near_rows = a.max_seqlen_q < (1 << 24) && a.q_row_stride < (1 << 22) && a.do_row_stride < (1 << 22) &&
+                         (int64_t)a.max_seqlen_q * a.q_row_stride < (int64_t)0x7fff0000 && (int64_t)a.max_seqlen_q * a.do_row_stride < (int64_t)0x7fff0000;
+  return near_rows ? launch_dkdv_form<T, HD, DQP, KB, true>(a, ws, s) : launch_dkdv_form<T, HD, DQP, KB, false>(a, ws, s);
 }
 
 template <typename T, int HD, int RT>
