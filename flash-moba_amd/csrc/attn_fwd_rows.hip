@@ -639,6 +639,8 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
   Pack8 kf[KS];        // K operands of S(t + 1): read at the start of part0, their latency runs under its arithmetic
   Pack8 vt[2][2];      // V^T operands of the first feature tile of step t: read at the end of part1
   float neg_mc = 0.f;  // minus the reference point of the row's exponentials, scaled; -inf for a row that skips the step
+  int s_nx = sStep[0];  // entry of the next step and this row's word of selection bits for its chunk
+  uint32_t word_nx = sBits[((s_nx >> 16) >> 5) * kRows8 + wave * 32 + (lane & 31)];
   auto part0 = [&](auto par, int t) {
     constexpr int P = decltype(par)::value;
     f32x16(&sc)[2] = st[P];
@@ -648,9 +650,11 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) kf[ks] = k_frag(akn, 0, ks);
     }
-    const int s = sStep[t];
+    // (the step's entry and this row's selection word were read during the step before: two dependent LDS reads at
+    // this place would be waited for with nothing to do, by every wave at the start of every step)
+    const int s = s_nx;
     const int key0 = (s & 0xffff) << 6, c = s >> 16;
-    const uint32_t myword = sBits[(c >> 5) * kRows8 + wave * 32 + (lane & 31)];
+    const uint32_t myword = word_nx;
     const bool active = valid && ((myword >> (c & 31)) & 1u) != 0u && lim >= key0;
     const int lim_rel = active ? lim - key0 : -1;
     if (!__all(lim_rel >= 63 || lim_rel < 0)) {
@@ -712,6 +716,8 @@ __global__ __launch_bounds__(512) void attn_fwd_rows_kernel(fmoba_attn_fwd_args 
       const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[kte][2 * j + 1], scale_log2, neg_mc));
       lsum += p0 + p1;
       pf[kte][j / 4].w[j % 4] = pack2<T>(p0, p1);
+      if (g == 2) s_nx = sStep[min(t + 1, nstep - 1)];
+      if (g == 8) word_nx = sBits[((s_nx >> 16) >> 5) * kRows8 + wave * 32 + (lane & 31)];
       if (g == 14) {  // V^T operands of the first feature tile
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
