@@ -104,18 +104,18 @@ def time_events(fn, iters, warmup=1):
 # same counter reads for a plain 1 GiB copy (the summaries of those runs are kept under profiles/, one per workload).
 # Counter runs cannot be made from inside this script, so the figures are the committed measurement.
 MEASURED_TRAFFIC_BYTES = {
-    ("headline", "attn_fwd_rows_kernel"): 1.296e9,
-    ("headline", "attn_bwd_dkdv_kernel"): 6.680e9,
-    ("headline", "attn_bwd_dq_kernel"): 5.128e9,
+    ("headline", "attn_fwd_rows_kernel"): 1.278e9,
+    ("headline", "attn_bwd_dkdv_kernel"): 6.702e9,
+    ("headline", "attn_bwd_dq_kernel"): 5.139e9,
     ("c2", "attn_fwd_col_kernel"): 4.421e8,
-    ("c3", "attn_fwd_col_kernel"): 8.212e9,
-    ("c3", "attn_bwd_dkdv_kernel"): 1.273e10,
-    ("c5", "attn_fwd_col_kernel"): 3.996e10,
-    ("c5", "attn_bwd_dkdv_kernel"): 6.673e10,
-    ("sweep16k", "attn_fwd_col_kernel"): 1.943e9,
-    ("sweep16k", "attn_bwd_dkdv_kernel"): 2.924e9,
-    ("sweep64k", "attn_fwd_col_kernel"): 9.663e9,
-    ("sweep64k", "attn_bwd_dkdv_kernel"): 1.546e10,
+    ("c3", "attn_fwd_col_kernel"): 8.222e9,
+    ("c3", "attn_bwd_dkdv_kernel"): 1.299e10,
+    ("c5", "attn_fwd_col_kernel"): 3.995e10,
+    ("c5", "attn_bwd_dkdv_kernel"): 6.687e10,
+    ("sweep16k", "attn_fwd_col_kernel"): 1.941e9,
+    ("sweep16k", "attn_bwd_dkdv_kernel"): 2.939e9,
+    ("sweep64k", "attn_fwd_col_kernel"): 9.660e9,
+    ("sweep64k", "attn_bwd_dkdv_kernel"): 1.551e10,
 }
 
 
