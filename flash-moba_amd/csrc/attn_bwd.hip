@@ -234,7 +234,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(fmoba_attn_bwd_args 
   if (nround > 0) {
     // ---- feeding the tiles --------------------------------------------------------------------------
     // Nothing passes through registers: every wave fetches one of the four tiles of the NEXT round with loads that
-    // write straight to LDS, issued at the start of a round and awaited at its end.  Threads 0..127 carry the
+    // write straight to LDS, issued in the first half of a round and awaited at its end.  Threads 0..127 carry the
     // per-row scalars: the row id of round s+2 (it has to be in LDS one round before the tile loads that use it),
     // and LSE, delta and the dQ-partial slot of round s+1.
     const uint32_t ldsQ = (uint32_t)(uintptr_t)(smem + SM::oQ), ldsdO = (uint32_t)(uintptr_t)(smem + SM::odO);
