@@ -969,9 +969,13 @@ __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq
     for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[rt][dt][i] = 0.f;
+  // Which rows a wave owns: the waves w and w + 4 share a SIMD, and under the causal rule the later rows of the block
+  // take part in more steps (the first wave's rows sit out the block's last seven key blocks, the last wave's none), so
+  // a SIMD gets the rows w and 7 - w: the four SIMDs then have the same number of products to do.
+  const int wtile = wave < 4 ? wave : 11 - wave;
   int myrow[RT];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) myrow[rt] = (wave * RT + rt) * 32 + (lane & 31);
+  for (int rt = 0; rt < RT; ++rt) myrow[rt] = (wtile * RT + rt) * 32 + (lane & 31);
 
   // K tile loads of this wave: instruction i brings tile rows (wave * NKI + i) * RPI .. + RPI - 1, lane -> row rl, piece p;
   // piece c of tile row r is stored at piece c ^ tile_swz<HD>(r)
@@ -1159,7 +1163,7 @@ __global__ __launch_bounds__(512, (HD > 128 || RT > 1) ? 2 : 4) void attn_bwd_dq
 #pragma unroll
     for (int v0 = 0; v0 < 32 * VPR; v0 += 64) {
       const int v = v0 + lane, rl = v / VPR, e = (v - rl * VPR) * 8;
-      const int r2 = (wave * RT + rt) * 32 + rl;
+      const int r2 = (wtile * RT + rt) * 32 + rl;
       if (r2 < rows_sb && e < D)
         *reinterpret_cast<Pack8 *>(op + (int64_t)r2 * a.dq_row_stride + e) = *reinterpret_cast<const Pack8 *>(sOut + rl * LDO + e);
     }
