@@ -697,13 +697,15 @@ def test_backward_both_dq_forms(fm, dq_mode, d, chunk):
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
 
 
+@pytest.mark.parametrize("d,chunk", [(128, 64), (64, 64), (128, 128)])
 @pytest.mark.parametrize("dq_mode", [1, 2])
-def test_backward_with_rows_far_apart(fm, dq_mode):
+def test_backward_with_rows_far_apart(fm, dq_mode, d, chunk):
     # The dK/dV pass fetches the rows of a list with a 32-bit byte offset per lane where a sequence's rows lie within
-    # 4 GB of its first one, and with 64-bit addresses otherwise: q and dout as views with a row stride of 2^22
-    # elements (8 MB) take the second way and must give the bits of the packed tensors.
-    lens = [200, 90]
-    d, chunk, heads = 128, 64, 2
+    # 4 GB of its first one, and with 64-bit addresses otherwise (a kernel form of its own, chosen by the host, for
+    # each head dimension and key-block width): q and dout as views with a row stride of 2^22 elements (8 MB) take the
+    # second way and must give the bits of the packed tensors.
+    lens = [200, 90] if chunk == 64 else [300, 140]
+    heads = 2
     q, k, v, cu, dout = O.make_inputs(lens, heads, d, chunk, 35, torch.bfloat16, with_dout=True)
     Q, K, V, CU, DO = q.cuda(), k.cuda(), v.cuda(), cu.cuda(), dout.cuda()
     co, cn, ind = fm.api.flash_topk_varlen_func(Q, K, CU, CU, max(lens), max(lens), 2, chunk, causal=True)
